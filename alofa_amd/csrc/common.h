@@ -1,0 +1,83 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions,
+// wave and block reductions, and the error channel of the C entry points.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+namespace alofa {
+
+typedef uint16_t bf16_t;  // bfloat16 carried as its 16 bits
+
+constexpr int kWave = 64;  // CDNA wavefront
+
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+// ---- conversions -----------------------------------------------------------
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(static_cast<uint32_t>(v) << 16);
+}
+
+// round to nearest, ties to even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<bf16_t>(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float load_f32(const T* p);
+template <> __device__ __forceinline__ float load_f32<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_f32<bf16_t>(const bf16_t* p) { return bf16_to_f32(*p); }
+
+template <typename T> __device__ __forceinline__ void store_f32(T* p, float v);
+template <> __device__ __forceinline__ void store_f32<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// ---- reductions ------------------------------------------------------------
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+  return v;
+}
+
+// Sum over a block of kThreads (a multiple of 64) in a fixed tree, so the
+// result depends only on the inputs' places, never on timing. Every thread
+// gets the total. `scratch` holds kThreads / 64 values.
+template <typename T, int kThreads>
+__device__ __forceinline__ T block_sum(T v, T* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  T total = scratch[0];
+#pragma unroll
+  for (int w = 1; w < kThreads / kWave; ++w) total += scratch[w];
+  return total;
+}
+
+// ---- error channel ---------------------------------------------------------
+
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+}  // namespace alofa
+
+#define ALOFA_REQUIRE(cond, ...)          \
+  do {                                    \
+    if (!(cond)) {                        \
+      alofa::set_error(__VA_ARGS__);      \
+      return 1;                           \
+    }                                     \
+  } while (0)

@@ -1,0 +1,204 @@
+"""The step function: one batch of (request, its next tokens) — portions of
+prompts beside single decoded tokens, cut anywhere — run as one packed matrix
+from the cache that earlier steps left; logits come back at the wanted places
+only. Rows of one request are contiguous and in position order; requests lie in
+the order given (src/alofa/engine/executor.mojo:555-609 for the row layout,
+:665-859 for the pass)."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..errors import AlofaError
+
+
+@dataclass
+class StepEntry:
+    """Next tokens of one request. ``want``: places among these tokens whose
+    logits are asked for (may be empty)."""
+    request: object
+    tokens: list
+    want: list = field(default_factory=list)
+
+
+@dataclass(frozen=True)
+class Span:
+    """Where one request's rows lie in the step."""
+    request: object
+    slot: int        # its request slot (index into per-request state)
+    row0: int        # first row in the packed matrix
+    n: int           # rows
+    pos0: int        # absolute position of the first row
+
+
+@dataclass
+class KVView:
+    """What a mixer sees of its cache in one step."""
+    k: torch.Tensor
+    v: torch.Tensor
+    block_table: torch.Tensor      # int32 [requests, max_blocks], -1 where no page
+    slots: Optional[torch.Tensor]  # int64 [T] cache slot per row
+    owner: bool                    # False: reads another entry's cache, writes nothing
+    group: int
+
+
+class StepContext:
+    """Everything the parts need to know about one step."""
+
+    def __init__(self, fn: "StepFunction", spans: list, positions_host: np.ndarray):
+        self.fn = fn
+        self.spans = spans
+        self.positions_host = positions_host
+        self.tokens = int(positions_host.shape[0])
+        self.n_positions = fn.n_positions
+        self.positions: torch.Tensor = None
+        self.req_of_token: torch.Tensor = None
+        self._tables: list = []
+        self._slots: list = []
+
+    def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
+        return self.fn.scratch(name, shape, dtype)
+
+    def kv(self, entry: int) -> KVView:
+        owner_entry = self.fn.cache_entry[entry]
+        if owner_entry is None:
+            raise AlofaError("invalid_argument", "this entry keeps no cache", f"entry={entry}")
+        g = self.fn.cache.group_of_entry[owner_entry]
+        owns = owner_entry == entry
+        return KVView(self.fn.cache.k[owner_entry], self.fn.cache.v[owner_entry], self._tables[g],
+                      self._slots[g] if owns else None, owns, g)
+
+    def state(self, entry: int) -> torch.Tensor:
+        """Per-request state of an entry: [max_requests, *shape]; row = Span.slot."""
+        return self.fn.cache.state[entry]
+
+    def identity_rotation(self, head_dim: int):
+        return self.fn.identity_rotation(head_dim)
+
+
+class StepFunction:
+    def __init__(self, model, cache: CacheManager, n_positions: int):
+        self.model = model
+        self.cache = cache
+        self.n_positions = int(n_positions)
+        self.device = model.rt.device
+        self._scratch: dict = {}
+        self._identity: dict = {}
+        self.cache_entry = [i if e.cache_of is None else e.cache_of for i, e in enumerate(model.order)]
+        needs = model.cache_needs()
+        self.cache_entry = [c if needs[c] is not None else None for c in self.cache_entry]
+        self.steps_run = 0
+        self.rows_run = 0
+        # build position tables up to the context bound once, so they never move afterwards
+        for b in model.blocks:
+            pos = getattr(b.mixer, "position", None)
+            if pos is not None:
+                pos.table(self.n_positions)
+
+    # ------------------------------------------------------------- scratch
+    def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
+        """A named buffer re-used from step to step and layer to layer; it grows
+        (outside the steady state) when a step is larger than any before."""
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._scratch.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._scratch[key] = buf
+        return buf[:n].view(shape)
+
+    def identity_rotation(self, head_dim: int):
+        key = head_dim
+        if key not in self._identity:
+            self._identity[key] = (torch.ones(self.n_positions, head_dim // 2, dtype=torch.float32, device=self.device),
+                                   torch.zeros(self.n_positions, head_dim // 2, dtype=torch.float32, device=self.device))
+        return self._identity[key]
+
+    # ----------------------------------------------------------------- run
+    def plan(self, entries: list):
+        """Check a batch and lay out its rows (host only, nothing is changed)."""
+        if not entries:
+            raise AlofaError("invalid_argument", "a step needs at least one entry")
+        vocab = self.model.spec.vocab_size
+        spans, seen, row = [], set(), 0
+        for e in entries:
+            if e.request in seen:
+                raise AlofaError("invalid_argument", "a request appears twice in one step", f"request={e.request}")
+            seen.add(e.request)
+            n = len(e.tokens)
+            if n == 0:
+                raise AlofaError("invalid_argument", "an entry brings no tokens", f"request={e.request}")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise AlofaError("out_of_range", "token id outside the vocabulary", f"request={e.request} token={t} vocab={vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise AlofaError("out_of_range", "wanted place outside the entry's tokens", f"request={e.request} want={w} tokens={n}")
+            pos0 = self.cache.length(e.request)
+            if pos0 + n > self.n_positions:
+                raise AlofaError("capacity", "the request would pass the context bound", f"request={e.request} length={pos0 + n} bound={self.n_positions}")
+            spans.append(Span(e.request, self.cache.slot(e.request), row, n, pos0))
+            row += n
+        return spans
+
+    def run(self, entries: list) -> Optional[torch.Tensor]:
+        """Run the step. Returns float32 logits [wanted, vocab] on the device in
+        the order of the entries and of their ``want`` lists, or None when nothing
+        is wanted."""
+        spans = self.plan(entries)
+        cache = self.cache
+        # pages first: either every entry gets its pages or the step does not run
+        need = [0] * len(cache.groups)
+        for s in spans:
+            for g, n in enumerate(cache.blocks_needed(s.request, s.pos0 + s.n)):
+                need[g] += n
+        for g, grp in enumerate(cache.groups):
+            if need[g] > grp.pool.n_free:
+                raise AlofaError("capacity", "kv block pool is exhausted", f"group={g} need={need[g]} free={grp.pool.n_free}")
+        for s in spans:
+            cache.reserve(s.request, s.pos0 + s.n)
+        T = sum(s.n for s in spans)
+        ids = np.empty(T, dtype=np.int32)
+        positions = np.empty(T, dtype=np.int32)
+        req_of_token = np.empty(T, dtype=np.int32)
+        want_rows = []
+        for i, (e, s) in enumerate(zip(entries, spans)):
+            ids[s.row0:s.row0 + s.n] = np.asarray(e.tokens, dtype=np.int32)
+            positions[s.row0:s.row0 + s.n] = np.arange(s.pos0, s.pos0 + s.n, dtype=np.int32)
+            req_of_token[s.row0:s.row0 + s.n] = i
+            want_rows.extend(s.row0 + int(w) for w in e.want)
+        ctx = StepContext(self, spans, positions)
+        max_blocks = max(1, cache.max_blocks())
+        n_groups = len(cache.groups)
+        tables = np.full((n_groups, len(spans), max_blocks), -1, dtype=np.int32)
+        slots = np.empty((n_groups, T), dtype=np.int64)
+        for g in range(n_groups):
+            for i, s in enumerate(spans):
+                t = cache.table(s.request, g)
+                tables[g, i, :len(t)] = t
+                slots[g, s.row0:s.row0 + s.n] = cache.slots(s.request, g, s.pos0, s.n)
+        dev = self.device
+        ids_d = torch.from_numpy(ids).to(dev)
+        ctx.positions = torch.from_numpy(positions).to(dev)
+        ctx.req_of_token = torch.from_numpy(req_of_token).to(dev)
+        tables_d = torch.from_numpy(tables).to(dev)
+        slots_d = torch.from_numpy(slots).to(dev)
+        ctx._tables = [tables_d[g] for g in range(n_groups)]
+        ctx._slots = [slots_d[g] for g in range(n_groups)]
+
+        hidden = self.model.forward(ctx, ids_d)
+        logits = None
+        if want_rows:
+            rows = torch.tensor(want_rows, dtype=torch.int32, device=dev)
+            logits = self.model.logits(ctx, hidden, rows)
+        for s in spans:
+            cache.commit(s.request, s.pos0 + s.n)
+        self.steps_run += 1
+        self.rows_run += T
+        return logits

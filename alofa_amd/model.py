@@ -1,0 +1,93 @@
+"""A model put together from its ``ModelSpec``: embedding, layers (each a block
+of parts), final norm and head, run in the order the spec lists. The class
+knows no architecture; what differs between models is in the spec."""
+from __future__ import annotations
+
+from pathlib import Path
+
+import torch
+
+from . import models as _models  # noqa: F401  (registers the architectures)
+from .config.base import ModelSpec
+from .config.registry import load_config
+from .errors import AlofaError
+from .parts.base import Runtime, build_part, part_class, tensors_of
+from .weights.loader import load_weights
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "fp32": torch.float32, "bf16": torch.bfloat16}
+
+
+def check_spec(spec: ModelSpec) -> None:
+    """The run order must name existing layers, and an entry may read only the
+    cache of an earlier entry that keeps one of its own."""
+    for i, e in enumerate(spec.order):
+        if not 0 <= e.layer < len(spec.layers):
+            raise AlofaError("out_of_range", "run order names a layer that does not exist", f"entry={i} layer={e.layer}")
+        if e.cache_of is not None:
+            if not 0 <= e.cache_of < i or spec.order[e.cache_of].cache_of is not None:
+                raise AlofaError("invalid_argument", "an entry may read only the cache of an earlier entry that owns one", f"entry={i} cache_of={e.cache_of}")
+
+
+def expected_tensors(spec: ModelSpec) -> dict:
+    """name -> TensorRule for every tensor the model's parts read, in a fixed order."""
+    out = dict(tensors_of("embedding", spec.embedding))
+    for layer in spec.layers:
+        out.update(part_class("block", layer.block.kind).layer_tensors(layer))
+    out.update(tensors_of("norm", spec.final_norm))
+    for name, rule in tensors_of("head", spec.head).items():
+        out.setdefault(name, rule)
+    return out
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, weights: dict, rt: Runtime):
+        check_spec(spec)
+        self.spec = spec
+        self.rt = rt
+        self.embedding = build_part("embedding", spec.embedding, weights, rt)
+        self.blocks = [part_class("block", l.block.kind)(l, weights, rt) for l in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm, weights, rt)
+        self.head = build_part("head", spec.head, weights, rt, embedding=self.embedding)
+        self.order = list(spec.order)
+
+    # what the cache manager has to provide, one item per run entry
+    def cache_needs(self) -> list:
+        return [None if e.cache_of is not None else self.blocks[e.layer].mixer.cache_need() for e in self.order]
+
+    def state_needs(self) -> list:
+        return [self.blocks[e.layer].mixer.state_need() for e in self.order]
+
+    def forward(self, ctx, ids: torch.Tensor) -> torch.Tensor:
+        """Run the tokens of the step through every entry; returns the float32
+        residual stream [T, hidden]."""
+        hidden = self.embedding.forward(ctx, ids)
+        for i, e in enumerate(self.order):
+            self.blocks[e.layer].forward(ctx, i, hidden)
+        return hidden
+
+    def logits(self, ctx, hidden: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        """Final norm and head on the wanted rows only: float32 [len(rows), vocab]."""
+        y = ctx.scratch("final_normed", (rows.shape[0], self.spec.hidden_size), self.rt.dtype)
+        self.final_norm.forward(y, hidden, rows)
+        return self.head.forward(ctx, y)
+
+
+def runtime(dtype="bfloat16", device="cuda:0") -> Runtime:
+    if isinstance(dtype, str):
+        if dtype not in DTYPES:
+            raise AlofaError("invalid_argument", "dtype is float32 or bfloat16", f"dtype={dtype}")
+        dtype = DTYPES[dtype]
+    dev = torch.device(device)
+    if dev.type != "cuda" or not torch.cuda.is_available():
+        raise AlofaError("not_initialized", "the engine runs on a GPU only; none is available", f"device={device}")
+    return Runtime(dev, dtype)
+
+
+def load_model(model_dir, dtype="bfloat16", device="cuda:0"):
+    """(config, model) of a folder with config.json and model.safetensors; the
+    model class is chosen by config.json through the architecture registry."""
+    cfg = load_config(model_dir)
+    spec = cfg.spec()
+    check_spec(spec)
+    weights = load_weights(Path(model_dir), expected_tensors(spec))
+    return cfg, Model(spec, weights, runtime(dtype, device))

@@ -1,0 +1,235 @@
+"""Python face of the HIP kernels. Every function checks on the host that the
+operands' shapes, dtypes, strides and device fit what its kernel assumes, and
+only then launches on torch's current stream. There is no CPU or library
+fallback: a tensor that is not on the GPU, or a missing library, is an error."""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .csrc.build import load
+from .errors import AlofaError
+
+F32, BF16 = 0, 1
+STORE, ADD_TO_RESIDUAL = 0, 1
+MAX_HEAD_DIM = 256
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_L = ctypes.c_int64
+_F = ctypes.c_float
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype is torch.float32:
+        return F32
+    if t.dtype is torch.bfloat16:
+        return BF16
+    raise AlofaError("unsupported", "kernels take float32 or bfloat16 tensors", f"dtype={t.dtype}")
+
+
+def _gpu(name: str, t: torch.Tensor, dtype=None, dims: Optional[int] = None) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise AlofaError("invalid_argument", "kernel operand must be a GPU tensor", f"operand={name}")
+    if dtype is not None and t.dtype is not dtype:
+        raise AlofaError("invalid_argument", "kernel operand has the wrong dtype", f"operand={name} has={t.dtype} wants={dtype}")
+    if dims is not None and t.dim() != dims:
+        raise AlofaError("shape_mismatch", "kernel operand has the wrong rank", f"operand={name} shape={tuple(t.shape)} wants_rank={dims}")
+    return t
+
+
+def _rows(name: str, t: torch.Tensor) -> int:
+    """Leading dimension of a 2-d tensor whose rows are contiguous."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise AlofaError("shape_mismatch", "kernel operand must be 2-d with contiguous rows", f"operand={name} shape={tuple(t.shape)} strides={t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _contig(name: str, t: torch.Tensor) -> torch.Tensor:
+    if not t.is_contiguous():
+        raise AlofaError("shape_mismatch", "kernel operand must be contiguous", f"operand={name} shape={tuple(t.shape)} strides={t.stride()}")
+    return t
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _call(fn_name: str, *args) -> None:
+    lib = load()
+    if getattr(lib, fn_name)(*args) != 0:
+        raise AlofaError("invalid_argument", "kernel refused its arguments", lib.alofa_last_error().decode())
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return _P(t.data_ptr() if t is not None else None)
+
+
+# ----------------------------------------------------------------- embedding
+
+def embed_gather(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    """out[t] = table[ids[t]] widened to float32. ``ids`` must already be
+    checked against the vocabulary on the host."""
+    _gpu("out", out, torch.float32, 2), _gpu("table", table, None, 2), _gpu("ids", ids, torch.int32, 1)
+    _contig("out", out), _contig("table", table), _contig("ids", ids)
+    T, h = out.shape
+    if table.shape[1] != h or ids.shape[0] != T:
+        raise AlofaError("shape_mismatch", "embedding width or token count does not fit", f"out={tuple(out.shape)} table={tuple(table.shape)} ids={tuple(ids.shape)}")
+    _call("alofa_embed_gather", _ptr(out), _ptr(table), _I(dtype_code(table)), _ptr(ids), _I(T), _I(h), _stream())
+
+
+# ---------------------------------------------------------------------- norm
+
+def rmsnorm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, eps: float, exact: bool,
+            rows: Optional[torch.Tensor] = None) -> None:
+    """out[r] = rmsnorm(x[rows[r]] if rows is given else x[r]) * w."""
+    _gpu("out", out, None, 2), _gpu("x", x, torch.float32, 2), _gpu("w", w, torch.float32, 1)
+    _contig("out", out), _contig("x", x), _contig("w", w)
+    n, h = out.shape
+    if x.shape[1] != h or w.shape[0] != h:
+        raise AlofaError("shape_mismatch", "norm width does not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} w={tuple(w.shape)}")
+    if rows is not None:
+        _gpu("rows", rows, torch.int32, 1), _contig("rows", rows)
+        if rows.shape[0] != n:
+            raise AlofaError("shape_mismatch", "one row index per output row", f"rows={tuple(rows.shape)} out={tuple(out.shape)}")
+    elif x.shape[0] != n:
+        raise AlofaError("shape_mismatch", "norm row count does not fit", f"out={tuple(out.shape)} x={tuple(x.shape)}")
+    if exact and out.dtype is not torch.float32:
+        raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
+    _call("alofa_rmsnorm", _ptr(out), _I(dtype_code(out)), _ptr(x), _ptr(w), _ptr(rows), _I(n), _I(h), _F(eps), _I(int(exact)), _stream())
+
+
+# ------------------------------------------------------------ matrix product
+
+def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+         add_to_out: bool = False, exact: bool = False) -> None:
+    """out = a @ w.T (+ bias), or out += a @ w.T when ``add_to_out`` (out is then
+    the float32 residual stream). w is [out_features, in_features]."""
+    _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w", w, None, 2)
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(out.shape) != (M, N):
+        raise AlofaError("shape_mismatch", "matrix product shapes do not fit", f"a={tuple(a.shape)} w={tuple(w.shape)} out={tuple(out.shape)}")
+    if bias is not None:
+        _gpu("bias", bias, torch.float32, 1), _contig("bias", bias)
+        if bias.shape[0] != N:
+            raise AlofaError("shape_mismatch", "bias length does not fit", f"bias={tuple(bias.shape)} N={N}")
+    if add_to_out and out.dtype is not torch.float32:
+        raise AlofaError("invalid_argument", "the residual stream is float32", f"out={out.dtype}")
+    _call("alofa_gemm_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
+          _ptr(w), _I(dtype_code(w)), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
+          _I(ADD_TO_RESIDUAL if add_to_out else STORE), _I(int(exact)), _stream())
+
+
+def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, exact: bool = False) -> None:
+    """out = silu(a @ w_gate.T) * (a @ w_up.T)."""
+    _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w_gate", w_gate, None, 2), _gpu("w_up", w_up, None, 2)
+    M, K = a.shape
+    N = w_gate.shape[0]
+    if tuple(w_gate.shape) != (N, K) or tuple(w_up.shape) != (N, K) or tuple(out.shape) != (M, N):
+        raise AlofaError("shape_mismatch", "gate/up product shapes do not fit", f"a={tuple(a.shape)} gate={tuple(w_gate.shape)} up={tuple(w_up.shape)} out={tuple(out.shape)}")
+    if w_gate.dtype is not w_up.dtype or _rows("w_gate", w_gate) != _rows("w_up", w_up):
+        raise AlofaError("invalid_argument", "gate and up matrices must share dtype and layout")
+    _call("alofa_gemm_swiglu_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
+          _ptr(w_gate), _ptr(w_up), _I(dtype_code(w_gate)), _L(_rows("w_gate", w_gate)), _I(M), _I(N), _I(K), _I(int(exact)), _stream())
+
+
+def swiglu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, exact: bool = False) -> None:
+    for n, t in (("out", out), ("gate", gate), ("up", up)):
+        _gpu(n, t), _contig(n, t)
+    if out.shape != gate.shape or up.shape != gate.shape or out.dtype is not gate.dtype or up.dtype is not gate.dtype:
+        raise AlofaError("shape_mismatch", "swiglu operands must agree in shape and dtype")
+    _call("alofa_swiglu", _ptr(out), _ptr(gate), _ptr(up), _I(dtype_code(out)), _L(out.numel()), _I(int(exact)), _stream())
+
+
+# ----------------------------------------------------- positions + cache write
+
+def check_cache(name: str, cache: torch.Tensor, kv_heads: int, d: int) -> int:
+    """A cache is [blocks, kv_heads, block_size, d], contiguous. Returns block_size."""
+    _gpu(name, cache, None, 4), _contig(name, cache)
+    if cache.shape[1] != kv_heads or cache.shape[3] != d:
+        raise AlofaError("shape_mismatch", "cache does not fit the heads", f"{name}={tuple(cache.shape)} kv_heads={kv_heads} d={d}")
+    return cache.shape[2]
+
+
+def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                  heads: int, kv_heads: int, d: int, slots: Optional[torch.Tensor] = None,
+                  k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None) -> None:
+    """Rotate the query and key heads of qkv [T, (heads + 2 kv_heads) d] in place
+    by each token's position (half-split pairing); when caches are given, write
+    the rotated keys and the values to each token's slot. ``cos``/``sin`` are
+    float32 [positions, d/2]. Positions and slots are checked by the caller
+    against the table and the cache."""
+    _gpu("qkv", qkv, None, 2)
+    T = qkv.shape[0]
+    write = k_cache is not None
+    width = (heads + 2 * kv_heads) * d if write else qkv.shape[1]
+    if qkv.shape[1] != width or (not write and (heads + kv_heads) * d > width):
+        raise AlofaError("shape_mismatch", "qkv width does not fit the heads", f"qkv={tuple(qkv.shape)} heads={heads} kv_heads={kv_heads} d={d}")
+    _gpu("cos", cos, torch.float32, 2), _gpu("sin", sin, torch.float32, 2), _contig("cos", cos), _contig("sin", sin)
+    if cos.shape != sin.shape or cos.shape[1] != d // 2 or d % 2:
+        raise AlofaError("shape_mismatch", "rotary table must be [positions, d/2]", f"cos={tuple(cos.shape)} d={d}")
+    _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    if positions.shape[0] != T:
+        raise AlofaError("shape_mismatch", "one position per token", f"positions={tuple(positions.shape)} T={T}")
+    bs = 0
+    if write:
+        bs = check_cache("k_cache", k_cache, kv_heads, d)
+        check_cache("v_cache", v_cache, kv_heads, d)
+        if k_cache.shape != v_cache.shape or k_cache.dtype is not qkv.dtype or v_cache.dtype is not qkv.dtype:
+            raise AlofaError("shape_mismatch", "key and value caches must agree with each other and with qkv's dtype")
+        _gpu("slots", slots, torch.int64, 1), _contig("slots", slots)
+        if slots.shape[0] != T:
+            raise AlofaError("shape_mismatch", "one cache slot per token", f"slots={tuple(slots.shape)} T={T}")
+    _call("alofa_rope_kv_write", _ptr(qkv), _I(dtype_code(qkv)), _L(_rows("qkv", qkv)), _ptr(cos), _ptr(sin), _ptr(positions),
+          _ptr(slots if write else None), _ptr(k_cache), _ptr(v_cache), _I(T), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(write)), _stream())
+
+
+# ----------------------------------------------------------------- attention
+
+def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    block_table: torch.Tensor, req_of_token: torch.Tensor, positions: torch.Tensor,
+                    heads: int, kv_heads: int, d: int, window: Optional[int], scale: float, exact: bool) -> None:
+    """out[t] = attention of query token t (q [T, >= heads*d] rows, heads packed)
+    over the keys lo..positions[t] of its request's pages."""
+    _gpu("out", out, None, 2), _gpu("q", q, None, 2)
+    T = q.shape[0]
+    if out.shape[0] != T or out.shape[1] < heads * d or q.shape[1] < heads * d or out.dtype is not q.dtype:
+        raise AlofaError("shape_mismatch", "attention rows do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} heads={heads} d={d}")
+    if d % 2 or d > MAX_HEAD_DIM or d <= 0:
+        raise AlofaError("unsupported", f"head size must be even and at most {MAX_HEAD_DIM}", f"head_dim={d}")
+    bs = check_cache("k_cache", k_cache, kv_heads, d)
+    check_cache("v_cache", v_cache, kv_heads, d)
+    if k_cache.shape != v_cache.shape or k_cache.dtype is not q.dtype or v_cache.dtype is not q.dtype:
+        raise AlofaError("shape_mismatch", "caches must agree with each other and with q's dtype")
+    _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
+    _gpu("req_of_token", req_of_token, torch.int32, 1), _contig("req_of_token", req_of_token)
+    _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    if req_of_token.shape[0] != T or positions.shape[0] != T:
+        raise AlofaError("shape_mismatch", "one request index and one position per token")
+    _call("alofa_attention_simple", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
+          _I(dtype_code(q)), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T),
+          _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(int(exact)), _stream())
+
+
+# ------------------------------------------------------------------ sampling
+
+def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
+    """out[r] = first index of the maximum of logits[r] (lowest index on ties)."""
+    _gpu("out", out, torch.int32, 1), _gpu("logits", logits, torch.float32, 2), _contig("out", out)
+    if out.shape[0] != logits.shape[0]:
+        raise AlofaError("shape_mismatch", "one choice per row")
+    _call("alofa_argmax", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(logits.shape[0]), _I(logits.shape[1]), _stream())
+
+
+def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor) -> None:
+    """out[r] = inverse-CDF draw from softmax(logits[r] / temperature[r]) at uniform[r] in [0, 1)."""
+    _gpu("out", out, torch.int32, 1), _gpu("logits", logits, torch.float32, 2), _contig("out", out)
+    _gpu("temperature", temperature, torch.float64, 1), _gpu("uniform", uniform, torch.float64, 1)
+    _contig("temperature", temperature), _contig("uniform", uniform)
+    n = logits.shape[0]
+    if out.shape[0] != n or temperature.shape[0] != n or uniform.shape[0] != n:
+        raise AlofaError("shape_mismatch", "one choice, temperature and uniform number per row")
+    _call("alofa_sample", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(n), _I(logits.shape[1]), _ptr(temperature), _ptr(uniform), _stream())

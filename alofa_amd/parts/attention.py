@@ -1,0 +1,96 @@
+"""Grouped-query attention over a paged cache.
+
+q = x Wq^T + bq, k = x Wk^T + bk, v = x Wv^T + bv, heads packed in the channel
+dimension (channel = head * d + j); q and k take the position encoding, v does
+not; rotated k and v go to the token's cache slot; each query head attends the
+keys of key head (head // group) causally (optionally only the last ``window``
+keys), scale 1/sqrt(d); then the output projection, added to the residual
+stream (src/alofa/engine/executor.mojo:715-804, src/alofa/kernels/cpu/paged.mojo:249-336).
+
+The three input projections run as one matrix product: their matrices are
+stacked by rows ([out, in] layout, nothing is transposed)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..errors import AlofaError
+from ..weights.loader import TensorRule
+from .base import CacheNeed, Mixer, build_part, register_part
+
+
+class GQAAttention(Mixer):
+    """params: prefix, hidden, heads, kv_heads, head_dim, qkv_bias, out_bias,
+    window (None or a count of keys), position (PartSpec)."""
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        pre, h, qd, kvd = p["prefix"], p["hidden"], p["heads"] * p["head_dim"], p["kv_heads"] * p["head_dim"]
+        out = {pre + "q_proj.weight": TensorRule((qd, h)), pre + "k_proj.weight": TensorRule((kvd, h)),
+               pre + "v_proj.weight": TensorRule((kvd, h)), pre + "o_proj.weight": TensorRule((h, qd))}
+        if p.get("qkv_bias", False):
+            out.update({pre + "q_proj.bias": TensorRule((qd,), "bias"), pre + "k_proj.bias": TensorRule((kvd,), "bias"),
+                        pre + "v_proj.bias": TensorRule((kvd,), "bias")})
+        if p.get("out_bias", False):
+            out[pre + "o_proj.bias"] = TensorRule((h,), "bias")
+        return out
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.heads, self.kv_heads, self.d = int(p["hidden"]), int(p["heads"]), int(p["kv_heads"]), int(p["head_dim"])
+        self.window = p.get("window")
+        if self.kv_heads <= 0 or self.heads % self.kv_heads:
+            raise AlofaError("unsupported", "kv_heads must be positive and divide heads", f"heads={self.heads} kv_heads={self.kv_heads}")
+        if self.d % 16 or not 16 <= self.d <= ops.MAX_HEAD_DIM:
+            raise AlofaError("unsupported", f"the attention kernels take head sizes 16..{ops.MAX_HEAD_DIM} in steps of 16", f"head_dim={self.d}")
+        if self.window is not None and self.window <= 0:
+            raise AlofaError("invalid_argument", "an attention window must be positive", f"window={self.window}")
+        pre = p["prefix"]
+        mats = [weights[pre + n + "_proj.weight"] for n in ("q", "k", "v")]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        self.w_qkv = rt.matrix(torch.cat(mats, dim=0))
+        self.b_qkv = (rt.vector(torch.cat([weights[pre + n + "_proj.bias"].float() for n in ("q", "k", "v")]))
+                      if p.get("qkv_bias", False) else None)
+        self.w_o = rt.matrix(weights[pre + "o_proj.weight"])
+        self.b_o = rt.vector(weights[pre + "o_proj.bias"]) if p.get("out_bias", False) else None
+        self.position = build_part("position", p["position"], weights, rt)
+        # float32 1 / sqrt(float32 d), as the reference forms it (scalar.mojo:421)
+        self.scale = float(np.float32(1.0) / np.sqrt(np.float32(self.d)))
+        self.qkv_width = (self.heads + 2 * self.kv_heads) * self.d
+
+    def cache_need(self):
+        return CacheNeed(self.kv_heads, self.d, self.window)
+
+    def forward(self, ctx, entry, x, residual):
+        T = x.shape[0]
+        exact = self.rt.exact
+        qkv = ctx.scratch("qkv", (T, self.qkv_width), self.rt.dtype)
+        ops.gemm(qkv, x, self.w_qkv, self.b_qkv, exact=exact)
+        kv = ctx.kv(entry)
+        table = self.position.table(ctx.n_positions)
+        if table is None:
+            hd = self.heads * self.d
+            self.position.apply(ctx, qkv[:, :hd].unflatten(1, (self.heads, self.d)),
+                                qkv[:, hd:hd + self.kv_heads * self.d].unflatten(1, (self.kv_heads, self.d)))
+            table = ctx.identity_rotation(self.d)
+        cos, sin = table
+        if kv.owner:
+            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d, kv.slots, kv.k, kv.v)
+        else:
+            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
+        attn = ctx.scratch("attn", (T, self.heads * self.d), self.rt.dtype)
+        ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions,
+                            self.heads, self.kv_heads, self.d, self.window, self.scale, exact)
+        if self.b_o is not None:
+            proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
+            ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)
+            residual.add_(proj)
+        else:
+            ops.gemm(residual, attn, self.w_o, add_to_out=True, exact=exact)
+
+
+register_part("mixer", "gqa_attention", GQAAttention)

@@ -1,0 +1,39 @@
+"""Dense SwiGLU feed-forward: down(silu(gate(x)) * up(x)), no biases; silu is
+x / (1 + exp(-x)) (src/alofa/kernels/cpu/scalar.mojo:219-231,
+src/alofa/engine/executor.mojo:806-837). Gate and up run as one kernel that
+applies the activation before anything is written."""
+from __future__ import annotations
+
+from .. import ops
+from ..weights.loader import TensorRule
+from .base import FeedForward, register_part
+
+
+class SwiGLU(FeedForward):
+    """params: prefix, hidden, intermediate."""
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        pre, h, i = p["prefix"], p["hidden"], p["intermediate"]
+        return {pre + "gate_proj.weight": TensorRule((i, h)), pre + "up_proj.weight": TensorRule((i, h)),
+                pre + "down_proj.weight": TensorRule((h, i))}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.intermediate = int(p["hidden"]), int(p["intermediate"])
+        pre = p["prefix"]
+        gate, up = weights[pre + "gate_proj.weight"], weights[pre + "up_proj.weight"]
+        if gate.dtype is not up.dtype:
+            gate, up = gate.float(), up.float()
+        self.w_gate, self.w_up = rt.matrix(gate), rt.matrix(up)
+        self.w_down = rt.matrix(weights[pre + "down_proj.weight"])
+
+    def forward(self, ctx, x, residual):
+        act = ctx.scratch("ff_act", (x.shape[0], self.intermediate), self.rt.dtype)
+        ops.gemm_swiglu(act, x, self.w_gate, self.w_up, exact=self.rt.exact)
+        ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact)
+
+
+register_part("feed_forward", "swiglu", SwiGLU)

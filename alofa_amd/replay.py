@@ -1,0 +1,90 @@
+"""Trace replay: feeds given token ids through a model step by step and writes
+logits; it samples nothing. It drives the engine's own model, step function,
+cache and kernels — the ones generation uses.
+
+    bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+
+Steps come on standard input, one JSON object a line:
+
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+
+For a step in which something is wanted, ``DIR/<step>.f32`` receives the logits
+at the wanted places ([wanted, vocab] little-endian float32, in the order of the
+entries and of ``want``). After every step a line ``done <step>`` is printed."""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+from pathlib import Path
+
+from .errors import AlofaError
+
+
+class Replayer:
+    """The replay loop as an object: one ``step`` per input line."""
+
+    def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device: str = "cuda:0"):
+        from .csrc.build import load
+        load()  # compile at the first call if nothing is built; fail loudly if it cannot
+        from .cache.manager import CacheManager
+        from .engine.step import StepFunction
+        from .model import load_model
+
+        self.config, self.model = load_model(model_dir, dtype, device)
+        n_blocks = max(1, (int(max_tokens) + block_size - 1) // block_size)
+        self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), n_blocks, block_size,
+                                  max_requests=8, device=self.model.rt.device, dtype=self.model.rt.dtype)
+        self.fn = StepFunction(self.model, self.cache,
+                               n_positions=min(self.model.spec.max_positions, max(int(max_tokens), 64)))
+
+    def step(self, rec: dict):
+        """Run one step record; returns float32 logits [wanted, vocab] as a NumPy
+        array, or None when nothing is wanted."""
+        from .engine.step import StepEntry
+        entries = []
+        for e in rec.get("entries", []):
+            if not self.cache.has(e["id"]):
+                self.cache.admit(e["id"])
+            entries.append(StepEntry(e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+        out = None
+        if entries:
+            logits = self.fn.run(entries)
+            if logits is not None:
+                out = logits.detach().cpu().numpy().astype("<f4")
+        for r in rec.get("end", []):
+            if self.cache.has(r):
+                self.cache.free(r)
+        return out
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="trace_run", description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="most tokens live requests hold at any time (each request rounded up to a multiple of 64)")
+    ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
+    args = ap.parse_args(argv)
+    out = Path(args.out)
+    out.mkdir(parents=True, exist_ok=True)
+    replayer = Replayer(args.model, args.dtype, args.max_tokens, args.block_size)
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        rec = json.loads(line)
+        logits = replayer.step(rec)
+        if logits is not None:
+            logits.tofile(out / f"{rec['step']}.f32")
+        print(f"done {rec['step']}", flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    try:
+        sys.exit(main())
+    except AlofaError as e:
+        print(f"trace_run: {e}", file=sys.stderr)
+        sys.exit(1)

@@ -1,0 +1,61 @@
+"""Shared test set-up: markers, the repository on sys.path, tiny model folders."""
+import json
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+if str(ROOT / "tests") not in sys.path:
+    sys.path.insert(0, str(ROOT / "tests"))
+
+FIXTURES = Path(__file__).resolve().parent / "fixtures"
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an MI355X and the built HIP library")
+
+
+# Tiny configurations that differ in every size and option. A and B follow the
+# benchmark description's tiny models; C adds a sliding window on its upper
+# layers, an explicit head_dim key and a page-crossing window.
+TINY = {
+    "A": {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+        "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4,
+        "num_key_value_heads": 2, "intermediate_size": 176, "vocab_size": 256,
+        "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+        "use_sliding_window": False, "max_position_embeddings": 128,
+    },
+    "B": {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+        "num_hidden_layers": 3, "hidden_size": 96, "num_attention_heads": 3,
+        "num_key_value_heads": 1, "intermediate_size": 256, "vocab_size": 512,
+        "rope_theta": 1000000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": False,
+        "use_sliding_window": False, "max_position_embeddings": 256,
+    },
+    "C": {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+        "num_hidden_layers": 4, "hidden_size": 240, "num_attention_heads": 5,
+        "num_key_value_heads": 5, "head_dim": 48, "intermediate_size": 200,
+        "vocab_size": 331, "rope_theta": 50000.0, "rms_norm_eps": 3e-5,
+        "tie_word_embeddings": True, "use_sliding_window": True,
+        "sliding_window": 40, "max_window_layers": 1,
+        "max_position_embeddings": 512,
+    },
+}
+
+
+@pytest.fixture(scope="session")
+def tiny_dirs(tmp_path_factory):
+    """Model folders (config.json + model.safetensors) of the tiny
+    configurations, written by the engine's random-weights mode."""
+    from alofa_amd.weights import write_random_model
+    out = {}
+    for name, cfg in TINY.items():
+        d = tmp_path_factory.mktemp(f"tiny_{name}")
+        write_random_model(cfg, d, seed=1000 + ord(name))
+        out[name] = d
+    return out

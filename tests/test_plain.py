@@ -1,0 +1,225 @@
+"""The plain implementation, pinned by what fixes it beside the reference's
+text: vectors the reference's own tests hold (captured at the operator
+boundaries of layer 0 of the real model), special cases that reduce to a
+library routine, and invariants. Each check is chosen so that a plausible
+mistake fails it."""
+import math
+
+import numpy as np
+import pytest
+
+from conftest import FIXTURES
+from plain import model as pm
+from plain import sampler as ps
+
+
+@pytest.fixture(scope="module")
+def l0():
+    return np.load(FIXTURES / "layer0_subset.npz")
+
+
+def close(got, ref, rel=1e-5):
+    # the reference's own criterion: tests/unit/test_layer0_parity.mojo:46, :63-92
+    bound = rel * max(1.0, float(np.abs(ref).max()))
+    return float(np.abs(got.astype(np.float64) - ref.astype(np.float64)).max()) <= bound
+
+
+# ------------------------------------------------ vectors from the reference
+
+def test_rmsnorm_vectors(l0):
+    assert close(pm.rmsnorm(l0["embed_out"], l0["norm_w"], 1e-6), l0["norm_out"])
+    assert close(pm.rmsnorm(l0["hidden1"], l0["norm2_w"], 1e-6), l0["norm2_out"])
+    # a norm with 1+w, or with eps outside the root, must not pass
+    bad = pm.rmsnorm(l0["embed_out"], 1.0 + l0["norm_w"], 1e-6)
+    assert not close(bad, l0["norm_out"])
+
+
+def test_linear_bias_vector(l0):
+    assert close(pm.linear(l0["norm_out"], l0["k_w"], l0["k_b"]), l0["k_out"])
+    assert not close(pm.linear(l0["norm_out"], l0["k_w"]), l0["k_out"])
+
+
+def test_rope_vectors(l0):
+    cos, sin = pm.rope_table(16, 64, 1000000.0)
+    # derived table against the captured one: the reference measured 5.96e-8
+    # (tests/unit/test_real_model_dir.mojo:73-80)
+    assert np.abs(cos - l0["cos"]).max() <= 1e-6
+    assert np.abs(sin - l0["sin"]).max() <= 1e-6
+    pos = np.arange(16)
+    assert close(pm.rope_apply(l0["q_out"], l0["cos"], l0["sin"], pos, 64), l0["q_rot"])
+    assert close(pm.rope_apply(l0["k_out"], l0["cos"], l0["sin"], pos, 64), l0["k_rot"])
+    # wrong sign or an interleaved pairing must fail
+    assert not close(pm.rope_apply(l0["q_out"], l0["cos"], -l0["sin"], pos, 64), l0["q_rot"])
+    x = l0["q_out"].reshape(16, 14, 32, 2).transpose(0, 1, 3, 2).reshape(16, 896)
+    assert not close(pm.rope_apply(x, l0["cos"], l0["sin"], pos, 64), l0["q_rot"])
+
+
+def test_attention_vector(l0):
+    got = pm.attention(l0["q_rot"], l0["k_rot"], l0["v_out"], 14, 2, 64)
+    assert close(got, l0["attn_out"])
+    # head h reads key head h // 7; reading key head h % 2 must fail
+    k = l0["k_rot"].reshape(16, 2, 64)
+    kk = np.stack([k[:, h % 2] for h in range(14)], axis=1).reshape(16, 14 * 64)
+    v = l0["v_out"].reshape(16, 2, 64)
+    vv = np.stack([v[:, h % 2] for h in range(14)], axis=1).reshape(16, 14 * 64)
+    assert not close(pm.attention(l0["q_rot"], kk, vv, 14, 14, 64), l0["attn_out"])
+
+
+def test_residual_and_activation_vectors(l0):
+    assert close(pm.add(l0["embed_out"], l0["o_out"]), l0["hidden1"])
+    assert close(pm.silu(l0["gate_out"]), l0["silu_out"])
+    assert close(pm.swiglu(l0["gate_out"], l0["up_out"]), l0["swiglu_out"])
+    assert not close(pm.swiglu(l0["up_out"], l0["gate_out"]), l0["swiglu_out"])
+
+
+# ------------------------------------- special cases and invariants
+
+def test_rmsnorm_special_cases():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((3, 50)).astype(np.float32)
+    one = np.ones(50, dtype=np.float32)
+    want = x * math.sqrt(50) / np.linalg.norm(x.astype(np.float64), axis=1, keepdims=True)
+    assert np.allclose(pm.rmsnorm(x, one, 1e-12), want, rtol=1e-6)
+    assert np.allclose(pm.rmsnorm(7.0 * x, one, 1e-12), pm.rmsnorm(x, one, 1e-12), rtol=1e-6)
+    w = rng.standard_normal(50).astype(np.float32)
+    row = np.full((1, 50), -3.0, dtype=np.float32)
+    assert np.allclose(pm.rmsnorm(row, w, 1e-12), -w, rtol=1e-6)
+
+
+def test_linear_is_a_matrix_product():
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((5, 33)).astype(np.float32)
+    w = rng.standard_normal((7, 33)).astype(np.float32)
+    b = rng.standard_normal(7).astype(np.float32)
+    assert np.allclose(pm.linear(x, w, b), x.astype(np.float64) @ w.T.astype(np.float64) + b, rtol=1e-6)
+    assert np.array_equal(pm.linear(np.zeros_like(x), w, b), np.tile(b, (5, 1)))
+
+
+def test_rope_invariants():
+    d = 32
+    cos, sin = pm.rope_table(300, d, 1e6)
+    assert np.array_equal(cos[:, :16], cos[:, 16:]) and np.array_equal(sin[:, :16], sin[:, 16:])
+    assert np.abs(cos * cos + sin * sin - 1).max() < 1e-6
+    rng = np.random.default_rng(2)
+    q = rng.standard_normal((1, 2 * d)).astype(np.float32)
+    k = rng.standard_normal((1, 2 * d)).astype(np.float32)
+    assert np.array_equal(pm.rope_apply(q, cos, sin, [0], d), q)  # position 0 is the identity
+    r = pm.rope_apply(q, cos, sin, [123], d).reshape(2, d)
+    for j in range(16):  # each pair keeps its length
+        assert np.allclose(np.hypot(r[:, j], r[:, j + 16]), np.hypot(q.reshape(2, d)[:, j], q.reshape(2, d)[:, j + 16]), rtol=1e-5)
+
+    def dot(p, s):
+        return float(pm.rope_apply(q, cos, sin, [p], d)[0, :d].astype(np.float64)
+                     @ pm.rope_apply(k, cos, sin, [s], d)[0, :d].astype(np.float64))
+    assert abs(dot(17, 5) - dot(117, 105)) < 2e-4     # only the distance counts
+    assert abs(dot(17, 5) - dot(5, 17)) > 1e-3        # and its sign
+
+
+def test_attention_special_cases():
+    rng = np.random.default_rng(3)
+    H, d, L = 4, 16, 9
+    q = rng.standard_normal((L, H * d)).astype(np.float32)
+    k = rng.standard_normal((L, H * d)).astype(np.float32)
+    v = rng.standard_normal((L, H * d)).astype(np.float32)
+    # one key: the output is v
+    assert np.allclose(pm.attention(q[:1], k[:1], v[:1], H, H, d), v[:1])
+    # zero queries: the running mean of v
+    mean = np.cumsum(v.astype(np.float64), axis=0) / np.arange(1, L + 1)[:, None]
+    assert np.allclose(pm.attention(np.zeros_like(q), k, v, H, H, d), mean, atol=1e-6)
+    # as many key heads as query heads: library softmax over a masked product
+    from scipy.special import softmax
+    got = pm.attention(q, k, v, H, H, d)
+    for h in range(H):
+        s = q[:, h * d:(h + 1) * d].astype(np.float64) @ k[:, h * d:(h + 1) * d].astype(np.float64).T / math.sqrt(d)
+        s[np.triu_indices(L, 1)] = -np.inf
+        want = softmax(s, axis=1) @ v[:, h * d:(h + 1) * d].astype(np.float64)
+        assert np.allclose(got[:, h * d:(h + 1) * d], want, atol=2e-6)
+    # later keys do not change earlier rows; fewer queries than keys = the last rows
+    assert np.array_equal(pm.attention(q[:5], k[:5], v[:5], H, H, d), got[:5])
+    assert np.array_equal(pm.attention(q[6:], k, v, H, H, d), got[6:])
+    # a window as long as the sequence changes nothing; a window of one returns v
+    assert np.array_equal(pm.attention(q, k, v, H, H, d, window=L), got)
+    assert np.allclose(pm.attention(q, k, v, H, H, d, window=1), v)
+
+
+def test_swiglu_special_cases():
+    from scipy.special import expit
+    x = np.linspace(-30, 30, 101).astype(np.float32)
+    assert np.allclose(pm.swiglu(x, np.ones_like(x)), x * expit(x.astype(np.float64)), rtol=1e-6)
+    assert np.array_equal(pm.swiglu(np.zeros_like(x), x), np.zeros_like(x))
+    big = pm.swiglu(np.array([-1e4], dtype=np.float32), np.array([3.0], dtype=np.float32))
+    assert big[0] == 0 and not np.isnan(big[0])
+
+
+def test_argmax_lowest_index_on_ties():
+    assert pm.argmax(np.array([1, 5, 5, 2], dtype=np.float32)) == 1
+    assert pm.argmax(np.array([-3, -3], dtype=np.float32)) == 0
+
+
+def test_whole_model_shift_of_positions(tiny_dirs):
+    """Only distances between positions count: logits are the same when every
+    position is shifted, up to the rounding of the table."""
+    cfg = pm.read_config(tiny_dirs["B"])
+    w = pm.read_weights(tiny_dirs["B"])
+    ids = list(np.random.default_rng(4).integers(0, cfg["V"], 12))
+    a = pm.forward_logits(w, cfg, ids)
+    b = pm.forward_logits(w, cfg, ids, first_position=57)
+    assert a.shape == (12, cfg["V"])
+    assert np.abs(a - b).max() < 2e-4 * max(1.0, np.abs(a).max())
+    # earlier logits do not depend on later tokens
+    ids2 = ids[:7] + [(ids[7] + 1) % cfg["V"]] + ids[8:]
+    c = pm.forward_logits(w, cfg, ids2)
+    assert np.array_equal(a[:7], c[:7]) and not np.array_equal(a[7:], c[7:])
+
+
+def test_window_config_reaches_the_layers(tiny_dirs):
+    cfg = pm.read_config(tiny_dirs["C"])
+    assert cfg["windows"] == [None, 40, 40, 40] and cfg["d"] == 48
+    assert pm.read_config(tiny_dirs["A"])["windows"] == [None, None]
+
+
+# ------------------------------------------------------------------ sampler
+
+def test_splitmix64_vector():
+    rows = [l.split("\t") for l in (FIXTURES / "sampler" / "draws.tsv").read_text().splitlines()]
+    assert rows[0][0] == "seed"
+    rng = ps.SplitMix64(int(rows[0][1]))
+    for k, want in rows[1:]:
+        assert rng.next_u64() == int(want), k
+    u = ps.SplitMix64(7).next_uniform()
+    assert 0.0 <= u < 1.0
+
+
+def test_top_k_keeps_ties_at_the_threshold():
+    logits = np.fromfile(FIXTURES / "sampler" / "ties_logits.f32", dtype="<f4")
+    cases = dict(l.split("\t") for l in (FIXTURES / "sampler" / "ties_cases.tsv").read_text().splitlines())
+    for line in (FIXTURES / "sampler" / "ties_sets.tsv").read_text().splitlines():
+        name, count, members = line.split("\t")
+        values, probs = ps.distribution(logits, top_k=int(cases[name]))
+        alive = [i for i, v in enumerate(values) if v > ps.FLOOR]
+        assert alive == [int(m) for m in members.split(",")] and len(alive) == int(count)
+        assert abs(sum(probs) - 1.0) < 1e-12
+
+
+def test_sampler_special_cases():
+    from scipy.special import softmax
+    rng = np.random.default_rng(5)
+    logits = rng.standard_normal(40).astype(np.float32)
+    _, p = ps.distribution(logits)
+    assert np.allclose(p, softmax(logits.astype(np.float64)), rtol=1e-12)
+    _, p0 = ps.distribution(logits, temperature=0.0)
+    assert p0[int(np.argmax(logits))] == 1.0 and sum(p0) == 1.0
+    _, pc = ps.distribution(logits, temperature=0.001)
+    assert int(np.argmax(pc)) == int(np.argmax(logits)) and max(pc) > 0.99
+    assert ps.pick_from([0.25, 0.25, 0.5], 0.25) == 1
+    assert ps.pick_from([0.25, 0.25, 0.5], 0.2499) == 0
+    assert ps.pick_from([0.5, 0.5], 1.0) == 1
+    values, p = ps.distribution(logits, top_p=0.5)
+    kept = sorted(p, reverse=True)
+    n_alive = sum(1 for v in values if v > ps.FLOOR)
+    full = sorted(softmax(logits.astype(np.float64)), reverse=True)
+    assert sum(full[:n_alive]) >= 0.5 > sum(full[:n_alive - 1])
+    v2, _ = ps.distribution(np.array([2.0, -2.0], dtype=np.float32), repetition_penalty=2.0, history=[0, 1, 1])
+    assert v2 == [1.0, -4.0]
+    v3, _ = ps.distribution(np.array([2.0, -2.0], dtype=np.float32), frequency_penalty=0.5, presence_penalty=0.25, history=[1, 1])
+    assert v3 == [2.0, -3.25]
