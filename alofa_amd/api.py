@@ -1,0 +1,76 @@
+"""Python entry point: an engine over a model folder that generates tokens for
+batches of prompts (token ids; the tokenizer is outside this engine)."""
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Optional
+
+from .cache.manager import CacheManager
+from .engine.core import EngineCore
+from .engine.scheduler import SchedConfig
+from .engine.step import StepFunction
+from .errors import AlofaError
+from .model import load_model
+from .sampling.sampler import SampleParams
+
+
+class Engine:
+    """``max_tokens`` is the context window of one request (prompt + generated),
+    as the reference's ALOFA_MAX_TOKENS (src/alofa/srv/config.mojo:94-97).
+    ``kv_blocks`` pages of ``block_size`` tokens make the pool of each cache group;
+    by default enough for ``max_batch`` requests of ``max_tokens``."""
+
+    def __init__(self, model_dir, dtype: str = "bfloat16", max_tokens: int = 256, max_batch: int = 8,
+                 kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 256, max_chunk: int = 64,
+                 watermark_permille: int = 900, max_wait_ticks: int = 8, seed: int = 1234, device: str = "cuda:0",
+                 trace_path=None):
+        from .csrc.build import load
+        load()
+        self.config, self.model = load_model(Path(model_dir), dtype, device)
+        if max_tokens > self.model.spec.max_positions:
+            raise AlofaError("out_of_range", "max_tokens passes the model's position bound", f"max_tokens={max_tokens} max_position_embeddings={self.model.spec.max_positions}")
+        per_request = (max_tokens + block_size - 1) // block_size
+        if kv_blocks is None:
+            # enough for max_batch whole windows below the scheduler's watermark
+            kv_blocks = (per_request * max_batch * 1000 + watermark_permille - 1) // watermark_permille + 1
+        self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), kv_blocks, block_size,
+                                  max_requests=max(32, max_batch), device=self.model.rt.device, dtype=self.model.rt.dtype)
+        self.step_fn = StepFunction(self.model, self.cache, n_positions=max_tokens)
+        self.sched_cfg = SchedConfig(token_budget, max_chunk, block_size, kv_blocks, watermark_permille, max_wait_ticks,
+                                     n_slots=max(32, max_batch))
+        self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path)
+        self.seed = seed
+        self._next_id = 1
+
+    def generate(self, prompts: list, max_new: int = 16, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0,
+                 min_p: float = 0.0, repetition_penalty: float = 1.0, frequency_penalty: float = 0.0,
+                 presence_penalty: float = 0.0, seed: Optional[int] = None, max_ticks: int = 1 << 30) -> list:
+        """Greedy (temperature 0) or sampled continuation of every prompt; every
+        request draws from its own generator seeded with ``seed``."""
+        params = SampleParams(temperature=temperature, top_k=top_k, top_p=top_p, min_p=min_p,
+                              repetition_penalty=repetition_penalty, frequency_penalty=frequency_penalty,
+                              presence_penalty=presence_penalty)
+        use_seed = self.seed if seed is None else seed
+        ids, waiting = [], []
+        for p in prompts:
+            ids.append(self._next_id)
+            waiting.append((self._next_id, list(p)))
+            self._next_id += 1
+        ticks = 0
+        while waiting or self.core.has_work():
+            # requests the watermark cannot hold yet wait here until earlier ones end
+            while waiting and self.core.can_admit(len(waiting[0][1]), max_new):
+                rid, p = waiting.pop(0)
+                self.core.submit(rid, p, max_new, params, use_seed)
+            if not self.core.has_work():
+                raise AlofaError("capacity", "a request can never be admitted: it does not fit under the kv watermark",
+                                 f"prompt={len(waiting[0][1])} max_new={max_new}")
+            self.core.tick()
+            ticks += 1
+            if ticks > max_ticks:
+                raise AlofaError("capacity", "generation did not finish within the tick limit", f"max_ticks={max_ticks}")
+        outs = {}
+        for rid in ids:
+            outs[rid] = self.core.output(rid)
+            self.core.release(rid)
+        return [outs[rid] for rid in ids]

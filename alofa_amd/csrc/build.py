@@ -128,6 +128,9 @@ def load() -> ctypes.CDLL:
     no fallback: without the library nothing runs."""
     global _lib
     if _lib is None:
+        # torch first: its HIP runtime must be the one in the process, so that the
+        # library shares it (and torch's streams and memory) instead of loading a second copy
+        import torch  # noqa: F401
         path = find_built() or build()
         try:
             _lib = ctypes.CDLL(str(path))

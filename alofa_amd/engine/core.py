@@ -1,0 +1,245 @@
+"""The engine loop above the step function: prepare -> forward -> choose ->
+settle, one scheduler action per tick (src/alofa/engine/core.mojo:382-694).
+
+  prepare  reports last tick's news to the scheduler (arrivals, cancels,
+           completions, pages given back), takes its action, drops cancelled and
+           preempted requests from the cache, and turns prefill slices and
+           decodes into the entries of one step;
+  forward  runs the step function once;
+  choose   picks a token for every entry that owes one (greedy or sampled);
+  settle   records the tokens, queues each as its request's next row, and ends
+           requests that have produced ``max_new`` tokens: their pages go back
+           at once and the scheduler hears of it on the next tick.
+
+Preemption is recompute: the victim loses its pages, its generated tokens and
+its generator state, and is fed again from its first prompt token. There is no
+end-of-sequence check: a request ends by count or by cancel (core.mojo:659-665)."""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..errors import AlofaError
+from ..sampling.sampler import SampleParams, Sampler, SplitMix64
+from .scheduler import Action, SchedConfig, SchedInput, Scheduler, blocks_for
+from .step import StepEntry, StepFunction
+from .trace import config_line, trace_line
+
+QUEUED, RESIDENT, DONE = "queued", "resident", "done"
+
+
+@dataclass
+class Request:
+    id: int
+    prompt: list
+    max_new: int
+    params: SampleParams
+    seed: int
+    state: str = QUEUED
+    fed: int = 0                     # prompt tokens delivered to the cache
+    out: list = field(default_factory=list)
+    rng: Optional[SplitMix64] = None
+    reported: bool = False
+    preemptions: int = 0
+
+
+class EngineCore:
+    def __init__(self, step_fn: StepFunction, sched_cfg: SchedConfig, trace_path=None):
+        self.fn = step_fn
+        self.cache = step_fn.cache
+        pool_blocks = min((g.pool.n_blocks for g in self.cache.groups), default=sched_cfg.capacity_blocks)
+        if sched_cfg.capacity_blocks > pool_blocks:
+            raise AlofaError("invalid_argument", "the scheduler counts more blocks than the pool has", f"scheduler={sched_cfg.capacity_blocks} pool={pool_blocks}")
+        if sched_cfg.block_size != self.cache.block_size:
+            raise AlofaError("invalid_argument", "scheduler and cache disagree on the block size", f"scheduler={sched_cfg.block_size} cache={self.cache.block_size}")
+        self.sched = Scheduler(sched_cfg)
+        self.requests: dict = {}
+        self._arrivals: list = []
+        self._cancels: list = []
+        self._to_report: list = []
+        self._freed_blocks = 0
+        self.sampler = Sampler()
+        self.ticks = 0
+        self.last_rows = 0
+        self.last_action: Optional[Action] = None
+        self._trace = open(trace_path, "w") if trace_path else None
+        if self._trace:
+            self._trace.write(config_line(sched_cfg) + "\n")
+
+    # ------------------------------------------------------------ requests
+    def submit(self, req: int, prompt: list, max_new: int, params: Optional[SampleParams] = None, seed: int = 1234) -> None:
+        if req in self.requests:
+            raise AlofaError("invalid_argument", "duplicate request id", f"request={req}")
+        if len(prompt) == 0 or max_new <= 0:
+            raise AlofaError("invalid_argument", "a request needs a prompt and a positive max_new", f"request={req}")
+        if len(prompt) + max_new > self.fn.n_positions:
+            raise AlofaError("out_of_range", "prompt plus max_new passes the context bound", f"request={req} need={len(prompt) + max_new} bound={self.fn.n_positions}")
+        vocab = self.fn.model.spec.vocab_size
+        if min(prompt) < 0 or max(prompt) >= vocab:
+            raise AlofaError("out_of_range", "token id outside the vocabulary", f"request={req} vocab={vocab}")
+        self.requests[req] = Request(req, [int(t) for t in prompt], int(max_new), params or SampleParams(temperature=0.0), int(seed),
+                                     rng=SplitMix64(seed))
+        self._arrivals.append(req)
+
+    def can_admit(self, prompt_len: int, max_new: int) -> bool:
+        """Whether the scheduler would take such a request on the next tick."""
+        pending = tuple((len(self.requests[a].prompt), self.requests[a].max_new) for a in self._arrivals)
+        return self.sched.would_admit(prompt_len, max_new, pending)
+
+    def cancel(self, req: int) -> None:
+        if req in self.requests and self.requests[req].state != DONE:
+            self._cancels.append(req)
+
+    def is_done(self, req: int) -> bool:
+        return self.requests[req].state == DONE
+
+    def output(self, req: int) -> list:
+        return list(self.requests[req].out)
+
+    def release(self, req: int) -> None:
+        if self.requests[req].state != DONE:
+            raise AlofaError("invalid_argument", "only a finished request can be released", f"request={req}")
+        del self.requests[req]
+
+    def has_work(self) -> bool:
+        return (bool(self._arrivals) or bool(self._cancels) or bool(self._to_report) or self._freed_blocks > 0
+                or any(r.state != DONE for r in self.requests.values()))
+
+    # ---------------------------------------------------------------- tick
+    def _drop(self, r: Request) -> None:
+        if self.cache.has(r.id):
+            self.cache.free(r.id)
+
+    def prepare(self) -> list:
+        """One scheduler tick; returns the entries of the step and who owes a token."""
+        inp = SchedInput(
+            arrivals=[(a, len(self.requests[a].prompt), self.requests[a].max_new) for a in self._arrivals],
+            cancelled=list(self._cancels), finished=list(self._to_report), freed_blocks=self._freed_blocks)
+        arrivals, self._arrivals = self._arrivals, []
+        self._cancels, self._to_report, self._freed_blocks = [], [], 0
+        try:
+            act = self.sched.step(inp)
+        except AlofaError:
+            for a in arrivals:  # a refused admission retires the whole tick's arrivals
+                self.requests[a].state = DONE
+            raise
+        if self._trace:
+            self._trace.write(trace_line(inp, act) + "\n")
+            self._trace.flush()
+        self.last_action = act
+        for c in inp.cancelled:
+            r = self.requests.get(c)
+            if r is not None and r.state != DONE:
+                self._drop(r)
+                r.state = DONE
+        for p in act.preempted:
+            r = self.requests[p]
+            self._drop(r)
+            r.out, r.fed, r.state, r.rng = [], 0, QUEUED, SplitMix64(r.seed)
+            r.preemptions += 1
+        bs = self.sched.cfg.block_size
+        for f in act.finished:
+            # the scheduler moved this sequence's blocks to its "cached" count; this
+            # engine keeps no prefix cache, so they are reported back next tick
+            r = self.requests.get(f)
+            if r is not None:
+                self._freed_blocks += blocks_for(len(r.prompt) + r.max_new, bs)
+        entries, owes = [], []
+        for req, start, end in act.prefill:
+            r = self.requests[req]
+            if start == 0 and not self.cache.has(req):
+                self.cache.admit(req)
+            elif r.fed != start:
+                raise AlofaError("invalid_argument", "prefill slice does not continue the request", f"request={req} fed={r.fed} start={start}")
+            last = end == len(r.prompt)
+            entries.append(StepEntry(req, r.prompt[start:end], [end - start - 1] if last else []))
+            owes.append(req if last else None)
+            r.fed, r.state = end, RESIDENT
+        for req in act.decode:
+            r = self.requests[req]
+            if req in act.preempted or r.state == DONE:
+                continue
+            if r.state != RESIDENT or not r.out:
+                raise AlofaError("invalid_argument", "decode for a request that is not resident", f"request={req}")
+            entries.append(StepEntry(req, [r.out[-1]], [0]))
+            owes.append(req)
+        return entries, owes
+
+    def choose(self, logits: torch.Tensor, owes: list) -> list:
+        """One token per row of ``logits``, for the requests in ``owes`` (in order)."""
+        reqs = [self.requests[o] for o in owes]
+        chosen = [None] * len(reqs)
+        dev = [i for i, r in enumerate(reqs) if r.params.plain]
+        if dev:
+            greedy = [i for i in dev if r_is_greedy(reqs[i])]
+            drawn = [i for i in dev if not r_is_greedy(reqs[i])]
+            if greedy:
+                rows = logits if len(greedy) == len(reqs) else logits[torch.tensor(greedy, device=logits.device)]
+                out = torch.empty(len(greedy), dtype=torch.int32, device=logits.device)
+                ops.argmax(out, rows)
+                for i, t in zip(greedy, out.tolist()):
+                    chosen[i] = int(t)
+            if drawn:
+                rows = logits[torch.tensor(drawn, device=logits.device)].contiguous()
+                temp = torch.tensor([reqs[i].params.temperature for i in drawn], dtype=torch.float64, device=logits.device)
+                u = torch.tensor([reqs[i].rng.next_uniform() for i in drawn], dtype=torch.float64, device=logits.device)
+                out = torch.empty(len(drawn), dtype=torch.int32, device=logits.device)
+                ops.sample(out, rows, temp, u)
+                for i, t in zip(drawn, out.tolist()):
+                    chosen[i] = int(t)
+        host = [i for i in range(len(reqs)) if chosen[i] is None]
+        if host:
+            rows = logits[torch.tensor(host, device=logits.device)].cpu().numpy()
+            for k, i in enumerate(host):
+                r = reqs[i]
+                self.sampler.build(rows[k], r.params, r.prompt + r.out)
+                chosen[i] = self.sampler.pick(r.rng.next_uniform()) if not r.params.greedy else int(np.argmax(self.sampler.weights))
+        return chosen
+
+    def settle(self, owes: list, chosen: list) -> None:
+        it = iter(chosen)
+        for o in owes:
+            if o is None:
+                continue
+            r = self.requests[o]
+            r.out.append(next(it))
+            if len(r.out) >= r.max_new:
+                self._drop(r)
+                r.state = DONE
+                if self.sched.find(r.id) >= 0 and r.id not in self.last_action.finished:
+                    self._to_report.append(r.id)
+        for f in self.last_action.finished:
+            r = self.requests.get(f)
+            if r is not None and r.state != DONE:
+                self._drop(r)
+                r.state = DONE
+
+    def tick(self) -> int:
+        """One whole tick; returns the rows that ran."""
+        entries, owes = self.prepare()
+        self.ticks += 1
+        self.last_rows = sum(len(e.tokens) for e in entries)
+        if entries:
+            logits = self.fn.run(entries)
+            wanted = [o for o in owes if o is not None]
+            chosen = self.choose(logits, wanted) if wanted else []
+            self.settle(owes, chosen)
+        else:
+            self.settle([], [])
+        return self.last_rows
+
+    def run(self, max_ticks: int = 1 << 30) -> None:
+        n = 0
+        while self.has_work():
+            if n >= max_ticks:
+                raise AlofaError("capacity", "the engine did not finish within the tick limit", f"max_ticks={max_ticks}")
+            self.tick()
+            n += 1
+
+
+def r_is_greedy(r: Request) -> bool:
+    return r.params.greedy

@@ -147,13 +147,12 @@ class StepFunction:
             row += n
         return spans
 
-    def run(self, entries: list) -> Optional[torch.Tensor]:
-        """Run the step. Returns float32 logits [wanted, vocab] on the device in
-        the order of the entries and of their ``want`` lists, or None when nothing
-        is wanted."""
+    def begin(self, entries: list):
+        """Take the pages the entries need and lay the step out on the device.
+        Returns (context, token ids [T] int32, wanted rows or None). Either every
+        entry gets its pages or nothing is changed (capacity error)."""
         spans = self.plan(entries)
         cache = self.cache
-        # pages first: either every entry gets its pages or the step does not run
         need = [0] * len(cache.groups)
         for s in spans:
             for g, n in enumerate(cache.blocks_needed(s.request, s.pos0 + s.n)):
@@ -191,14 +190,23 @@ class StepFunction:
         slots_d = torch.from_numpy(slots).to(dev)
         ctx._tables = [tables_d[g] for g in range(n_groups)]
         ctx._slots = [slots_d[g] for g in range(n_groups)]
+        rows = torch.tensor(want_rows, dtype=torch.int32, device=dev) if want_rows else None
+        return ctx, ids_d, rows
 
-        hidden = self.model.forward(ctx, ids_d)
-        logits = None
-        if want_rows:
-            rows = torch.tensor(want_rows, dtype=torch.int32, device=dev)
-            logits = self.model.logits(ctx, hidden, rows)
-        for s in spans:
-            cache.commit(s.request, s.pos0 + s.n)
+    def finish(self, ctx: StepContext) -> None:
+        """The step's tokens are written: lengths advance and pages that a window
+        has passed go back to the pool."""
+        for s in ctx.spans:
+            self.cache.commit(s.request, s.pos0 + s.n)
         self.steps_run += 1
-        self.rows_run += T
+        self.rows_run += ctx.tokens
+
+    def run(self, entries: list) -> Optional[torch.Tensor]:
+        """Run the step. Returns float32 logits [wanted, vocab] on the device in
+        the order of the entries and of their ``want`` lists, or None when nothing
+        is wanted. The buffer is re-used by the next step."""
+        ctx, ids, rows = self.begin(entries)
+        hidden = self.model.forward(ctx, ids)
+        logits = self.model.logits(ctx, hidden, rows) if rows is not None else None
+        self.finish(ctx)
         return logits

@@ -1,0 +1,129 @@
+"""Helpers of the GPU tests: traces in the replay program's step format, cut in
+different ways, and the comparison with the plain implementation."""
+import functools
+
+import numpy as np
+
+from plain import model as pm
+
+
+def round64(n):
+    return (n + 63) // 64 * 64
+
+
+@functools.lru_cache(maxsize=None)
+def plain_model(model_dir):
+    return pm.read_config(model_dir), pm.read_weights(model_dir)
+
+
+def plain_logits(model_dir, ids):
+    cfg, w = plain_model(str(model_dir))
+    return pm.forward_logits(w, cfg, list(ids))
+
+
+def random_ids(seed, n, vocab):
+    return [int(t) for t in np.random.default_rng(seed).integers(0, vocab, n)]
+
+
+def bound(dtype, ref):
+    """float32: the reference's criterion 1e-5 * max(1, max|ref|)
+    (tests/unit/test_layer0_parity.mojo:46 there). bfloat16: activations are
+    rounded to 8 bits of mantissa between kernels; 1e-2 of the same scale."""
+    return (1e-5 if dtype == "float32" else 1e-2) * max(1.0, float(np.abs(ref).max()))
+
+
+def assert_close(got, ref, dtype, what=""):
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+    assert np.isfinite(got).all(), f"{what}: not finite"
+    err = np.abs(got - ref)
+    b = bound(dtype, ref)
+    if err.max() > b:
+        at = np.unravel_index(np.argmax(err), err.shape)
+        first = int(np.argmax(err.reshape(err.shape[0], -1).max(axis=1) > b))
+        raise AssertionError(f"{what}: max abs diff {err.max():.3e} > {b:.3e} at {at}; first wrong row {first}")
+    if got.ndim == 2 and got.shape[1] > 8:
+        cos = (got * ref).sum(1) / (np.linalg.norm(got, axis=1) * np.linalg.norm(ref, axis=1) + 1e-30)
+        assert cos.min() >= (0.999999 if dtype == "float32" else 0.999), f"{what}: cosine {cos.min()}"
+
+
+# ------------------------------------------------------------------ cuttings
+
+def whole(req, ids, step0=0):
+    return [{"step": step0, "entries": [{"id": req, "tokens": list(ids), "want": list(range(len(ids)))}], "end": [req]}]
+
+
+def bulk_and_tail(req, ids, tail=32, step0=0):
+    """Most of it in one step, the last ``tail`` tokens one by one."""
+    n = len(ids) - tail
+    steps = [{"step": step0, "entries": [{"id": req, "tokens": list(ids[:n]), "want": list(range(n))}], "end": []}]
+    for i in range(n, len(ids)):
+        steps.append({"step": step0 + len(steps), "entries": [{"id": req, "tokens": [ids[i]], "want": [0]}],
+                      "end": [req] if i == len(ids) - 1 else []})
+    return steps
+
+
+def portions(req, ids, sizes=(7, 2, 16, 3, 2, 31, 5, 2, 17), step0=0):
+    steps, pos, k = [], 0, 0
+    while pos < len(ids):
+        n = min(sizes[k % len(sizes)], len(ids) - pos)
+        if len(ids) - pos - n == 1:      # never leave a single token: portions go down to two, not one
+            n += 1
+        k += 1
+        steps.append({"step": step0 + len(steps), "entries": [{"id": req, "tokens": list(ids[pos:pos + n]), "want": list(range(n))}],
+                      "end": [req] if pos + n == len(ids) else []})
+        pos += n
+    return steps
+
+
+def mixed(requests, seed, tail=32, max_live=4, step0=0):
+    """Up to ``max_live`` live requests: portions of some beside single decoded
+    tokens of others, a request left out of a step now and then; a finished
+    request ends and the next one starts, so its pages are used again.
+    Returns (steps, peak of the live requests' token counts rounded up to 64)."""
+    rnd = np.random.default_rng(seed)
+    waiting = list(requests.items())
+    live, pos, steps, peak = [], {}, [], 0
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            r, ids = waiting.pop(0)
+            live.append(r)
+            pos[r] = 0
+        entries, ended = [], []
+        for r in list(live):
+            ids = requests[r]
+            if len(live) > 1 and rnd.random() < 0.2:
+                continue                                       # left out of this step
+            left = len(ids) - pos[r]
+            if left <= tail:
+                n = 1                                          # decoding: one token
+            else:
+                n = int(min(rnd.integers(2, 24), left - tail))
+                if left - tail - n == 1:
+                    n += 1
+            entries.append({"id": r, "tokens": list(ids[pos[r]:pos[r] + n]), "want": list(range(n))})
+            pos[r] += n
+            if pos[r] == len(ids):
+                ended.append(r)
+        peak = max(peak, sum(round64(len(requests[r])) for r in live))
+        for r in ended:
+            live.remove(r)
+        if entries:
+            steps.append({"step": step0 + len(steps), "entries": entries, "end": ended})
+    return steps, peak
+
+
+def collect(replayer, steps):
+    """Run steps through a Replayer; returns {request: [logits row per position]}."""
+    out, at = {}, {}
+    for rec in steps:
+        logits = replayer.step(rec)
+        k = 0
+        for e in rec["entries"]:
+            base = at.get(e["id"], 0)
+            for w in e["want"]:
+                out.setdefault(e["id"], {})[base + w] = logits[k].copy()
+                k += 1
+            at[e["id"]] = base + len(e["tokens"])
+        assert (logits is None and k == 0) or logits.shape[0] == k
+    return {r: np.stack([rows[p] for p in sorted(rows)]) for r, rows in out.items()}

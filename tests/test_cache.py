@@ -1,0 +1,149 @@
+"""The cache manager's accounting (no GPU): no page lost, held twice or freed
+twice, under random orders of requests; windows give pages back; pages are
+used again; state slots."""
+import random
+
+import pytest
+
+from alofa_amd.cache import BlockPool, CacheManager, blocks_for
+from alofa_amd.errors import AlofaError
+from alofa_amd.parts import CacheNeed, StateNeed
+
+
+def err_name(fn, *a):
+    with pytest.raises(AlofaError) as e:
+        fn(*a)
+    return e.value.name
+
+
+def test_pool_order_and_errors():
+    # order is the reference's contract (src/alofa/runtime/kv/pool.mojo:8-12, :42-46)
+    p = BlockPool(4)
+    assert [p.alloc_one() for _ in range(3)] == [0, 1, 2]
+    assert p.release(1) is True and p.alloc_one() == 1          # a released page is the next one out
+    p.retain(2)
+    assert p.release(2) is False and p.refcnt_of(2) == 1 and p.release(2) is True
+    assert err_name(p.release, 2) == "double_free" and err_name(p.retain, 2) == "double_free"
+    assert err_name(p.release, 9) == "out_of_range"
+    assert p.alloc_one() == 2 and p.alloc_one() == 3
+    assert err_name(p.alloc_one) == "capacity"
+    assert p.n_free + p.used == 4 and p.high_water == 4
+    assert err_name(BlockPool, 0) == "invalid_argument"
+
+
+def manager(n_blocks=12, windows=(None, 24, 24, None), state=False, bs=8):
+    needs = [CacheNeed(2, 16, w) for w in windows]
+    states = [StateNeed((4,)) if state else None for _ in windows]
+    return CacheManager(needs, states, n_blocks, bs, max_requests=4)
+
+
+def test_groups_by_need():
+    m = manager()
+    assert [(g.window, g.entries) for g in m.groups] == [(None, [0, 3]), (24, [1, 2])]
+    assert m.group_of_entry == {0: 0, 3: 0, 1: 1, 2: 1}
+    shared = CacheManager([CacheNeed(1, 16), None, CacheNeed(1, 16)], [None] * 3, 4, 8)
+    assert shared.groups[0].entries == [0, 2]
+
+
+def test_tables_grow_and_windows_give_pages_back():
+    m = manager()
+    m.admit("a")
+    m.reserve("a", 20)
+    assert m.table("a", 0) == [0, 1, 2] and m.table("a", 1) == [0, 1, 2]
+    assert m.slots("a", 0, 6, 4) == [6, 7, 8, 9]
+    assert m.commit("a", 20) == [[], []]                    # window 24 not yet passed
+    m.reserve("a", 41)
+    m.commit("a", 41)                                       # next query 41 sees keys >= 18: blocks 0, 1 passed
+    assert m.table("a", 1)[:2] == [-1, -1] and m.table("a", 0)[:2] == [0, 1]
+    assert m.groups[1].pool.n_free == 12 - 6 + 2
+    assert err_name(m.slots, "a", 1, 3, 2) == "capacity"    # no page behind the window
+    m.check()
+    m.admit("b")
+    m.reserve("b", 8)
+    assert m.table("b", 1) == [1] and m.table("b", 0) == [6]    # the page the window gave back is used again
+    m.free("a")
+    m.check()
+    assert m.groups[0].pool.n_free == 11 and m.groups[1].pool.n_free == 11
+    assert err_name(m.free, "a") == "invalid_argument"
+
+
+def test_reserve_is_all_or_nothing():
+    m = manager(n_blocks=4, windows=(None,))
+    m.admit("a"), m.admit("b")
+    m.reserve("a", 24)
+    assert err_name(m.reserve, "b", 17) == "capacity"
+    assert m.table("b", 0) == [] and m.groups[0].pool.n_free == 1
+    m.reserve("b", 8)
+    assert err_name(m.reserve, "a", 25) == "capacity"
+    m.commit("a", 24)
+    assert err_name(m.reserve, "a", 10) == "invalid_argument"   # a request cannot shrink
+    m.check()
+    assert err_name(m.commit, "b", 9) == "invalid_argument"     # beyond what was reserved
+    assert err_name(m.admit, "a") == "invalid_argument"
+    m.admit("c"), m.admit("d")
+    assert err_name(m.admit, "e") == "capacity"                 # request slots run out
+
+
+def test_shared_prefix_by_reference_count():
+    m = manager(n_blocks=8, windows=(None, None))
+    m.admit("a")
+    m.reserve("a", 20), m.commit("a", 20)
+    m.admit("b")
+    assert m.share_prefix("a", "b", 20) == 16                   # whole blocks only
+    assert m.table("b", 0) == [0, 1] and m.groups[0].pool.refcnt_of(0) == 2
+    m.reserve("b", 20)
+    assert m.table("b", 0) == [0, 1, 3]                         # never the tail of a shared block
+    m.check()
+    m.free("a")
+    assert m.groups[0].pool.refcnt_of(0) == 1 and m.groups[0].pool.refcnt_of(2) == 0
+    m.free("b")
+    m.check()
+    assert m.groups[0].pool.n_free == 8
+    w = manager()
+    w.admit("a"), w.reserve("a", 8), w.commit("a", 8), w.admit("b")
+    assert w.share_prefix("a", "b", 8) == 0                     # window groups do not share
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_the_invariants(seed):
+    rnd = random.Random(seed)
+    bs = rnd.choice([4, 8, 16])
+    m = manager(n_blocks=rnd.randint(10, 24), windows=(None, rnd.choice([5, 17, 40]), None), bs=bs)
+    live, names = {}, iter(range(10_000))
+    for _ in range(400):
+        op = rnd.random()
+        if op < 0.25 and len(live) < 4:
+            r = next(names)
+            m.admit(r)
+            live[r] = 0
+        elif op < 0.85 and live:
+            r = rnd.choice(list(live))
+            target = live[r] + rnd.randint(1, 3 * bs)
+            try:
+                m.reserve(r, target)
+                m.commit(r, target)
+                live[r] = target
+                w = m.groups[1].window
+                held = [b for b in m.table(r, 1) if b >= 0]
+                assert len(held) <= blocks_for(w, bs) + 1          # a window holds a bounded number of pages
+                assert len(m.table(r, 0)) == blocks_for(target, bs)
+                assert m.slots(r, 1, max(0, target - w), min(w, target))
+            except AlofaError as e:
+                assert e.name == "capacity"
+        elif live:
+            r = rnd.choice(list(live))
+            m.free(r)
+            del live[r]
+        m.check()
+    for r in list(live):
+        m.free(r)
+    m.check()
+    assert all(g.pool.n_free == g.pool.n_blocks for g in m.groups) and len(m.free_slots) == 4
+
+
+def test_state_slots_without_a_device_are_counted_only():
+    m = manager(state=True)
+    s = m.admit("a")
+    assert s == 0 and m.slot("a") == 0 and m.admit("b") == 1
+    m.free("a")
+    assert m.admit("c") == 0                                      # the slot is used again

@@ -1,0 +1,165 @@
+"""The engine against the plain implementation on the GPU, in float32 and in
+bfloat16: every way of cutting the same requests into steps must give the same
+logits at every position."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, TINY
+from helpers import (assert_close, bound, bulk_and_tail, collect, mixed, plain_logits, portions, random_ids, round64, whole)
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"A": 100, "B": 150, "C": 190}
+
+
+@pytest.fixture(scope="module")
+def replayers(tiny_dirs):
+    from alofa_amd.replay import Replayer
+    made = {}
+
+    def get(name, dtype, max_tokens=512, block_size=16):
+        key = (name, dtype, max_tokens, block_size)
+        if key not in made:
+            made[key] = Replayer(tiny_dirs[name], dtype, max_tokens, block_size)
+        r = made[key]
+        assert not r.cache.requests, "a test left requests behind"
+        return r
+    return get
+
+
+def ids_of(name, seed=11, n=None):
+    return random_ids(seed, n or LENGTHS[name], TINY[name]["vocab_size"])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_alone_and_whole(replayers, tiny_dirs, name, dtype):
+    ids = ids_of(name)
+    got = collect(replayers(name, dtype), whole("w", ids))["w"]
+    assert_close(got, plain_logits(tiny_dirs[name], tuple(ids)), dtype, f"{name} whole")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_bulk_then_last_32_one_by_one(replayers, tiny_dirs, name, dtype):
+    ids = ids_of(name)
+    got = collect(replayers(name, dtype), bulk_and_tail("t", ids))["t"]
+    assert_close(got, plain_logits(tiny_dirs[name], tuple(ids)), dtype, f"{name} bulk+tail")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(replayers, tiny_dirs, name, dtype):
+    ids = ids_of(name)
+    steps = portions("p", ids)
+    assert min(len(s["entries"][0]["tokens"]) for s in steps) == 2
+    got = collect(replayers(name, dtype), steps)["p"]
+    assert_close(got, plain_logits(tiny_dirs[name], tuple(ids)), dtype, f"{name} portions")
+    other = collect(replayers(name, dtype), portions("q", ids, sizes=(2, 29, 2, 2, 40, 3)))["q"]
+    assert_close(other, plain_logits(tiny_dirs[name], tuple(ids)), dtype, f"{name} other portions")
+    if dtype == "float32":                      # the cut changes nothing beyond rounding
+        assert np.abs(other - got).max() <= 1e-6 * max(1.0, np.abs(got).max())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_requests_with_pages_used_again(tiny_dirs, name, dtype):
+    from alofa_amd.replay import Replayer
+    vocab, top = TINY[name]["vocab_size"], LENGTHS[name]
+    requests = {f"r{i}": random_ids(100 + i, n, vocab) for i, n in enumerate([top, 41, top - 37, 64, 35, top - 9, 50])}
+    steps, peak = mixed(requests, seed=5)
+    assert max(len(s["entries"]) for s in steps) == 4
+    assert any(len(e["tokens"]) > 1 for s in steps for e in s["entries"]) and any(
+        len({len(e["tokens"]) == 1 for e in s["entries"]}) == 2 for s in steps), "portions beside decoded tokens"
+    r = Replayer(tiny_dirs[name], dtype, peak)           # so few pages that they are used again
+    got = collect(r, steps)
+    pool = r.cache.groups[0].pool
+    assert pool.high_water <= pool.n_blocks and sum(round64(len(v)) for v in requests.values()) > peak
+    r.cache.check()
+    assert all(g.pool.n_free == g.pool.n_blocks for g in r.cache.groups)
+    for k, ids in requests.items():
+        assert_close(got[k], plain_logits(tiny_dirs[name], tuple(ids)), dtype, f"{name} mixed {k}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(replayers, tiny_dirs, dtype):
+    ids = ids_of("C", seed=3, n=400)                     # crosses many pages and the window many times
+    got = collect(replayers("C", dtype), bulk_and_tail("d", ids, tail=380))["d"]
+    assert_close(got, plain_logits(tiny_dirs["C"], tuple(ids)), dtype, "C long decode")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_first_tokens_of_a_sequence(replayers, tiny_dirs, name, dtype):
+    ids = ids_of(name, seed=9, n=5)
+    ref = plain_logits(tiny_dirs[name], tuple(ids))
+    assert_close(collect(replayers(name, dtype), whole("f", ids[:1]))["f"], ref[:1], dtype, "one token")
+    assert_close(collect(replayers(name, dtype), bulk_and_tail("g", ids, tail=4))["g"], ref, dtype, "token by token from the first")
+    assert_close(collect(replayers(name, dtype), whole("h", ids[:2]))["h"], ref[:2], dtype, "two tokens")
+
+
+@pytest.mark.parametrize("block_size", [16, 32, 64])
+def test_page_size_does_not_matter(replayers, tiny_dirs, block_size):
+    ids = ids_of("B")
+    ref = plain_logits(tiny_dirs["B"], tuple(ids))
+    assert_close(collect(replayers("B", "float32", 512, block_size), portions("p", ids))["p"], ref, "float32", f"page {block_size}")
+
+
+def test_causality_and_other_tables(replayers, tiny_dirs):
+    """A changed token changes the logits from its place on and not before; a
+    request never sees another request's pages."""
+    ids = ids_of("A")
+    changed = list(ids)
+    changed[40] = (changed[40] + 1) % TINY["A"]["vocab_size"]
+    r = replayers("A", "float32")
+    a = collect(r, portions("a", ids))["a"]
+    b = collect(r, portions("b", changed))["b"]
+    assert np.array_equal(a[:40], b[:40]) and not np.array_equal(a[40], b[40]) and not np.array_equal(a[-1], b[-1])
+    # two requests side by side equal each alone
+    both = collect(r, [{"step": 0, "entries": [{"id": "x", "tokens": ids[:30], "want": [29]},
+                                                {"id": "y", "tokens": changed[:50], "want": [49]}], "end": ["x", "y"]}])
+    assert np.array_equal(both["x"][0], a[29]) and np.array_equal(both["y"][0], b[49])
+
+
+def test_trace_run_program(tiny_dirs, tmp_path):
+    """The program itself: steps on standard input, <step>.f32 files, 'done' lines, exit 0."""
+    ids = ids_of("B", seed=21, n=90)
+    steps = bulk_and_tail("a", ids, tail=32)
+    steps[3]["entries"][0]["want"] = []                        # a step in which nothing is wanted writes no file
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    env = dict(os.environ, HOME=str(tmp_path / "home"))
+    p = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(tiny_dirs["B"]), "--dtype", "float32",
+                        "--out", str(tmp_path / "out"), "--max-tokens", "128"], input=text, capture_output=True, text=True, env=env, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert p.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    ref = plain_logits(tiny_dirs["B"], tuple(ids))
+    first = np.fromfile(tmp_path / "out" / "0.f32", dtype="<f4").reshape(-1, TINY["B"]["vocab_size"])
+    assert_close(first, ref[:58], "float32", "program, first step")
+    assert not (tmp_path / "out" / "3.f32").exists()
+    last = np.fromfile(tmp_path / "out" / f"{steps[-1]['step']}.f32", dtype="<f4").reshape(1, -1)
+    assert_close(last, ref[-1:], "float32", "program, last step")
+    # unknown dtype and a missing model are refused, not worked around
+    bad = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(tmp_path / "none"), "--dtype", "float32",
+                          "--out", str(tmp_path / "o2"), "--max-tokens", "64"], input="", capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "config.json" in bad.stderr
+
+
+def test_pool_too_small_is_a_named_error(tiny_dirs):
+    from alofa_amd.errors import AlofaError
+    from alofa_amd.replay import Replayer
+    r = Replayer(tiny_dirs["A"], "float32", 64)
+    ids = ids_of("A", n=100)
+    with pytest.raises(AlofaError) as e:
+        r.step(whole("a", ids)[0])
+    assert e.value.name == "capacity"
+    r.cache.check()
+    assert r.cache.groups[0].pool.n_free == r.cache.groups[0].pool.n_blocks   # nothing was taken
+    with pytest.raises(AlofaError) as e:
+        r.step({"step": 1, "entries": [{"id": "b", "tokens": [TINY["A"]["vocab_size"]], "want": [0]}], "end": []})
+    assert e.value.name == "out_of_range"

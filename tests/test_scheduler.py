@@ -1,0 +1,136 @@
+"""The scheduler's decisions. The traces are the reference's own fixtures
+(tests/fixtures/scheduler/*.trace there): each line holds a tick's input and the
+expected action with the state digest, compared byte for byte; bad.trace and
+alt.trace are its negative controls and must not match."""
+import pytest
+
+from conftest import FIXTURES
+from alofa_amd.engine.scheduler import Action, SchedConfig, SchedInput, Scheduler, blocks_for
+from alofa_amd.engine.trace import action_line, config_line, input_line, parse_config, parse_input, trace_line
+from alofa_amd.errors import AlofaError
+
+TRACES = sorted(p.name for p in (FIXTURES / "scheduler").glob("s0*.trace"))
+
+
+def replay(path):
+    """Yields (expected line, produced line); checks the per-tick invariants
+    (the reference's five: tests/unit/test_scheduler.mojo:136-156)."""
+    lines = path.read_text().splitlines()
+    cfg = parse_config(lines[0])
+    assert config_line(cfg) == lines[0]
+    s = Scheduler(cfg)
+    for line in lines[1:]:
+        inp = parse_input(line.split(" OUT=")[0])
+        assert input_line(inp) == line.split(" OUT=")[0]
+        try:
+            act = s.step(inp)
+            got = trace_line(inp, act)
+            assert act.tokens() <= cfg.token_budget
+            assert s.blocks_used <= cfg.capacity_blocks
+            assert s.blocks_used == s.blocks_held() + s.cached_blocks
+            assert len({r for r, _, _ in act.prefill}) == len(act.prefill)
+            if s.blocks_used > cfg.threshold_blocks:
+                assert not any(s.state[i] == 2 and s.done[i] + s.generated[i] > 0 for i in range(cfg.n_slots))
+        except AlofaError as e:
+            got = input_line(inp) + " ERR=" + e.name
+        yield line, got
+
+
+@pytest.mark.parametrize("name", TRACES)
+def test_reference_traces_byte_for_byte(name):
+    pairs = list(replay(FIXTURES / "scheduler" / name))
+    assert len(pairs) > 3
+    for want, got in pairs:
+        assert got == want
+
+
+@pytest.mark.parametrize("name", ["bad.trace", "alt.trace"])
+def test_negative_controls_do_not_match(name):
+    assert any(want != got for want, got in replay(FIXTURES / "scheduler" / name))
+
+
+def test_replay_is_deterministic():
+    a = [g for _, g in replay(FIXTURES / "scheduler" / "s02_preempt_storm.trace")]
+    b = [g for _, g in replay(FIXTURES / "scheduler" / "s02_preempt_storm.trace")]
+    assert a == b
+
+
+def test_prompt_is_cut_under_the_budget_and_decode_goes_first():
+    s = Scheduler(SchedConfig(token_budget=10, max_chunk=8, block_size=4, capacity_blocks=64))
+    a = s.step(SchedInput(arrivals=[(1, 20, 3), (2, 5, 2)]))
+    assert a.prefill == [(1, 0, 8), (2, 0, 2)] and a.decode == []
+    a = s.step(SchedInput())
+    assert a.prefill == [(1, 8, 16), (2, 2, 4)]
+    a = s.step(SchedInput())
+    assert a.prefill == [(1, 16, 20), (2, 4, 5)]
+    a = s.step(SchedInput())          # both promoted: decode before any prefill
+    assert a.decode == [1, 2] and a.prefill == []
+    a = s.step(SchedInput(arrivals=[(3, 30, 1)]))
+    assert a.decode == [1, 2] and a.finished == [2] and a.prefill == [(3, 0, 8)]
+    assert a.tokens() <= 10
+
+
+def test_pages_run_out():
+    # admission refused against the watermark, atomically for the tick
+    s = Scheduler(SchedConfig(token_budget=64, max_chunk=64, block_size=4, capacity_blocks=10, watermark_permille=800))
+    with pytest.raises(AlofaError) as e:
+        s.step(SchedInput(arrivals=[(1, 8, 8), (2, 16, 8)]))
+    assert e.value.name == "capacity" and s.n_live() == 0 and s.blocks_used == 0
+    # prefill waits when pages are gone (hard capacity), nothing is preempted for it
+    s = Scheduler(SchedConfig(token_budget=64, max_chunk=64, block_size=4, capacity_blocks=6, watermark_permille=1000))
+    a = s.step(SchedInput(arrivals=[(1, 12, 4)]))
+    assert a.prefill == [(1, 0, 12)]
+    s.cfg = SchedConfig(token_budget=64, max_chunk=64, block_size=4, capacity_blocks=6, watermark_permille=1000)
+    a = s.step(SchedInput())
+    assert a.decode == [1]
+    # decode that needs a page preempts the newest running request, which restarts
+    # from zero. Admission keeps live sequences under the watermark, so pages can
+    # only run out while blocks of a finished request are still counted as cached.
+    s = Scheduler(SchedConfig(token_budget=64, max_chunk=64, block_size=4, capacity_blocks=6, watermark_permille=1000))
+    s.step(SchedInput(arrivals=[(1, 4, 1)]))
+    assert s.step(SchedInput()).finished == [1] and s.cached_blocks == 2
+    s.step(SchedInput(arrivals=[(2, 6, 6), (3, 6, 6)]))
+    seen = None
+    for _ in range(6):
+        a = s.step(SchedInput())
+        assert s.blocks_used <= 6 and s.blocks_used == s.blocks_held() + s.cached_blocks
+        if a.preempted:
+            seen = a
+            break
+    assert seen is not None and seen.preempted == [3] and 2 in seen.decode and 3 not in seen.decode
+    slot = s.find(3)
+    assert s.done[slot] == 0 and s.generated[slot] == 0 and s.state[slot] == 1 and s.preempt_count[slot] == 1
+    # nobody left to preempt: an error, not a dropped token
+    s = Scheduler(SchedConfig(token_budget=64, max_chunk=64, block_size=4, capacity_blocks=3, watermark_permille=1000))
+    s.step(SchedInput(arrivals=[(1, 4, 1)]))
+    s.step(SchedInput())
+    s.step(SchedInput(arrivals=[(2, 4, 4)]))
+    with pytest.raises(AlofaError) as e:
+        s.step(SchedInput())
+    assert e.value.name == "capacity"
+
+
+def test_cancel_blocks_arrival_in_the_same_tick_and_refusals_are_named():
+    s = Scheduler(SchedConfig())
+    a = s.step(SchedInput(arrivals=[(7, 5, 2)], cancelled=[7]))
+    assert a.prefill == [] and s.n_live() == 0
+    for bad in [(1, 0, 1), (1, 3, 0)]:
+        with pytest.raises(AlofaError) as e:
+            s.step(SchedInput(arrivals=[bad]))
+        assert e.value.name == "invalid_argument"
+    s.step(SchedInput(arrivals=[(1, 3, 1)]))
+    with pytest.raises(AlofaError) as e:
+        s.step(SchedInput(arrivals=[(1, 3, 1)]))
+    assert e.value.name == "invalid_argument"
+    with pytest.raises(AlofaError):
+        s.step(SchedInput(freed_blocks=1))
+    assert blocks_for(0, 16) == 0 and blocks_for(16, 16) == 1 and blocks_for(17, 16) == 2
+
+
+def test_trace_lines_round_trip():
+    inp = SchedInput(arrivals=[(1, 300, 8), (2, 64, 4)], cancelled=[3], freed_blocks=2)
+    assert parse_input(input_line(inp)) == inp
+    act = Action(prefill=[(1, 0, 16)], decode=[4], tick_seq=7, preempt_total=2, state_digest=99)
+    assert action_line(act) == "OUT=t=7 P=1:0:16 D=4 X=- F=- C=2 K=99"
+    with pytest.raises(AlofaError):
+        parse_input("A=-|C=-")
