@@ -1,0 +1,267 @@
+"""Each kernel alone against the plain implementation's function of the same
+operation, at sizes other than the engine's tiny models: widths and
+vocabularies that are no power of two, odd group sizes, head sizes in steps
+of 16, pages of several sizes."""
+import numpy as np
+import pytest
+import torch
+
+from plain import model as pm
+from plain import sampler as ps
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def ops():
+    from alofa_amd import ops as o
+    return o
+
+
+def t(a, dtype=torch.float32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV).to(dtype)
+
+
+def bf(a):
+    """Round a float32 array to bfloat16 and back: what the bfloat16 kernels are given."""
+    return torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).float().numpy()
+
+
+def close(got, ref, rel, what=""):
+    got = got.detach().float().cpu().numpy() if isinstance(got, torch.Tensor) else got
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64)).max()
+    b = rel * max(1.0, float(np.abs(ref).max()))
+    assert np.isfinite(got).all() and err <= b, f"{what}: {err:.3e} > {b:.3e}"
+
+
+EXACT, BF16 = 1e-6, 1e-2     # exact kernels round where the plain code rounds; bfloat16 outputs carry 8 bits
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_gather(dtype):
+    rng = np.random.default_rng(0)
+    table = bf(rng.standard_normal((331, 72)).astype(np.float32))
+    ids = rng.integers(0, 331, 19)
+    out = torch.empty(19, 72, device=DEV)
+    ops().embed_gather(out, t(table, dtype), t(ids.astype(np.int32), torch.int32))
+    assert np.array_equal(out.cpu().numpy(), pm.embed(table, ids))
+
+
+@pytest.mark.parametrize("width", [80, 896, 1000])
+def test_rmsnorm(width):
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal((9, width)) * 3).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(width)).astype(np.float32)
+    out = torch.empty(9, width, device=DEV)
+    ops().rmsnorm(out, t(x), t(w), 1e-5, True)
+    close(out, pm.rmsnorm(x, w, 1e-5), EXACT, "exact")
+    outb = torch.empty(9, width, device=DEV, dtype=torch.bfloat16)
+    ops().rmsnorm(outb, t(x), t(w), 1e-5, False)
+    close(outb, pm.rmsnorm(x, w, 1e-5), BF16, "bf16")
+    rows = np.array([8, 0, 3, 3], dtype=np.int32)                       # with the row gather
+    outg = torch.empty(4, width, device=DEV)
+    ops().rmsnorm(outg, t(x), t(w), 1e-5, True, t(rows, torch.int32))
+    close(outg, pm.rmsnorm(x[rows], w, 1e-5), EXACT, "gather")
+
+
+SHAPES = [(1, 100, 72), (5, 130, 200), (70, 33, 264), (130, 257, 48), (3, 64, 1000)]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_gemm_exact(M, N, K):
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    w = rng.standard_normal((N, K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    out = torch.empty(M, N, device=DEV)
+    ops().gemm(out, t(a), t(w), t(b), exact=True)
+    close(out, pm.linear(a, w, b), EXACT, "bias")
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    acc = t(res)
+    ops().gemm(acc, t(a), t(w), add_to_out=True, exact=True)
+    close(acc, pm.add(res, pm.linear(a, w)), EXACT, "residual")
+    # a row's result does not depend on what else is in the batch
+    one = torch.empty(1, N, device=DEV)
+    ops().gemm(one, t(a[M - 1:]), t(w), t(b), exact=True)
+    assert torch.equal(one[0], out[M - 1])
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_gemm_bf16(M, N, K):
+    rng = np.random.default_rng(3)
+    a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
+    b = rng.standard_normal(N).astype(np.float32)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm(out, t(a, torch.bfloat16), t(w, torch.bfloat16), t(b))
+    close(out, pm.linear(a, w, b), BF16, "bf16 out")
+    outf = torch.empty(M, N, device=DEV)
+    ops().gemm(outf, t(a, torch.bfloat16), t(w, torch.bfloat16))
+    close(outf, pm.linear(a, w), 1e-4, "f32 out")
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    acc = t(res)
+    ops().gemm(acc, t(a, torch.bfloat16), t(w, torch.bfloat16), add_to_out=True)
+    close(acc, pm.add(res, pm.linear(a, w)), 1e-4, "residual")
+    # a weight stored in float32 stays float32 and is multiplied as such
+    outw = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    w32 = rng.standard_normal((N, K)).astype(np.float32) * 0.1
+    ops().gemm(outw, t(a, torch.bfloat16), t(w32), t(b))
+    close(outw, pm.linear(a, w32, b), BF16, "f32 weight")
+
+
+def test_gemm_takes_a_strided_view():
+    rng = np.random.default_rng(4)
+    big = rng.standard_normal((6, 300)).astype(np.float32)
+    w = rng.standard_normal((20, 100)).astype(np.float32)
+    out = torch.empty(6, 20, device=DEV)
+    ops().gemm(out, t(big)[:, 100:200], t(w), exact=True)
+    close(out, pm.linear(big[:, 100:200], w), EXACT)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 176, 64), (37, 200, 240), (130, 97, 80)])
+def test_gemm_swiglu(M, N, K):
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    wg, wu = rng.standard_normal((N, K)).astype(np.float32), rng.standard_normal((N, K)).astype(np.float32)
+    out = torch.empty(M, N, device=DEV)
+    ops().gemm_swiglu(out, t(a), t(wg), t(wu), exact=True)
+    close(out, pm.swiglu(pm.linear(a, wg), pm.linear(a, wu)), EXACT, "exact")
+    ab, gb, ub = bf(a), bf(wg * 0.2), bf(wu * 0.2)
+    outb = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm_swiglu(outb, t(ab, torch.bfloat16), t(gb, torch.bfloat16), t(ub, torch.bfloat16))
+    close(outb, pm.swiglu(pm.linear(ab, gb), pm.linear(ab, ub)), BF16, "bf16")
+    g, u = rng.standard_normal((M, N)).astype(np.float32) * 8, rng.standard_normal((M, N)).astype(np.float32)
+    g[0, 0] = -1e4                                                     # far negative gate: 0, not NaN
+    sep = torch.empty(M, N, device=DEV)
+    ops().swiglu(sep, t(g), t(u), exact=True)
+    close(sep, pm.swiglu(g, u), EXACT, "unfused")
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (3, 1, 32, 16), (4, 4, 128, 32)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_and_cache_write(heads, kv_heads, d, bs, dtype):
+    rng = np.random.default_rng(6)
+    T, n_blocks = 11, 7
+    qkv = bf(rng.standard_normal((T, (heads + 2 * kv_heads) * d)).astype(np.float32))
+    pos = rng.integers(0, 200, T)
+    cos, sin = pm.rope_table(200, d, 1e4)
+    slots = rng.permutation(n_blocks * bs)[:T]
+    dev = t(qkv, dtype)
+    kc = torch.full((n_blocks, kv_heads, bs, d), 7.0, device=DEV, dtype=dtype)
+    vc = torch.full((n_blocks, kv_heads, bs, d), 7.0, device=DEV, dtype=dtype)
+    ops().rope_kv_write(dev, t(cos[:, :d // 2]), t(sin[:, :d // 2]), t(pos.astype(np.int32), torch.int32), heads, kv_heads, d,
+                        t(slots.astype(np.int64), torch.int64), kc, vc)
+    rel = EXACT if dtype is torch.float32 else BF16
+    q_ref = pm.rope_apply(qkv[:, :heads * d], cos, sin, pos, d)
+    k_ref = pm.rope_apply(qkv[:, heads * d:(heads + kv_heads) * d], cos, sin, pos, d)
+    close(dev[:, :heads * d], q_ref, rel, "q in place")
+    kc_h, vc_h = kc.float().cpu().numpy(), vc.float().cpu().numpy()
+    written = np.zeros((n_blocks, bs), bool)
+    for i, s in enumerate(slots):
+        written[s // bs, s % bs] = True
+        close(kc_h[s // bs, :, s % bs].reshape(-1), k_ref[i], rel, "k slot")
+        assert np.array_equal(vc_h[s // bs, :, s % bs].reshape(-1), qkv[i, (heads + kv_heads) * d:])   # v is copied, not rotated
+    assert (kc_h.transpose(0, 2, 1, 3)[~written] == 7.0).all() and (vc_h.transpose(0, 2, 1, 3)[~written] == 7.0).all()                               # other slots untouched
+
+
+def paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, dtype, scale_key=None):
+    """Builds requests with their keys and values scattered over pages in a
+    shuffled (not ascending) order, pages not in any table filled with NaN."""
+    n_req = len(lens)
+    blocks_per = [(L + bs - 1) // bs for L in lens]
+    n_blocks = sum(blocks_per) + 3
+    order = rng.permutation(n_blocks)
+    kc = np.full((n_blocks, kv_heads, bs, d), np.nan, np.float32)
+    vc = np.full((n_blocks, kv_heads, bs, d), np.nan, np.float32)
+    table = np.full((n_req, max(blocks_per)), -1, np.int32)
+    ks, vs, qs, pos, req = [], [], [], [], []
+    used = 0
+    for r, L in enumerate(lens):
+        k = bf(rng.standard_normal((L, kv_heads * d)).astype(np.float32))
+        v = bf(rng.standard_normal((L, kv_heads * d)).astype(np.float32))
+        q = bf(rng.standard_normal((q_lens[r], heads * d)).astype(np.float32))
+        if scale_key is not None:                  # one far key stands out for the last query of every head
+            j = scale_key
+            for h in range(heads):
+                hk = h // (heads // kv_heads)
+                q[-1, h * d:(h + 1) * d] = bf(6.0 * k[j, hk * d:(hk + 1) * d])
+        table[r, :blocks_per[r]] = order[used:used + blocks_per[r]]
+        used += blocks_per[r]
+        for p in range(L):
+            b = table[r, p // bs]
+            kc[b, :, p % bs] = k[p].reshape(kv_heads, d)
+            vc[b, :, p % bs] = v[p].reshape(kv_heads, d)
+        ks.append(k), vs.append(v), qs.append(q)
+        pos.extend(range(L - q_lens[r], L))
+        req.extend([r] * q_lens[r])
+    return dict(k=ks, v=vs, q=qs, kc=t(kc, dtype), vc=t(vc, dtype), table=t(table, torch.int32),
+                pos=t(np.array(pos, np.int32), torch.int32), req=t(np.array(req, np.int32), torch.int32),
+                qcat=t(np.concatenate(qs), dtype))
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 80, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16)])
+@pytest.mark.parametrize("dtype,exact", [(torch.float32, True), (torch.bfloat16, False)])
+@pytest.mark.parametrize("window", [None, 21])
+def test_paged_attention(heads, kv_heads, d, bs, dtype, exact, window):
+    rng = np.random.default_rng(7)
+    lens, q_lens = [37, 1, 130, 64], [37, 1, 5, 1]      # a whole prompt, a first token, a portion, a decode at a page's edge
+    c = paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, dtype)
+    out = torch.empty(sum(q_lens), heads * d, device=DEV, dtype=dtype)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    ops().paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, exact)
+    ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(4)])
+    close(out, ref, 2e-6 if exact else BF16, "paged attention")
+
+
+@pytest.mark.parametrize("dtype,exact", [(torch.float32, True), (torch.bfloat16, False)])
+def test_attention_far_key_and_window_edge(dtype, exact):
+    """One far key among hundreds carries the weight: dropping it, or any page of
+    the table, shows. With a window the same key is cut off exactly at the edge."""
+    rng = np.random.default_rng(8)
+    heads, kv_heads, d, bs, L, far = 6, 2, 64, 16, 700, 3
+    c = paged_case(rng, [L], [1], heads, kv_heads, d, bs, dtype, scale_key=far)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    out = torch.empty(1, heads * d, device=DEV, dtype=dtype)
+    ops().paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, None, scale, exact)
+    ref = pm.attention(c["q"][0], c["k"][0], c["v"][0], heads, kv_heads, d)
+    close(out, ref, 2e-6 if exact else BF16, "far key")
+    v_far = np.concatenate([c["v"][0][far, (h // 3) * d:(h // 3 + 1) * d] for h in range(heads)])
+    assert np.abs(ref[0] - v_far).max() < 1e-3                          # the far key really decides the output
+    for window, sees in ((L - far, True), (L - far - 1, False)):         # the window's edge, to the key
+        ops().paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, exact)
+        refw = pm.attention(c["q"][0], c["k"][0], c["v"][0], heads, kv_heads, d, window)
+        close(out, refw, 2e-6 if exact else BF16, f"window {window}")
+        assert (np.abs(refw[0] - v_far).max() < 1e-3) == sees
+
+
+def test_argmax_and_sample():
+    rng = np.random.default_rng(9)
+    vocab = 1537
+    logits = rng.standard_normal((5, vocab)).astype(np.float32)
+    logits[1, [40, 900, 7]] = 9.0          # ties: the lowest index wins
+    logits[2, :] = -3.0                    # all equal
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    ops().argmax(out, t(logits))
+    assert out.tolist() == [pm.argmax(r) for r in logits] and out[1].item() == 7 and out[2].item() == 0
+    rows = np.repeat(logits[:1], 64, axis=0)
+    temps = np.full(64, 0.8)
+    us = np.array([ps.SplitMix64(3).next_uniform() for _ in range(1)] + list(rng.random(61)) + [0.0, 0.9999999999999999])
+    picks = torch.empty(64, dtype=torch.int32, device=DEV)
+    ops().sample(picks, t(rows), t(temps, torch.float64), t(us, torch.float64))
+    _, p = ps.distribution(logits[0], temperature=0.8)
+    assert picks.tolist() == [ps.pick_from(p, u) for u in us]
+    # a low temperature converges to the greedy choice
+    ops().sample(picks, t(rows), t(np.full(64, 1e-4), torch.float64), t(np.clip(us, 0.01, 0.99), torch.float64))
+    assert set(picks.tolist()) == {int(np.argmax(logits[0]))}
+
+
+def test_kernels_refuse_what_they_cannot_take():
+    from alofa_amd.errors import AlofaError
+    o = ops()
+    with pytest.raises(AlofaError):
+        o.gemm(torch.empty(2, 3, device=DEV), torch.empty(2, 4, device=DEV), torch.empty(3, 5, device=DEV))
+    with pytest.raises(AlofaError):
+        o.gemm(torch.empty(2, 3), torch.empty(2, 4), torch.empty(3, 4))                  # not on the GPU
+    with pytest.raises(AlofaError):
+        o.rmsnorm(torch.empty(2, 8, device=DEV, dtype=torch.bfloat16), torch.empty(2, 8, device=DEV), torch.empty(8, device=DEV), 1e-6, True)
+    with pytest.raises(AlofaError):
+        o.argmax(torch.empty(2, dtype=torch.int32, device=DEV), torch.empty(3, 8, device=DEV))
