@@ -1,0 +1,234 @@
+// Paged grouped-query attention for few query tokens per request (decode steps
+// and short portions), bfloat16. The work is reading every visible key and value
+// once, so all query heads of one key head are served together.
+//
+// One wavefront handles (token, key head, split): a contiguous share of the
+// token's visible keys lo..p. d / 16 lanes share a key (16 channels each), so a
+// wave takes 64 / (d / 16) keys per round with fully used 32-byte loads. Every
+// lane group keeps a running softmax of its own (maximum, sum of weights,
+// weighted sum of its 16 value channels, per head, all float); dot products use
+// the packed bfloat16 dot instruction with float accumulation. At the end the
+// groups' states meet in LDS and are combined in group order; with several
+// splits the per-split states go to a scratch buffer and a second kernel
+// combines them in split order. The order of additions depends only on the
+// key range and the split count, never on timing.
+// Cache layout: [block, kv_head, slot_in_block, d].
+#include "common.h"
+
+#include <float.h>
+
+namespace alofa {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kMaxSplits = 64;
+
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+}
+
+// GC: query heads handled at once (the group is walked in chunks of GC).
+template <int GC>
+__global__ void __launch_bounds__(64) attention_decode_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ partial, const bf16_t* __restrict__ q,
+    int64_t q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
+    const int32_t* __restrict__ positions, int heads, int kv_heads, int d, int block_size, int window, float scale,
+    int n_splits) {
+  extern __shared__ float lds[];  // [GC][kpi][d] weighted sums, then [GC][kpi] maxima, [GC][kpi] sums
+  const int t = blockIdx.x, hk = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+  const int group = heads / kv_heads;
+  const int lpk = d / 16;          // lanes per key
+  const int kpi = 64 / lpk;        // keys per round
+  const int slot = lane / lpk, part = lane % lpk;
+  const bool active = slot < kpi;
+  const int p = positions[t];
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int n_keys = p - lo + 1;
+  const int per_split = (n_keys + n_splits - 1) / n_splits;
+  const int begin = lo + split * per_split;
+  const int end = (begin + per_split < p + 1) ? begin + per_split : p + 1;
+  const int32_t* table = block_table + static_cast<int64_t>(req_of_token[t]) * max_blocks;
+  const int64_t head_stride = static_cast<int64_t>(block_size) * d;
+
+  for (int h0 = 0; h0 < group; h0 += GC) {
+    uint32_t qp[GC][8];
+#pragma unroll
+    for (int i = 0; i < GC; ++i) {
+      const int h = hk * group + ((h0 + i < group) ? h0 + i : h0);
+      const uint4* src = reinterpret_cast<const uint4*>(q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(h) * d + part * 16);
+      uint4 a = make_uint4(0, 0, 0, 0), b = a;
+      if (active) { a = src[0]; b = src[1]; }
+      qp[i][0] = a.x; qp[i][1] = a.y; qp[i][2] = a.z; qp[i][3] = a.w;
+      qp[i][4] = b.x; qp[i][5] = b.y; qp[i][6] = b.z; qp[i][7] = b.w;
+    }
+    float m[GC], l[GC], o[GC][16];
+#pragma unroll
+    for (int i = 0; i < GC; ++i) {
+      m[i] = -FLT_MAX;
+      l[i] = 0.f;
+#pragma unroll
+      for (int c = 0; c < 16; ++c) o[i][c] = 0.f;
+    }
+
+    auto fetch = [&](int j, uint4& k0, uint4& k1, uint4& v0, uint4& v1) {
+      if (active && j < end) {
+        const int64_t blk = table[j / block_size];
+        const int64_t base = (blk * kv_heads + hk) * head_stride + static_cast<int64_t>(j % block_size) * d + part * 16;
+        const uint4* kp = reinterpret_cast<const uint4*>(k_cache + base);
+        const uint4* vp = reinterpret_cast<const uint4*>(v_cache + base);
+        k0 = kp[0]; k1 = kp[1]; v0 = vp[0]; v1 = vp[1];
+      }
+    };
+
+    uint4 k0, k1, v0, v1, nk0, nk1, nv0, nv1;
+    k0 = k1 = v0 = v1 = nk0 = nk1 = nv0 = nv1 = make_uint4(0, 0, 0, 0);
+    fetch(begin + slot, k0, k1, v0, v1);
+    for (int j0 = begin; j0 < end; j0 += kpi) {
+      const int j = j0 + slot;
+      fetch(j + kpi, nk0, nk1, nv0, nv1);
+      const uint32_t kw[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+      const uint32_t vw[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+      float s[GC];
+#pragma unroll
+      for (int i = 0; i < GC; ++i) {
+        float acc = 0.f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc = dot2(qp[i][c], kw[c], acc);
+        s[i] = acc;
+      }
+      // add up the lanes that share the key
+      if ((lpk & (lpk - 1)) == 0) {
+        for (int off = 1; off < lpk; off <<= 1)
+#pragma unroll
+          for (int i = 0; i < GC; ++i) s[i] += __shfl_xor(s[i], off, 64);
+      } else {
+#pragma unroll
+        for (int i = 0; i < GC; ++i) {
+          float total = 0.f;
+          for (int x = 0; x < lpk; ++x) total += __shfl(s[i], slot * lpk + x, 64);
+          s[i] = total;
+        }
+      }
+      if (active && j < end) {
+        float vf[16];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          vf[2 * c] = __uint_as_float(vw[c] << 16);
+          vf[2 * c + 1] = __uint_as_float(vw[c] & 0xffff0000u);
+        }
+#pragma unroll
+        for (int i = 0; i < GC; ++i) {
+          const float sc = s[i] * scale;
+          if (sc > m[i]) {  // a new maximum: bring what was gathered so far to its scale
+            const float corr = __expf(m[i] - sc);
+            l[i] *= corr;
+#pragma unroll
+            for (int c = 0; c < 16; ++c) o[i][c] *= corr;
+            m[i] = sc;
+          }
+          const float w = __expf(sc - m[i]);
+          l[i] += w;
+#pragma unroll
+          for (int c = 0; c < 16; ++c) o[i][c] += w * vf[c];
+        }
+      }
+      k0 = nk0; k1 = nk1; v0 = nv0; v1 = nv1;
+    }
+
+    // the lane groups' states meet in LDS and are combined in group order
+    float* lds_o = lds;
+    float* lds_m = lds + GC * kpi * d;
+    float* lds_l = lds_m + GC * kpi;
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < GC; ++i) {
+#pragma unroll
+        for (int c = 0; c < 16; ++c) lds_o[(i * kpi + slot) * d + part * 16 + c] = o[i][c];
+        if (part == 0) { lds_m[i * kpi + slot] = m[i]; lds_l[i * kpi + slot] = l[i]; }
+      }
+    }
+    __syncthreads();
+    for (int i = 0; i < GC && h0 + i < group; ++i) {
+      const int h = hk * group + h0 + i;
+      float big = -FLT_MAX;
+      for (int s2 = 0; s2 < kpi; ++s2) big = fmaxf(big, lds_m[i * kpi + s2]);
+      float total = 0.f;
+      for (int s2 = 0; s2 < kpi; ++s2) total += lds_l[i * kpi + s2] * __expf(lds_m[i * kpi + s2] - big);
+      for (int c = lane; c < d; c += 64) {
+        float acc = 0.f;
+        for (int s2 = 0; s2 < kpi; ++s2) acc += lds_o[(i * kpi + s2) * d + c] * __expf(lds_m[i * kpi + s2] - big);
+        if (n_splits == 1) {
+          store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
+        } else {
+          float* dst = partial + ((static_cast<int64_t>(t) * heads + h) * n_splits + split) * (d + 2);
+          dst[2 + c] = acc;
+          if (c == 0) { dst[0] = big; dst[1] = total; }
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Combines the splits' states of one (token, head) in split order.
+__global__ void __launch_bounds__(64) attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
+                                                             const float* __restrict__ partial, int heads, int d,
+                                                             int n_splits) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* src = partial + (static_cast<int64_t>(t) * heads + h) * n_splits * (d + 2);
+  float big = -FLT_MAX;
+  for (int s = 0; s < n_splits; ++s) big = fmaxf(big, src[s * (d + 2)]);
+  float total = 0.f;
+  for (int s = 0; s < n_splits; ++s) total += src[s * (d + 2) + 1] * __expf(src[s * (d + 2)] - big);
+  for (int c = threadIdx.x; c < d; c += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < n_splits; ++s) acc += src[s * (d + 2) + 2 + c] * __expf(src[s * (d + 2)] - big);
+    store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
+  }
+}
+
+}  // namespace alofa
+
+using namespace alofa;
+
+// Floats of scratch that n_splits > 1 needs.
+extern "C" int64_t alofa_attention_decode_scratch(int tokens, int heads, int d, int n_splits) {
+  return n_splits > 1 ? static_cast<int64_t>(tokens) * heads * n_splits * (d + 2) : 0;
+}
+
+extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
+                                      const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                      int max_blocks, const int32_t* req_of_token, const int32_t* positions,
+                                      int tokens, int heads, int kv_heads, int d, int block_size, int window,
+                                      float scale, int n_splits, hipStream_t stream) {
+  ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
+                "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
+  ALOFA_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention_decode: head size %d must be 16..256 in steps of 16", d);
+  ALOFA_REQUIRE(block_size > 0 && max_blocks > 0 && window >= 0, "attention_decode: block_size=%d max_blocks=%d window=%d", block_size, max_blocks, window);
+  ALOFA_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || partial), "attention_decode: n_splits=%d (1..%d) needs scratch when above 1", n_splits, kMaxSplits);
+  ALOFA_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_decode: q rows must be 16-byte aligned");
+  const int group = heads / kv_heads;
+  const int kpi = 64 / (d / 16);
+  dim3 grid(tokens, kv_heads, n_splits);
+#define ALOFA_DECODE(GC)                                                                                                  \
+  {                                                                                                                       \
+    const size_t lds = static_cast<size_t>(GC) * kpi * (d + 2) * sizeof(float);                                           \
+    attention_decode_kernel<GC><<<grid, 64, lds, stream>>>(                                                               \
+        static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                          \
+        static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, max_blocks, req_of_token,  \
+        positions, heads, kv_heads, d, block_size, window, scale, n_splits);                                              \
+  }
+  if (group == 1) ALOFA_DECODE(1)
+  else if (group == 2) ALOFA_DECODE(2)
+  else if (group <= 4) ALOFA_DECODE(4)
+  else ALOFA_DECODE(8)
+#undef ALOFA_DECODE
+  if (check_launch("attention_decode")) return 1;
+  if (n_splits > 1) {
+    attention_merge_kernel<<<dim3(tokens, heads), 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, heads, d, n_splits);
+    return check_launch("attention_merge");
+  }
+  return 0;
+}

@@ -1,0 +1,194 @@
+// Matrix products for few rows (decode steps and small portions), bfloat16:
+// out[m, n] = sum_k A[m, k] * W[n, k] with M <= 64. The work is streaming W
+// once from memory; the arithmetic rides on MFMA 16x16x32 tiles.
+//
+// A block of kWaves wavefronts owns 16 * NT output columns. The waves split K
+// among themselves in interleaved steps of 32 (so that together they read
+// contiguous runs of every weight row), each accumulates its share for all
+// rows in registers, and the partial sums meet in LDS, added in wave order:
+// the result is the same on every run and for every batch the row is part of
+// (M only selects how many 16-row tiles are computed).
+//
+// Operand layout of v_mfma_f32_16x16x32_bf16, lane l: A holds row l % 16,
+// B holds column l % 16, both the 8 reduction indices 8 * (l / 16) .. + 7 of
+// the step; D holds column l % 16, rows 4 * (l / 16) .. + 3.
+#include "common.h"
+
+namespace alofa {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+enum SkinnyEpilogue : int { kSkStore = 0, kSkResidual = 1, kSkSwiglu = 2 };
+
+constexpr int kUnroll = 4;
+
+__device__ __forceinline__ bf16x8 load_frag(const bf16_t* __restrict__ p, bool ok) {
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (ok) v = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// MT: 16-row tiles of A; NT: 16-column tiles per block (kSkSwiglu: tile 0 is the
+// gate matrix, tile 1 the up matrix, same columns); TO: float or bf16_t.
+template <int MT, int NT, int kWaves, int kEpilogue, typename TO>
+__global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
+    TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
+    const bf16_t* __restrict__ W2, int64_t ldw, const float* __restrict__ bias, int M, int N, int K) {
+  __shared__ f32x4 red[kWaves][MT * NT][64];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int r = lane % 16, g = lane / 16;
+  constexpr int kColsPerBlock = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
+  const int n0 = blockIdx.x * kColsPerBlock;
+
+  const bf16_t* a_row[MT];
+  bool a_ok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + r;
+    a_ok[mt] = m < M;
+    a_row[mt] = A + static_cast<int64_t>(a_ok[mt] ? m : 0) * lda;
+  }
+  const bf16_t* w_row[NT];
+  bool w_ok[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
+    w_ok[nt] = n < N;
+    const bf16_t* base = (kEpilogue == kSkSwiglu && nt == 1) ? W2 : W;
+    w_row[nt] = base + static_cast<int64_t>(w_ok[nt] ? n : 0) * ldw;
+  }
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int n_steps = (K + 31) / 32;  // steps of 32 along K; this wave takes steps wave, wave + kWaves, ...
+  bf16x8 a_cur[kUnroll][MT], w_cur[kUnroll][NT], a_nxt[kUnroll][MT], w_nxt[kUnroll][NT];
+
+  auto load = [&](bf16x8 (&a)[kUnroll][MT], bf16x8 (&w)[kUnroll][NT], int first) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int k = (first + u * kWaves) * 32 + g * 8;
+      const bool k_ok = k < K;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) w[u][nt] = load_frag(w_row[nt] + k, k_ok && w_ok[nt]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) a[u][mt] = load_frag(a_row[mt] + k, k_ok && a_ok[mt]);
+    }
+  };
+
+  load(a_cur, w_cur, wave);
+  for (int s = wave; s < n_steps; s += kUnroll * kWaves) {
+    if (s + kUnroll * kWaves < n_steps) load(a_nxt, w_nxt, s + kUnroll * kWaves);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[u][mt], w_cur[u][nt], acc[mt][nt], 0, 0, 0);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) a_cur[u][mt] = a_nxt[u][mt];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) w_cur[u][nt] = w_nxt[u][nt];
+    }
+  }
+
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) red[wave][mt * NT + nt][lane] = acc[mt][nt];
+  __syncthreads();
+
+  // tiles are shared out among the waves; each adds the partial sums in wave order
+  constexpr int kOutTiles = (kEpilogue == kSkSwiglu) ? MT : MT * NT;
+  for (int tile = wave; tile < kOutTiles; tile += kWaves) {
+    const int mt = (kEpilogue == kSkSwiglu) ? tile : tile / NT;
+    const int nt = (kEpilogue == kSkSwiglu) ? 0 : tile % NT;
+    f32x4 sum = red[0][mt * NT + nt][lane];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) sum += red[w][mt * NT + nt][lane];
+    f32x4 up = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (kEpilogue == kSkSwiglu) {
+      up = red[0][mt * NT + 1][lane];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) up += red[w][mt * NT + 1][lane];
+    }
+    const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
+    if (n >= N) continue;
+    const float b = (bias && kEpilogue == kSkStore) ? bias[n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = mt * 16 + g * 4 + i;
+      if (m >= M) continue;
+      TO* dst = out + static_cast<int64_t>(m) * ldo + n;
+      if (kEpilogue == kSkStore) {
+        store_f32(dst, sum[i] + b);
+      } else if (kEpilogue == kSkResidual) {
+        store_f32(dst, load_f32(dst) + sum[i]);
+      } else {
+        const float gv = sum[i];
+        store_f32(dst, gv / (1.f + __expf(-gv)) * up[i]);
+      }
+    }
+  }
+}
+
+template <int MT, int NT, int kWaves, int kEpilogue, typename TO>
+static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
+                         const float* bias, int M, int N, int K, hipStream_t stream) {
+  constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
+  gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO><<<(N + cols - 1) / cols, kWaves * 64, 0, stream>>>(
+      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
+      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K);
+  return check_launch("gemm_skinny");
+}
+
+template <int kEpilogue, typename TO>
+static int dispatch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
+                           const float* bias, int M, int N, int K, hipStream_t stream) {
+  // few columns: one 16-column tile per block and eight waves along K keep more of the chip busy
+  const bool narrow = (kEpilogue != kSkSwiglu) && N <= 4096;
+#define ALOFA_SKINNY(MT)                                                                                              \
+  if (kEpilogue == kSkSwiglu)                                                                                         \
+    return launch_skinny<MT, 2, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);               \
+  if (narrow) return launch_skinny<MT, 1, 8, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);     \
+  return launch_skinny<MT, 2, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+  if (M <= 16) { ALOFA_SKINNY(1) }
+  if (M <= 32) { ALOFA_SKINNY(2) }
+  ALOFA_SKINNY(4)
+#undef ALOFA_SKINNY
+}
+
+}  // namespace alofa
+
+using namespace alofa;
+
+// bfloat16 A [M, K] (M <= 64) and W [N, K] (W2 for the swiglu epilogue); K a multiple of 8,
+// rows 16-byte aligned. Epilogues: 0 store (+ bias) as o_dtype, 1 add to the float residual, 2 swiglu.
+extern "C" int alofa_gemm_skinny(void* out, int o_dtype, int64_t ldo, const void* A, int64_t lda, const void* W,
+                                 const void* W2, int64_t ldw, const float* bias, int M, int N, int K, int epilogue,
+                                 hipStream_t stream) {
+  ALOFA_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: M=%d (1..64) N=%d K=%d", M, N, K);
+  ALOFA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K=%d, lda=%lld, ldw=%lld must be multiples of 8", K,
+                static_cast<long long>(lda), static_cast<long long>(ldw));
+  ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(W2) % 16 == 0, "gemm_skinny: operands must be 16-byte aligned");
+  ALOFA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_skinny: a leading dimension is shorter than its row");
+  if (epilogue == kSkStore && o_dtype == kBF16)
+    return dispatch_skinny<kSkStore, bf16_t>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream);
+  if (epilogue == kSkStore && o_dtype == kF32)
+    return dispatch_skinny<kSkStore, float>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream);
+  if (epilogue == kSkResidual && o_dtype == kF32)
+    return dispatch_skinny<kSkResidual, float>(out, ldo, A, lda, W, nullptr, ldw, nullptr, M, N, K, stream);
+  if (epilogue == kSkSwiglu && o_dtype == kBF16) {
+    ALOFA_REQUIRE(W2 != nullptr, "gemm_skinny: the swiglu epilogue needs the up matrix");
+    return dispatch_skinny<kSkSwiglu, bf16_t>(out, ldo, A, lda, W, W2, ldw, nullptr, M, N, K, stream);
+  }
+  ALOFA_REQUIRE(false, "gemm_skinny: unsupported epilogue %d with out dtype %d", epilogue, o_dtype);
+}

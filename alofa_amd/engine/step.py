@@ -54,6 +54,8 @@ class StepContext:
         self.spans = spans
         self.positions_host = positions_host
         self.tokens = int(positions_host.shape[0])
+        self.max_q_len = max(s.n for s in spans)            # most rows of one request
+        self.max_context = max(s.pos0 + s.n for s in spans)  # longest context after this step
         self.n_positions = fn.n_positions
         self.positions: torch.Tensor = None
         self.req_of_token: torch.Tensor = None

@@ -103,6 +103,20 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, eps: float, exa
 
 # ------------------------------------------------------------ matrix product
 
+SKINNY_MAX_ROWS = 64
+SWIGLU = 2
+
+
+def _mfma_operands(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the bfloat16 MFMA kernels can take these operands: 16-byte loads
+    along K need K and the leading dimensions in multiples of 8 and aligned bases."""
+    if a.dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16:
+        return False
+    K = a.shape[1]
+    return (K % 8 == 0 and _rows("a", a) % 8 == 0 and _rows("w", w) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
          add_to_out: bool = False, exact: bool = False) -> None:
     """out = a @ w.T (+ bias), or out += a @ w.T when ``add_to_out`` (out is then
@@ -118,6 +132,10 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
             raise AlofaError("shape_mismatch", "bias length does not fit", f"bias={tuple(bias.shape)} N={N}")
     if add_to_out and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the residual stream is float32", f"out={out.dtype}")
+    if not exact and _mfma_operands(a, w) and M <= SKINNY_MAX_ROWS:
+        _call("alofa_gemm_skinny", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None),
+              _L(_rows("w", w)), _ptr(None if add_to_out else bias), _I(M), _I(N), _I(K), _I(ADD_TO_RESIDUAL if add_to_out else STORE), _stream())
+        return
     _call("alofa_gemm_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
           _ptr(w), _I(dtype_code(w)), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
           _I(ADD_TO_RESIDUAL if add_to_out else STORE), _I(int(exact)), _stream())
@@ -132,6 +150,10 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: 
         raise AlofaError("shape_mismatch", "gate/up product shapes do not fit", f"a={tuple(a.shape)} gate={tuple(w_gate.shape)} up={tuple(w_up.shape)} out={tuple(out.shape)}")
     if w_gate.dtype is not w_up.dtype or _rows("w_gate", w_gate) != _rows("w_up", w_up):
         raise AlofaError("invalid_argument", "gate and up matrices must share dtype and layout")
+    if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up) and M <= SKINNY_MAX_ROWS:
+        _call("alofa_gemm_skinny", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
+              _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), _stream())
+        return
     _call("alofa_gemm_swiglu_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
           _ptr(w_gate), _ptr(w_up), _I(dtype_code(w_gate)), _L(_rows("w_gate", w_gate)), _I(M), _I(N), _I(K), _I(int(exact)), _stream())
 
@@ -189,11 +211,35 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
 
 # ----------------------------------------------------------------- attention
 
+DECODE_MAX_Q = 4          # requests with at most this many query tokens use the decode kernel
+_decode_scratch: dict = {}
+
+
+def _scratch(device, floats: int) -> torch.Tensor:
+    buf = _decode_scratch.get(device)
+    if buf is None or buf.numel() < floats:
+        buf = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=device)
+        _decode_scratch[device] = buf
+    return buf
+
+
+def decode_splits(tokens: int, kv_heads: int, d: int, max_context: int) -> int:
+    """Shares of the keys per (token, key head): enough waves to fill the chip,
+    but at least four rounds of keys each."""
+    keys_per_round = 64 // (d // 16)
+    by_chip = -(-1024 // max(1, tokens * kv_heads))
+    by_length = max(1, max_context // (4 * keys_per_round))
+    return max(1, min(64, by_chip, by_length))
+
+
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, req_of_token: torch.Tensor, positions: torch.Tensor,
-                    heads: int, kv_heads: int, d: int, window: Optional[int], scale: float, exact: bool) -> None:
+                    heads: int, kv_heads: int, d: int, window: Optional[int], scale: float, exact: bool,
+                    max_q_len: Optional[int] = None, max_context: Optional[int] = None) -> None:
     """out[t] = attention of query token t (q [T, >= heads*d] rows, heads packed)
-    over the keys lo..positions[t] of its request's pages."""
+    over the keys lo..positions[t] of its request's pages. ``max_q_len`` (most
+    query tokens of one request in this step) and ``max_context`` (longest
+    context) only choose the kernel and its launch shape."""
     _gpu("out", out, None, 2), _gpu("q", q, None, 2)
     T = q.shape[0]
     if out.shape[0] != T or out.shape[1] < heads * d or q.shape[1] < heads * d or out.dtype is not q.dtype:
@@ -209,6 +255,15 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
     if req_of_token.shape[0] != T or positions.shape[0] != T:
         raise AlofaError("shape_mismatch", "one request index and one position per token")
+    if (not exact and q.dtype is torch.bfloat16 and max_q_len is not None and max_q_len <= DECODE_MAX_Q and d % 16 == 0
+            and _rows("q", q) % 8 == 0 and q.data_ptr() % 16 == 0):
+        n_splits = decode_splits(T, kv_heads, d, min(max_context or 1 << 30, window or 1 << 30))
+        floats = T * heads * n_splits * (d + 2) if n_splits > 1 else 0
+        partial = _scratch(q.device, floats) if floats else None
+        _call("alofa_attention_decode", _ptr(out), _L(_rows("out", out)), _ptr(partial), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
+              _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T), _I(heads), _I(kv_heads), _I(d),
+              _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits), _stream())
+        return
     _call("alofa_attention_simple", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
           _I(dtype_code(q)), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T),
           _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(int(exact)), _stream())

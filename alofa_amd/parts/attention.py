@@ -84,7 +84,8 @@ class GQAAttention(Mixer):
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
         attn = ctx.scratch("attn", (T, self.heads * self.d), self.rt.dtype)
         ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions,
-                            self.heads, self.kv_heads, self.d, self.window, self.scale, exact)
+                            self.heads, self.kv_heads, self.d, self.window, self.scale, exact,
+                            max_q_len=ctx.max_q_len, max_context=ctx.max_context)
         if self.b_o is not None:
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
             ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)

@@ -212,6 +212,30 @@ def test_paged_attention(heads, kv_heads, d, bs, dtype, exact, window):
     close(out, ref, 2e-6 if exact else BF16, "paged attention")
 
 
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 80, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (18, 2, 32, 64)])
+@pytest.mark.parametrize("window", [None, 21, 300])
+def test_decode_attention(heads, kv_heads, d, bs, window):
+    """The kernel for few query tokens per request: single tokens and short
+    portions, contexts from one key to many pages (several splits), groups of
+    1 to 9 heads per key head, head sizes whose lanes-per-key is no power of two."""
+    rng = np.random.default_rng(17)
+    lens, q_lens = [1, 37, 700, 64, 333], [1, 2, 1, 4, 3]
+    c = paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16)
+    out = torch.empty(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    o = ops()
+    o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, False,
+                      max_q_len=4, max_context=700)
+    ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(5)])
+    close(out, ref, BF16, "decode attention")
+    if (heads, d, window) == (14, 64, None):
+        assert o.decode_splits(sum(q_lens), kv_heads, d, 700) == 10                       # several splits are really in play
+    one = torch.empty(1, heads * d, device=DEV, dtype=torch.bfloat16)        # one split, one token
+    o.paged_attention(one, c["qcat"][:1], c["kc"], c["vc"], c["table"], c["req"][:1], c["pos"][:1], heads, kv_heads, d, window, scale, False,
+                      max_q_len=1, max_context=1)
+    close(one, ref[:1], BF16, "decode attention, first token")
+
+
 @pytest.mark.parametrize("dtype,exact", [(torch.float32, True), (torch.bfloat16, False)])
 def test_attention_far_key_and_window_edge(dtype, exact):
     """One far key among hundreds carries the weight: dropping it, or any page of
@@ -227,7 +251,8 @@ def test_attention_far_key_and_window_edge(dtype, exact):
     v_far = np.concatenate([c["v"][0][far, (h // 3) * d:(h // 3 + 1) * d] for h in range(heads)])
     assert np.abs(ref[0] - v_far).max() < 1e-3                          # the far key really decides the output
     for window, sees in ((L - far, True), (L - far - 1, False)):         # the window's edge, to the key
-        ops().paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, exact)
+        ops().paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, exact,
+                              max_q_len=None if exact else 1, max_context=L)
         refw = pm.attention(c["q"][0], c["k"][0], c["v"][0], heads, kv_heads, d, window)
         close(out, refw, 2e-6 if exact else BF16, f"window {window}")
         assert (np.abs(refw[0] - v_far).max() < 1e-3) == sees
