@@ -6,6 +6,7 @@ the order given (src/alofa/engine/executor.mojo:555-609 for the row layout,
 :665-859 for the pass)."""
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass, field
 from typing import Optional
 
@@ -14,6 +15,10 @@ import torch
 
 from ..cache.manager import CacheManager
 from ..errors import AlofaError
+
+
+def _pow2_ceil(n: int) -> int:
+    return max(64, 1 << (int(n) - 1).bit_length())
 
 
 @dataclass
@@ -55,7 +60,9 @@ class StepContext:
         self.positions_host = positions_host
         self.tokens = int(positions_host.shape[0])
         self.max_q_len = max(s.n for s in spans)            # most rows of one request
-        self.max_context = max(s.pos0 + s.n for s in spans)  # longest context after this step
+        # longest context after this step, rounded up to a power of two: it only shapes
+        # launches, and a coarse value lets captured decode graphs be used again
+        self.max_context = _pow2_ceil(max(s.pos0 + s.n for s in spans))
         self.n_positions = fn.n_positions
         self.positions: torch.Tensor = None
         self.req_of_token: torch.Tensor = None
@@ -95,6 +102,13 @@ class StepFunction:
         self.cache_entry = [c if needs[c] is not None else None for c in self.cache_entry]
         self.steps_run = 0
         self.rows_run = 0
+        # decode steps (one token per request) replay a captured HIP graph when every
+        # part runs native kernels only; ALOFA_GRAPHS=0 switches that off
+        self.use_graphs = os.environ.get("ALOFA_GRAPHS", "1") != "0" and all(
+            getattr(b.mixer, "capturable", False) and getattr(b.feed_forward, "capturable", False) for b in model.blocks)
+        self._graphs: dict = {}
+        self._graph_buffers: dict = {}
+        self.graph_replays = 0
         # build position tables up to the context bound once, so they never move afterwards
         for b in model.blocks:
             pos = getattr(b.mixer, "position", None)
@@ -203,10 +217,92 @@ class StepFunction:
         self.steps_run += 1
         self.rows_run += ctx.tokens
 
+    # ---------------------------------------------------------- decode graphs
+    def _decode_buffers(self, B: int) -> dict:
+        """Static device buffers of the decode graphs for batch B, and the pinned
+        host block that is copied over them in one piece before a replay."""
+        if B not in self._graph_buffers:
+            W = max(1, (self.n_positions + self.cache.block_size - 1) // self.cache.block_size)
+            G = len(self.cache.groups)
+            n32 = 3 * B + G * B * W                      # ids, positions, req_of_token, tables
+            n32 += n32 % 2                               # keep the int64 part 8-byte aligned
+            nbytes = 4 * n32 + 8 * G * B                 # + slots
+            host = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+            devb = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+            h32, d32 = host[:4 * n32].view(torch.int32), devb[:4 * n32].view(torch.int32)
+            h64, d64 = host[4 * n32:].view(torch.int64), devb[4 * n32:].view(torch.int64)
+            buf = {"host": host, "dev": devb, "W": W, "scratch": {},
+                   "h_ids": h32[:B].numpy(), "h_pos": h32[B:2 * B].numpy(), "h_req": h32[2 * B:3 * B].numpy(),
+                   "h_tables": h32[3 * B:3 * B + G * B * W].view(G, B, W).numpy(), "h_slots": h64.view(G, B).numpy(),
+                   "ids": d32[:B], "positions": d32[B:2 * B], "req_of_token": d32[2 * B:3 * B],
+                   "tables": d32[3 * B:3 * B + G * B * W].view(G, B, W), "slots": d64.view(G, B),
+                   "rows": torch.arange(B, dtype=torch.int32, device=self.device), "copied": torch.cuda.Event()}
+            buf["h_req"][:] = np.arange(B, dtype=np.int32)
+            self._graph_buffers[B] = buf
+        return self._graph_buffers[B]
+
+    def _run_decode_graph(self, entries: list) -> torch.Tensor:
+        spans = self.plan(entries)
+        cache = self.cache
+        need = [0] * len(cache.groups)
+        for s in spans:
+            for g, n in enumerate(cache.blocks_needed(s.request, s.pos0 + 1)):
+                need[g] += n
+        for g, grp in enumerate(cache.groups):
+            if need[g] > grp.pool.n_free:
+                raise AlofaError("capacity", "kv block pool is exhausted", f"group={g} need={need[g]} free={grp.pool.n_free}")
+        for s in spans:
+            cache.reserve(s.request, s.pos0 + 1)
+        B = len(spans)
+        buf = self._decode_buffers(B)
+        buf["copied"].synchronize()                      # the last copy out of the host block is done
+        buf["h_tables"].fill(-1)
+        for i, (e, s) in enumerate(zip(entries, spans)):
+            buf["h_ids"][i] = e.tokens[0]
+            buf["h_pos"][i] = s.pos0
+            for g in range(len(cache.groups)):
+                t = cache.table(s.request, g)
+                buf["h_tables"][g, i, :len(t)] = t
+                buf["h_slots"][g, i] = cache.slots(s.request, g, s.pos0, 1)[0]
+        positions = buf["h_pos"].copy()
+        ctx = StepContext(self, spans, positions)
+        ctx.positions, ctx.req_of_token = buf["positions"], buf["req_of_token"]
+        ctx._tables = [buf["tables"][g] for g in range(len(cache.groups))]
+        ctx._slots = [buf["slots"][g] for g in range(len(cache.groups))]
+        buf["dev"].copy_(buf["host"], non_blocking=True)
+        buf["copied"].record()
+        key = (B, ctx.max_context)
+        saved, self._scratch = self._scratch, buf["scratch"]   # graphs of one batch size share their own buffers
+        try:
+            if key not in self._graphs:
+                # once eagerly, so that every buffer exists before the capture and the
+                # step's result does not depend on the capture itself
+                hidden = self.model.forward(ctx, buf["ids"])
+                logits = self.model.logits(ctx, hidden, buf["rows"])
+                torch.cuda.current_stream().synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    hidden = self.model.forward(ctx, buf["ids"])
+                    captured = self.model.logits(ctx, hidden, buf["rows"])
+                if captured.data_ptr() != logits.data_ptr():
+                    raise AlofaError("invalid_argument", "a buffer moved between the eager run and the capture")
+                self._graphs[key] = (graph, captured)
+                # the capture itself ran nothing: the eager results stand
+            else:
+                graph, logits = self._graphs[key]
+                graph.replay()
+                self.graph_replays += 1
+        finally:
+            self._scratch = saved
+        self.finish(ctx)
+        return logits
+
     def run(self, entries: list) -> Optional[torch.Tensor]:
         """Run the step. Returns float32 logits [wanted, vocab] on the device in
         the order of the entries and of their ``want`` lists, or None when nothing
         is wanted. The buffer is re-used by the next step."""
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            return self._run_decode_graph(entries)
         ctx, ids, rows = self.begin(entries)
         hidden = self.model.forward(ctx, ids)
         logits = self.model.logits(ctx, hidden, rows) if rows is not None else None

@@ -212,15 +212,6 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
 # ----------------------------------------------------------------- attention
 
 DECODE_MAX_Q = 4          # requests with at most this many query tokens use the decode kernel
-_decode_scratch: dict = {}
-
-
-def _scratch(device, floats: int) -> torch.Tensor:
-    buf = _decode_scratch.get(device)
-    if buf is None or buf.numel() < floats:
-        buf = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=device)
-        _decode_scratch[device] = buf
-    return buf
 
 
 def decode_splits(tokens: int, kv_heads: int, d: int, max_context: int) -> int:
@@ -232,14 +223,22 @@ def decode_splits(tokens: int, kv_heads: int, d: int, max_context: int) -> int:
     return max(1, min(64, by_chip, by_length))
 
 
+def decode_scratch_floats(tokens: int, heads: int, kv_heads: int, d: int, max_context: int, window: Optional[int]) -> int:
+    """Floats of scratch the decode kernel needs for these sizes (0: none)."""
+    n = decode_splits(tokens, kv_heads, d, min(max_context, window or max_context))
+    return tokens * heads * n * (d + 2) if n > 1 else 0
+
+
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, req_of_token: torch.Tensor, positions: torch.Tensor,
                     heads: int, kv_heads: int, d: int, window: Optional[int], scale: float, exact: bool,
-                    max_q_len: Optional[int] = None, max_context: Optional[int] = None) -> None:
+                    max_q_len: Optional[int] = None, max_context: Optional[int] = None,
+                    scratch: Optional[torch.Tensor] = None) -> None:
     """out[t] = attention of query token t (q [T, >= heads*d] rows, heads packed)
     over the keys lo..positions[t] of its request's pages. ``max_q_len`` (most
     query tokens of one request in this step) and ``max_context`` (longest
-    context) only choose the kernel and its launch shape."""
+    context) only choose the kernel and its launch shape; with them the caller
+    passes ``scratch`` (float32, ``decode_scratch_floats`` long) when that is not 0."""
     _gpu("out", out, None, 2), _gpu("q", q, None, 2)
     T = q.shape[0]
     if out.shape[0] != T or out.shape[1] < heads * d or q.shape[1] < heads * d or out.dtype is not q.dtype:
@@ -257,9 +256,14 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         raise AlofaError("shape_mismatch", "one request index and one position per token")
     if (not exact and q.dtype is torch.bfloat16 and max_q_len is not None and max_q_len <= DECODE_MAX_Q and d % 16 == 0
             and _rows("q", q) % 8 == 0 and q.data_ptr() % 16 == 0):
-        n_splits = decode_splits(T, kv_heads, d, min(max_context or 1 << 30, window or 1 << 30))
+        ctx_len = max_context or 1 << 30
+        n_splits = decode_splits(T, kv_heads, d, min(ctx_len, window or ctx_len))
         floats = T * heads * n_splits * (d + 2) if n_splits > 1 else 0
-        partial = _scratch(q.device, floats) if floats else None
+        partial = None
+        if floats:
+            if scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous():
+                raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")
+            partial = scratch
         _call("alofa_attention_decode", _ptr(out), _L(_rows("out", out)), _ptr(partial), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
               _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T), _I(heads), _I(kv_heads), _I(d),
               _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits), _stream())

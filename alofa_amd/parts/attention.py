@@ -23,6 +23,7 @@ from .base import CacheNeed, Mixer, build_part, register_part
 class GQAAttention(Mixer):
     """params: prefix, hidden, heads, kv_heads, head_dim, qkv_bias, out_bias,
     window (None or a count of keys), position (PartSpec)."""
+    capturable = True   # native kernels on the current stream only: a decode step may be graph-captured
 
     @classmethod
     def tensors(cls, spec):
@@ -61,6 +62,7 @@ class GQAAttention(Mixer):
         # float32 1 / sqrt(float32 d), as the reference forms it (scalar.mojo:421)
         self.scale = float(np.float32(1.0) / np.sqrt(np.float32(self.d)))
         self.qkv_width = (self.heads + 2 * self.kv_heads) * self.d
+        self.capturable = self.position.table(1) is not None   # an encoding applied by other code is not captured
 
     def cache_need(self):
         return CacheNeed(self.kv_heads, self.d, self.window)
@@ -83,9 +85,11 @@ class GQAAttention(Mixer):
         else:
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
         attn = ctx.scratch("attn", (T, self.heads * self.d), self.rt.dtype)
+        floats = 0 if exact else ops.decode_scratch_floats(T, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
+        partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
         ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions,
                             self.heads, self.kv_heads, self.d, self.window, self.scale, exact,
-                            max_q_len=ctx.max_q_len, max_context=ctx.max_context)
+                            max_q_len=ctx.max_q_len, max_context=ctx.max_context, scratch=partial)
         if self.b_o is not None:
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
             ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)

@@ -11,6 +11,7 @@ from .base import FeedForward, register_part
 
 class SwiGLU(FeedForward):
     """params: prefix, hidden, intermediate."""
+    capturable = True   # native kernels on the current stream only: a decode step may be graph-captured
 
     @classmethod
     def tensors(cls, spec):

@@ -163,3 +163,40 @@ def test_pool_too_small_is_a_named_error(tiny_dirs):
     with pytest.raises(AlofaError) as e:
         r.step({"step": 1, "entries": [{"id": "b", "tokens": [TINY["A"]["vocab_size"]], "want": [0]}], "end": []})
     assert e.value.name == "out_of_range"
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_decode_graph_replays_equal_eager_steps(tiny_dirs, name):
+    """Decode steps replay a captured HIP graph. Every replay is compared with
+    the same step run eagerly, with other work (portions of other requests,
+    synchronisations, a request ending and another taking its pages) between
+    the replays."""
+    from alofa_amd.replay import Replayer
+    vocab = TINY[name]["vocab_size"]
+    ids = {r: random_ids(60 + i, 90, vocab) for i, r in enumerate("abc")}
+    extra = random_ids(70, 60, vocab)
+
+    def play(graphs):
+        os.environ["ALOFA_GRAPHS"] = "1" if graphs else "0"
+        try:
+            r = Replayer(tiny_dirs[name], "bfloat16", 512)
+        finally:
+            os.environ.pop("ALOFA_GRAPHS")
+        assert r.fn.use_graphs == graphs
+        out = []
+        r.step({"step": 0, "entries": [{"id": k, "tokens": v[:40], "want": []} for k, v in ids.items()], "end": []})
+        for i in range(40, 90):
+            live = [k for k in ids if not (k == "c" and i >= 70)]
+            out.append(r.step({"step": i, "entries": [{"id": k, "tokens": [ids[k][i]], "want": [0]} for k in live],
+                               "end": ["c"] if i == 69 else []}).copy())
+            if i % 7 == 0:     # eager work between the replays: a portion of another request
+                out.append(r.step({"step": 1000 + i, "entries": [{"id": "x", "tokens": extra[(i - 40):(i - 40) + 7], "want": [6]}], "end": []}).copy())
+        return r, out
+    eager_r, eager = play(False)
+    graph_r, graphed = play(True)
+    assert graph_r.fn.graph_replays >= 40 and eager_r.fn.graph_replays == 0
+    assert len(graph_r.fn._graphs) >= 3            # batch 3 and batch 2, more than one context bucket
+    for i, (a, b) in enumerate(zip(eager, graphed)):
+        assert np.array_equal(a, b), f"step {i}: a replay differs from the eager step"
+    ref = plain_logits(tiny_dirs[name], tuple(ids["a"]))
+    assert_close(np.stack([o[0] for o in graphed if o.shape[0] in (2, 3)]), ref[40:90], "bfloat16", "graph decode vs plain")

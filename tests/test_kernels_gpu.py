@@ -224,8 +224,9 @@ def test_decode_attention(heads, kv_heads, d, bs, window):
     out = torch.empty(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
     scale = float(np.float32(1) / np.sqrt(np.float32(d)))
     o = ops()
+    scratch = torch.empty(max(1, o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, 700, window)), device=DEV)
     o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, False,
-                      max_q_len=4, max_context=700)
+                      max_q_len=4, max_context=700, scratch=scratch)
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(5)])
     close(out, ref, BF16, "decode attention")
     if (heads, d, window) == (14, 64, None):
@@ -234,6 +235,11 @@ def test_decode_attention(heads, kv_heads, d, bs, window):
     o.paged_attention(one, c["qcat"][:1], c["kc"], c["vc"], c["table"], c["req"][:1], c["pos"][:1], heads, kv_heads, d, window, scale, False,
                       max_q_len=1, max_context=1)
     close(one, ref[:1], BF16, "decode attention, first token")
+    if o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, 700, window):
+        from alofa_amd.errors import AlofaError
+        with pytest.raises(AlofaError):                                          # needed scratch is demanded, not allocated behind the back
+            o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, False,
+                              max_q_len=4, max_context=700)
 
 
 @pytest.mark.parametrize("dtype,exact", [(torch.float32, True), (torch.bfloat16, False)])
@@ -252,7 +258,7 @@ def test_attention_far_key_and_window_edge(dtype, exact):
     assert np.abs(ref[0] - v_far).max() < 1e-3                          # the far key really decides the output
     for window, sees in ((L - far, True), (L - far - 1, False)):         # the window's edge, to the key
         ops().paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, exact,
-                              max_q_len=None if exact else 1, max_context=L)
+                              max_q_len=None if exact else 1, max_context=L, scratch=torch.empty(1 << 16, device=DEV))
         refw = pm.attention(c["q"][0], c["k"][0], c["v"][0], heads, kv_heads, d, window)
         close(out, refw, 2e-6 if exact else BF16, f"window {window}")
         assert (np.abs(refw[0] - v_far).max() < 1e-3) == sees
