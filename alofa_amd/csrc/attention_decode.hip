@@ -2,8 +2,8 @@
 // and short portions), bfloat16. The work is reading every visible key and value
 // once, so all query heads of one key head are served together.
 //
-// One wavefront handles (token, key head, split): a contiguous share of the
-// token's visible keys lo..p. d / 16 lanes share a key (16 channels each), so a
+// One wavefront handles (token, key head and up to four of its query heads,
+// split): a contiguous share of the token's visible keys lo..p. d / 16 lanes share a key (16 channels each), so a
 // wave takes 64 / (d / 16) keys per round with fully used 32-byte loads. Every
 // lane group keeps a running softmax of its own (maximum, sum of weights,
 // weighted sum of its 16 value channels, per head, all float); dot products use
@@ -27,7 +27,7 @@ __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
 }
 
-// GC: query heads handled at once (the group is walked in chunks of GC).
+// GC: query heads per wavefront; blockIdx.y = key head * chunks + chunk of GC heads of its group.
 template <int GC>
 __global__ void __launch_bounds__(64) attention_decode_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ partial, const bf16_t* __restrict__ q,
@@ -35,9 +35,10 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ positions, int heads, int kv_heads, int d, int block_size, int window, float scale,
     int n_splits) {
-  extern __shared__ float lds[];  // [GC][kpi][d] weighted sums, then [GC][kpi] maxima, [GC][kpi] sums
-  const int t = blockIdx.x, hk = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+  extern __shared__ float lds[];  // [kpi][d]: one head's weighted value sums of every lane group
   const int group = heads / kv_heads;
+  const int chunks = (group + GC - 1) / GC;
+  const int t = blockIdx.x, hk = blockIdx.y / chunks, split = blockIdx.z, lane = threadIdx.x;
   const int lpk = d / 16;          // lanes per key
   const int kpi = 64 / lpk;        // keys per round
   const int slot = lane / lpk, part = lane % lpk;
@@ -51,7 +52,8 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
   const int32_t* table = block_table + static_cast<int64_t>(req_of_token[t]) * max_blocks;
   const int64_t head_stride = static_cast<int64_t>(block_size) * d;
 
-  for (int h0 = 0; h0 < group; h0 += GC) {
+  {
+    const int h0 = (blockIdx.y % chunks) * GC;
     uint32_t qp[GC][8];
 #pragma unroll
     for (int i = 0; i < GC; ++i) {
@@ -136,29 +138,30 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
       k0 = nk0; k1 = nk1; v0 = nv0; v1 = nv1;
     }
 
-    // the lane groups' states meet in LDS and are combined in group order
-    float* lds_o = lds;
-    float* lds_m = lds + GC * kpi * d;
-    float* lds_l = lds_m + GC * kpi;
-    __syncthreads();
-    if (active) {
+    // The lane groups' states are combined: the maximum over all groups, every group's
+    // weight exp(m - max), the sum of weights by a fixed butterfly, and the weighted
+    // value sums through LDS, added in group order.
+    float* lds_o = lds;                     // [kpi][d] of the head in work
 #pragma unroll
-      for (int i = 0; i < GC; ++i) {
-#pragma unroll
-        for (int c = 0; c < 16; ++c) lds_o[(i * kpi + slot) * d + part * 16 + c] = o[i][c];
-        if (part == 0) { lds_m[i * kpi + slot] = m[i]; lds_l[i * kpi + slot] = l[i]; }
-      }
-    }
-    __syncthreads();
-    for (int i = 0; i < GC && h0 + i < group; ++i) {
+    for (int i = 0; i < GC; ++i) {
+      if (h0 + i >= group) break;   // uniform over the block
       const int h = hk * group + h0 + i;
-      float big = -FLT_MAX;
-      for (int s2 = 0; s2 < kpi; ++s2) big = fmaxf(big, lds_m[i * kpi + s2]);
-      float total = 0.f;
-      for (int s2 = 0; s2 < kpi; ++s2) total += lds_l[i * kpi + s2] * __expf(lds_m[i * kpi + s2] - big);
+      const float big = wave_max(m[i]);
+      const float e = __expf(m[i] - big);   // 0 for groups that saw no key
+      const float total = wave_sum((active && part == 0) ? l[i] * e : 0.f);
+      __syncthreads();
+      if (active) {
+        float4* dst = reinterpret_cast<float4*>(lds_o + slot * d + part * 16);
+        dst[0] = make_float4(o[i][0] * e, o[i][1] * e, o[i][2] * e, o[i][3] * e);
+        dst[1] = make_float4(o[i][4] * e, o[i][5] * e, o[i][6] * e, o[i][7] * e);
+        dst[2] = make_float4(o[i][8] * e, o[i][9] * e, o[i][10] * e, o[i][11] * e);
+        dst[3] = make_float4(o[i][12] * e, o[i][13] * e, o[i][14] * e, o[i][15] * e);
+      }
+      __syncthreads();
       for (int c = lane; c < d; c += 64) {
         float acc = 0.f;
-        for (int s2 = 0; s2 < kpi; ++s2) acc += lds_o[(i * kpi + s2) * d + c] * __expf(lds_m[i * kpi + s2] - big);
+#pragma unroll 8
+        for (int s2 = 0; s2 < kpi; ++s2) acc += lds_o[s2 * d + c];
         if (n_splits == 1) {
           store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
         } else {
@@ -176,15 +179,18 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
 __global__ void __launch_bounds__(64) attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
                                                              const float* __restrict__ partial, int heads, int d,
                                                              int n_splits) {
-  const int t = blockIdx.x, h = blockIdx.y;
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float* src = partial + (static_cast<int64_t>(t) * heads + h) * n_splits * (d + 2);
-  float big = -FLT_MAX;
-  for (int s = 0; s < n_splits; ++s) big = fmaxf(big, src[s * (d + 2)]);
-  float total = 0.f;
-  for (int s = 0; s < n_splits; ++s) total += src[s * (d + 2) + 1] * __expf(src[s * (d + 2)] - big);
-  for (int c = threadIdx.x; c < d; c += 64) {
+  // lane s holds split s's maximum and sum (n_splits <= 64)
+  const float m = lane < n_splits ? src[lane * (d + 2)] : -FLT_MAX;
+  const float l = lane < n_splits ? src[lane * (d + 2) + 1] : 0.f;
+  const float big = wave_max(m);
+  const float e = __expf(m - big);
+  const float total = wave_sum(l * e);
+  for (int c = lane; c < d; c += 64) {
     float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s) acc += src[s * (d + 2) + 2 + c] * __expf(src[s * (d + 2)] - big);
+#pragma unroll 8
+    for (int s = 0; s < n_splits; ++s) acc += src[s * (d + 2) + 2 + c] * __shfl(e, s, 64);
     store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
   }
 }
@@ -211,19 +217,20 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   ALOFA_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_decode: q rows must be 16-byte aligned");
   const int group = heads / kv_heads;
   const int kpi = 64 / (d / 16);
-  dim3 grid(tokens, kv_heads, n_splits);
+  const int gc = group == 1 ? 1 : group == 2 ? 2 : group == 3 ? 3 : 4;
+  dim3 grid(tokens, kv_heads * ((group + gc - 1) / gc), n_splits);
 #define ALOFA_DECODE(GC)                                                                                                  \
   {                                                                                                                       \
-    const size_t lds = static_cast<size_t>(GC) * kpi * (d + 2) * sizeof(float);                                           \
+    const size_t lds = static_cast<size_t>(kpi) * d * sizeof(float);                                           \
     attention_decode_kernel<GC><<<grid, 64, lds, stream>>>(                                                               \
         static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                          \
         static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, max_blocks, req_of_token,  \
         positions, heads, kv_heads, d, block_size, window, scale, n_splits);                                              \
   }
-  if (group == 1) ALOFA_DECODE(1)
-  else if (group == 2) ALOFA_DECODE(2)
-  else if (group <= 4) ALOFA_DECODE(4)
-  else ALOFA_DECODE(8)
+  if (gc == 1) ALOFA_DECODE(1)
+  else if (gc == 2) ALOFA_DECODE(2)
+  else if (gc == 3) ALOFA_DECODE(3)
+  else ALOFA_DECODE(4)
 #undef ALOFA_DECODE
   if (check_launch("attention_decode")) return 1;
   if (n_splits > 1) {

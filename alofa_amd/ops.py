@@ -132,9 +132,11 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
             raise AlofaError("shape_mismatch", "bias length does not fit", f"bias={tuple(bias.shape)} N={N}")
     if add_to_out and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the residual stream is float32", f"out={out.dtype}")
-    if not exact and _mfma_operands(a, w) and M <= SKINNY_MAX_ROWS:
-        _call("alofa_gemm_skinny", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None),
-              _L(_rows("w", w)), _ptr(None if add_to_out else bias), _I(M), _I(N), _I(K), _I(ADD_TO_RESIDUAL if add_to_out else STORE), _stream())
+    if not exact and _mfma_operands(a, w):
+        # few rows: the weight-streaming kernel; many rows: the tiled one
+        _call("alofa_gemm_skinny" if M <= SKINNY_MAX_ROWS else "alofa_gemm_mfma", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
+              _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(None if add_to_out else bias), _I(M), _I(N), _I(K),
+              _I(ADD_TO_RESIDUAL if add_to_out else STORE), _stream())
         return
     _call("alofa_gemm_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
           _ptr(w), _I(dtype_code(w)), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
@@ -150,8 +152,8 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: 
         raise AlofaError("shape_mismatch", "gate/up product shapes do not fit", f"a={tuple(a.shape)} gate={tuple(w_gate.shape)} up={tuple(w_up.shape)} out={tuple(out.shape)}")
     if w_gate.dtype is not w_up.dtype or _rows("w_gate", w_gate) != _rows("w_up", w_up):
         raise AlofaError("invalid_argument", "gate and up matrices must share dtype and layout")
-    if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up) and M <= SKINNY_MAX_ROWS:
-        _call("alofa_gemm_skinny", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
+    if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up):
+        _call("alofa_gemm_skinny" if M <= SKINNY_MAX_ROWS else "alofa_gemm_mfma", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
               _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), _stream())
         return
     _call("alofa_gemm_swiglu_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
@@ -216,10 +218,10 @@ DECODE_MAX_Q = 4          # requests with at most this many query tokens use the
 
 def decode_splits(tokens: int, kv_heads: int, d: int, max_context: int) -> int:
     """Shares of the keys per (token, key head): enough waves to fill the chip,
-    but at least four rounds of keys each."""
+    but at least eight rounds of keys each."""
     keys_per_round = 64 // (d // 16)
-    by_chip = -(-1024 // max(1, tokens * kv_heads))
-    by_length = max(1, max_context // (4 * keys_per_round))
+    by_chip = -(-2048 // max(1, tokens * kv_heads))
+    by_length = max(1, max_context // (8 * keys_per_round))
     return max(1, min(64, by_chip, by_length))
 
 
