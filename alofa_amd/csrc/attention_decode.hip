@@ -33,12 +33,14 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ partial, const bf16_t* __restrict__ q,
     int64_t q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
-    const int32_t* __restrict__ positions, int heads, int kv_heads, int d, int block_size, int window, float scale,
-    int n_splits) {
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ rows, int heads, int kv_heads, int d,
+    int block_size, int window, float scale, int n_splits) {
   extern __shared__ float lds[];  // [kpi][d]: one head's weighted value sums of every lane group
   const int group = heads / kv_heads;
   const int chunks = (group + GC - 1) / GC;
-  const int t = blockIdx.x, hk = blockIdx.y / chunks, split = blockIdx.z, lane = threadIdx.x;
+  // the tokens served are rows[0..gridDim.x) of the packed batch, or all of it
+  const int t = rows ? rows[blockIdx.x] : blockIdx.x;
+  const int hk = blockIdx.y / chunks, split = blockIdx.z, lane = threadIdx.x;
   const int lpk = d / 16;          // lanes per key
   const int kpi = 64 / lpk;        // keys per round
   const int slot = lane / lpk, part = lane % lpk;
@@ -165,7 +167,7 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
         if (n_splits == 1) {
           store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
         } else {
-          float* dst = partial + ((static_cast<int64_t>(t) * heads + h) * n_splits + split) * (d + 2);
+          float* dst = partial + ((static_cast<int64_t>(blockIdx.x) * heads + h) * n_splits + split) * (d + 2);
           dst[2 + c] = acc;
           if (c == 0) { dst[0] = big; dst[1] = total; }
         }
@@ -177,10 +179,11 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
 
 // Combines the splits' states of one (token, head) in split order.
 __global__ void __launch_bounds__(64) attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
-                                                             const float* __restrict__ partial, int heads, int d,
+                                                             const float* __restrict__ partial,
+                                                             const int32_t* __restrict__ rows, int heads, int d,
                                                              int n_splits) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const float* src = partial + (static_cast<int64_t>(t) * heads + h) * n_splits * (d + 2);
+  const int t = rows ? rows[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* src = partial + (static_cast<int64_t>(blockIdx.x) * heads + h) * n_splits * (d + 2);
   // lane s holds split s's maximum and sum (n_splits <= 64)
   const float m = lane < n_splits ? src[lane * (d + 2)] : -FLT_MAX;
   const float l = lane < n_splits ? src[lane * (d + 2) + 1] : 0.f;
@@ -207,7 +210,7 @@ extern "C" int64_t alofa_attention_decode_scratch(int tokens, int heads, int d, 
 extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
                                       const void* k_cache, const void* v_cache, const int32_t* block_table,
                                       int max_blocks, const int32_t* req_of_token, const int32_t* positions,
-                                      int tokens, int heads, int kv_heads, int d, int block_size, int window,
+                                      const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
                                       float scale, int n_splits, hipStream_t stream) {
   ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
@@ -225,7 +228,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
     attention_decode_kernel<GC><<<grid, 64, lds, stream>>>(                                                               \
         static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                          \
         static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, max_blocks, req_of_token,  \
-        positions, heads, kv_heads, d, block_size, window, scale, n_splits);                                              \
+        positions, rows, heads, kv_heads, d, block_size, window, scale, n_splits);                                        \
   }
   if (gc == 1) ALOFA_DECODE(1)
   else if (gc == 2) ALOFA_DECODE(2)
@@ -234,7 +237,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
 #undef ALOFA_DECODE
   if (check_launch("attention_decode")) return 1;
   if (n_splits > 1) {
-    attention_merge_kernel<<<dim3(tokens, heads), 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, heads, d, n_splits);
+    attention_merge_kernel<<<dim3(tokens, heads), 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits);
     return check_launch("attention_merge");
   }
   return 0;

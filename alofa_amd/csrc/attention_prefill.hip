@@ -1,0 +1,223 @@
+// Paged causal grouped-query attention for prompt portions, bfloat16 on MFMA,
+// with a running softmax so that no score matrix is ever stored.
+//
+// A block of four wavefronts serves 64 consecutive query rows of one request
+// and one query head; every wave owns 16 rows. The visible keys are walked in
+// tiles of 32 that start at absolute multiples of 32, so the order of additions
+// for a row is the same however the prompt was cut into steps. Per tile the
+// block stages the keys [32, d] and the values transposed [d, 32] in LDS.
+//
+// Both products are taken transposed, so that one lane's data stays with one
+// query row throughout (v_mfma_f32_16x16x32_bf16; lane l: A row and B column
+// l % 16, D column l % 16 and rows 4 * (l / 16) .. + 3):
+//   S^T[key, q] = K[key, :] . Q[q, :]      A = keys from LDS, B = queries (registers)
+//   O^T[c, q] += V^T[c, key] * P^T[key, q]  A = values^T from LDS, B = weights (registers)
+// After the first product lane l holds, for query l % 16, the scores of keys
+// 4 g + r and 16 + 4 g + r (g = l / 16, r = 0..3); these eight are exactly the
+// reduction slots of the second product when the values are read in the same
+// order, so the weights never leave their registers.
+// Scores, the running maximum, the weights and their sum are float; the
+// weights are rounded to bfloat16 only as MFMA operands.
+// Cache layout: [block, kv_head, slot_in_block, d].
+#include "common.h"
+
+#include <float.h>
+
+namespace alofa {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int BQ = 64;    // query rows per block
+constexpr int BKV = 32;   // keys per tile
+constexpr int KPAD = 8, VPAD = 8;
+
+// tiles: int32 [n_tiles, 4] = (request index, first row in the packed batch, rows (<= 64), position of the first row)
+template <int DT>  // DT = d / 16
+__global__ void __launch_bounds__(256) attention_prefill_kernel(
+    bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
+    int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int block_size, int window,
+    float scale) {
+  constexpr int d = DT * 16;
+  constexpr int DS = (d + 31) / 32;           // steps of 32 along d in the first product
+  constexpr int KROW = d + KPAD, VROW = BKV + VPAD;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * KROW];
+  __shared__ __attribute__((aligned(16))) bf16_t Vt[d * VROW];
+
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int c16 = lane % 16, g = lane / 16;
+  const int32_t* tile = tiles + 4 * blockIdx.x;
+  const int req = tile[0], row0 = tile[1], n_rows = tile[2], pos0 = tile[3];
+  const int head = blockIdx.y, hk = head / (heads / kv_heads);
+  const int32_t* table = block_table + static_cast<int64_t>(req) * max_blocks;
+
+  // this lane's query row and its fragments of Q
+  const int my_row = wave * 16 + c16;                 // within the tile
+  const bool row_ok = my_row < n_rows;
+  const int my_pos = pos0 + my_row;
+  bf16x8 qf[DS];
+#pragma unroll
+  for (int ds = 0; ds < DS; ++ds) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    const int c = ds * 32 + g * 8;
+    if (row_ok && c < d)
+      v = *reinterpret_cast<const uint4*>(q + static_cast<int64_t>(row0 + my_row) * q_stride + static_cast<int64_t>(head) * d + c);
+    qf[ds] = __builtin_bit_cast(bf16x8, v);
+  }
+
+  f32x4 o[DT];
+#pragma unroll
+  for (int nt = 0; nt < DT; ++nt) o[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -FLT_MAX, l = 0.f;
+
+  // keys the block needs: from the first key its first row sees to the last row's own position
+  const int last_pos = pos0 + n_rows - 1;
+  const int first_key = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int t_begin = first_key / BKV, t_end = last_pos / BKV;     // inclusive
+
+  // staging: chunks of 8 channels; the block moves 32 * d / 8 chunks of K and of V per tile
+  constexpr int kChunks = BKV * d / 8;
+  constexpr int kPerThread = (kChunks + 255) / 256;
+  uint4 k_reg[kPerThread], v_reg[kPerThread];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      const int c = tid + 256 * j;
+      k_reg[j] = v_reg[j] = make_uint4(0, 0, 0, 0);
+      if (c < kChunks) {
+        const int key = t * BKV + c / (d / 8), ch = (c % (d / 8)) * 8;
+        if (key <= last_pos && key >= first_key) {
+          const int64_t blk = table[key / block_size];
+          const int64_t base = ((blk * kv_heads + hk) * block_size + key % block_size) * static_cast<int64_t>(d) + ch;
+          k_reg[j] = *reinterpret_cast<const uint4*>(k_cache + base);
+          v_reg[j] = *reinterpret_cast<const uint4*>(v_cache + base);
+        }
+      }
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      const int c = tid + 256 * j;
+      if (c < kChunks) {
+        const int key = c / (d / 8), ch = (c % (d / 8)) * 8;
+        *reinterpret_cast<uint4*>(&Ks[key * KROW + ch]) = k_reg[j];
+        const uint32_t w[4] = {v_reg[j].x, v_reg[j].y, v_reg[j].z, v_reg[j].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          Vt[(ch + 2 * e) * VROW + key] = static_cast<bf16_t>(w[e] & 0xffffu);
+          Vt[(ch + 2 * e + 1) * VROW + key] = static_cast<bf16_t>(w[e] >> 16);
+        }
+      }
+    }
+  };
+
+  fetch(t_begin);
+  for (int t = t_begin; t <= t_end; ++t) {
+    __syncthreads();      // the previous tile has been read by every wave
+    stage();
+    __syncthreads();
+    if (t < t_end) fetch(t + 1);
+
+    // S^T for the two 16-key halves of the tile
+    f32x4 s[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ds = 0; ds < DS; ++ds) {
+        const int c = ds * 32 + g * 8;
+        uint4 kv = make_uint4(0, 0, 0, 0);
+        if (c < d) kv = *reinterpret_cast<const uint4*>(&Ks[(kt * 16 + c16) * KROW + c]);
+        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kv), qf[ds], s[kt], 0, 0, 0);
+      }
+    }
+    // scale, mask, running maximum
+    float p[8];
+    bool seen[8];
+    float tile_max = -FLT_MAX;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int key = t * BKV + (i / 4) * 16 + g * 4 + i % 4;
+      seen[i] = key <= my_pos && (window <= 0 || key > my_pos - window);
+      p[i] = s[i / 4][i % 4] * scale;
+      if (seen[i]) tile_max = fmaxf(tile_max, p[i]);
+    }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(m, tile_max);
+    const float corr = __expf(m - m_new);   // 1 while nothing was seen yet (both -FLT_MAX)
+    m = m_new;
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      p[i] = seen[i] ? __expf(p[i] - m_new) : 0.f;
+      sum += p[i];
+    }
+    l = l * corr + sum;   // this lane's share of the row's sum; the four lanes of a row meet at the end
+    bf16x8 pf;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) pf[i] = static_cast<__bf16>(p[i]);
+    // O^T += V^T P^T
+#pragma unroll
+    for (int nt = 0; nt < DT; ++nt) {
+      o[nt] *= corr;
+      const bf16_t* vrow = &Vt[(nt * 16 + c16) * VROW];
+      const uint2 lo = *reinterpret_cast<const uint2*>(vrow + g * 4);
+      const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16 + g * 4);
+      const uint4 vv = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf, o[nt], 0, 0, 0);
+    }
+  }
+
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (row_ok) {
+    const float inv = 1.f / l;
+    bf16_t* dst = out + static_cast<int64_t>(row0 + my_row) * out_stride + static_cast<int64_t>(head) * d;
+#pragma unroll
+    for (int nt = 0; nt < DT; ++nt) {
+      uint2 w;
+      w.x = static_cast<uint32_t>(f32_to_bf16(o[nt][0] * inv)) | (static_cast<uint32_t>(f32_to_bf16(o[nt][1] * inv)) << 16);
+      w.y = static_cast<uint32_t>(f32_to_bf16(o[nt][2] * inv)) | (static_cast<uint32_t>(f32_to_bf16(o[nt][3] * inv)) << 16);
+      *reinterpret_cast<uint2*>(dst + nt * 16 + g * 4) = w;
+    }
+  }
+}
+
+}  // namespace alofa
+
+using namespace alofa;
+
+extern "C" int alofa_attention_prefill_supports(int d) {
+  return d == 16 || d == 32 || d == 48 || d == 64 || d == 96 || d == 128 || d == 256;
+}
+
+extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                       const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                       int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
+                                       int block_size, int window, float scale, hipStream_t stream) {
+  ALOFA_REQUIRE(n_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
+                "attention_prefill: tiles=%d heads=%d kv_heads=%d (kv_heads must divide heads)", n_tiles, heads, kv_heads);
+  ALOFA_REQUIRE(alofa_attention_prefill_supports(d), "attention_prefill: head size %d is not built (16, 32, 48, 64, 96, 128, 256 are)", d);
+  ALOFA_REQUIRE(block_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill: block_size=%d max_blocks=%d window=%d", block_size, max_blocks, window);
+  ALOFA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
+                "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
+  dim3 grid(n_tiles, heads);
+#define ALOFA_PREFILL(DT)                                                                                                 \
+  attention_prefill_kernel<DT><<<grid, 256, 0, stream>>>(                                                                 \
+      static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, block_size, window, scale)
+  switch (d / 16) {
+    case 1: ALOFA_PREFILL(1); break;
+    case 2: ALOFA_PREFILL(2); break;
+    case 3: ALOFA_PREFILL(3); break;
+    case 4: ALOFA_PREFILL(4); break;
+    case 6: ALOFA_PREFILL(6); break;
+    case 8: ALOFA_PREFILL(8); break;
+    case 16: ALOFA_PREFILL(16); break;
+  }
+#undef ALOFA_PREFILL
+  return check_launch("attention_prefill");
+}

@@ -17,6 +17,10 @@ from ..cache.manager import CacheManager
 from ..errors import AlofaError
 
 
+SHORT = 4     # rows of one request up to which attention treats them as single tokens
+TILE_ROWS = 64
+
+
 def _pow2_ceil(n: int) -> int:
     return max(64, 1 << (int(n) - 1).bit_length())
 
@@ -64,6 +68,12 @@ class StepContext:
         # launches, and a coarse value lets captured decode graphs be used again
         self.max_context = _pow2_ceil(max(s.pos0 + s.n for s in spans))
         self.n_positions = fn.n_positions
+        # how attention splits the rows: requests that bring at most SHORT rows are "short"
+        # (served key-head-wise, one token at a time), the others are cut into tiles of
+        # up to 64 rows. short_rows is None when every row is short.
+        self.n_short = sum(s.n for s in spans if s.n <= SHORT)
+        self.short_rows: Optional[torch.Tensor] = None
+        self.long_tiles: Optional[torch.Tensor] = None
         self.positions: torch.Tensor = None
         self.req_of_token: torch.Tensor = None
         self._tables: list = []
@@ -207,6 +217,13 @@ class StepFunction:
         ctx._tables = [tables_d[g] for g in range(n_groups)]
         ctx._slots = [slots_d[g] for g in range(n_groups)]
         rows = torch.tensor(want_rows, dtype=torch.int32, device=dev) if want_rows else None
+        if ctx.n_short < T:
+            tiles = [(i, s.row0 + q0, min(TILE_ROWS, s.n - q0), s.pos0 + q0)
+                     for i, s in enumerate(spans) if s.n > SHORT for q0 in range(0, s.n, TILE_ROWS)]
+            ctx.long_tiles = torch.tensor(tiles, dtype=torch.int32, device=dev)
+            if ctx.n_short:
+                ctx.short_rows = torch.tensor([r for s in spans if s.n <= SHORT for r in range(s.row0, s.row0 + s.n)],
+                                              dtype=torch.int32, device=dev)
         return ctx, ids_d, rows
 
     def finish(self, ctx: StepContext) -> None:

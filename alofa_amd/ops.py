@@ -258,21 +258,70 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         raise AlofaError("shape_mismatch", "one request index and one position per token")
     if (not exact and q.dtype is torch.bfloat16 and max_q_len is not None and max_q_len <= DECODE_MAX_Q and d % 16 == 0
             and _rows("q", q) % 8 == 0 and q.data_ptr() % 16 == 0):
-        ctx_len = max_context or 1 << 30
-        n_splits = decode_splits(T, kv_heads, d, min(ctx_len, window or ctx_len))
-        floats = T * heads * n_splits * (d + 2) if n_splits > 1 else 0
-        partial = None
-        if floats:
-            if scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous():
-                raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")
-            partial = scratch
-        _call("alofa_attention_decode", _ptr(out), _L(_rows("out", out)), _ptr(partial), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
-              _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T), _I(heads), _I(kv_heads), _I(d),
-              _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits), _stream())
+        attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
+                         max_context or 1 << 30, scratch)
         return
     _call("alofa_attention_simple", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
           _I(dtype_code(q)), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T),
           _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(int(exact)), _stream())
+
+
+def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d):
+    _gpu("out", out, torch.bfloat16, 2), _gpu("q", q, torch.bfloat16, 2)
+    T = q.shape[0]
+    if out.shape[0] != T or out.shape[1] < heads * d or q.shape[1] < heads * d:
+        raise AlofaError("shape_mismatch", "attention rows do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} heads={heads} d={d}")
+    if d % 16 or not 16 <= d <= MAX_HEAD_DIM or kv_heads <= 0 or heads % kv_heads:
+        raise AlofaError("unsupported", "head size 16..256 in steps of 16, kv_heads dividing heads", f"head_dim={d} heads={heads} kv_heads={kv_heads}")
+    bs = check_cache("k_cache", k_cache, kv_heads, d)
+    check_cache("v_cache", v_cache, kv_heads, d)
+    if k_cache.shape != v_cache.shape or k_cache.dtype is not torch.bfloat16 or v_cache.dtype is not torch.bfloat16:
+        raise AlofaError("shape_mismatch", "caches must agree with each other and be bfloat16")
+    _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
+    if _rows("q", q) % 8 or q.data_ptr() % 16 or _rows("out", out) % 4 or out.data_ptr() % 8:
+        raise AlofaError("alignment", "attention rows must be 16-byte aligned", f"q_stride={_rows('q', q)} out_stride={_rows('out', out)}")
+    return T, bs
+
+
+def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
+                     max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
+    """bfloat16 attention for tokens of requests that bring few tokens: every
+    token of the batch, or the tokens ``rows`` (int32 indices into the batch)."""
+    T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
+    for n, t in (("req_of_token", req_of_token), ("positions", positions)):
+        _gpu(n, t, torch.int32, 1), _contig(n, t)
+        if t.shape[0] != T:
+            raise AlofaError("shape_mismatch", "one request index and one position per token")
+    n_tok = T
+    if rows is not None:
+        _gpu("rows", rows, torch.int32, 1), _contig("rows", rows)
+        n_tok = rows.shape[0]
+    n_splits = decode_splits(n_tok, kv_heads, d, min(max_context, window or max_context))
+    floats = n_tok * heads * n_splits * (d + 2) if n_splits > 1 else 0
+    if floats and (scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous()):
+        raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")
+    _call("alofa_attention_decode", _ptr(out), _L(_rows("out", out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
+          _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(rows),
+          _I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits), _stream())
+
+
+PREFILL_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 256)
+
+
+def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale) -> None:
+    """bfloat16 attention for portions of prompts. ``tiles`` is int32 [n, 4]:
+    (request index, first row, rows <= 64, position of the first row) for every
+    run of up to 64 consecutive rows of one request; the caller builds it from
+    the same spans as the block tables."""
+    T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
+    if d not in PREFILL_HEAD_DIMS:
+        raise AlofaError("unsupported", "the prefill attention kernel is not built for this head size", f"head_dim={d} built={PREFILL_HEAD_DIMS}")
+    _gpu("tiles", tiles, torch.int32, 2), _contig("tiles", tiles)
+    if tiles.shape[1] != 4 or tiles.shape[0] == 0:
+        raise AlofaError("shape_mismatch", "tiles must be [n, 4]", f"tiles={tuple(tiles.shape)}")
+    _call("alofa_attention_prefill", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
+          _ptr(block_table), _I(block_table.shape[1]), _ptr(tiles), _I(tiles.shape[0]), _I(heads), _I(kv_heads), _I(d), _I(bs),
+          _I(int(window or 0)), _F(scale), _stream())
 
 
 # ------------------------------------------------------------------ sampling

@@ -85,11 +85,19 @@ class GQAAttention(Mixer):
         else:
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
         attn = ctx.scratch("attn", (T, self.heads * self.d), self.rt.dtype)
-        floats = 0 if exact else ops.decode_scratch_floats(T, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
-        partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
-        ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions,
-                            self.heads, self.kv_heads, self.d, self.window, self.scale, exact,
-                            max_q_len=ctx.max_q_len, max_context=ctx.max_context, scratch=partial)
+        common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
+        fast_prefill = not exact and self.d in ops.PREFILL_HEAD_DIMS
+        if exact or (ctx.long_tiles is not None and not fast_prefill):
+            # the exact path, and head sizes the tiled kernel is not built for
+            ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
+        else:
+            if ctx.long_tiles is not None:      # portions of prompts
+                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, ctx.long_tiles, *common)
+            if ctx.n_short:                     # single tokens and very short portions, all key heads' groups together
+                floats = ops.decode_scratch_floats(ctx.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
+                partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
+                ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common,
+                                     ctx.max_context, partial, rows=ctx.short_rows)
         if self.b_o is not None:
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
             ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)

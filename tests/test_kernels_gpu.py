@@ -242,6 +242,37 @@ def test_decode_attention(heads, kv_heads, d, bs, window):
                               max_q_len=4, max_context=700)
 
 
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 96, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (3, 1, 32, 64)])
+@pytest.mark.parametrize("window", [None, 21, 300])
+def test_prefill_attention(heads, kv_heads, d, bs, window):
+    """The tiled kernel for portions of prompts: whole prompts, portions deep in
+    a context, runs of exactly 64 and 65 rows, several tiles per request."""
+    rng = np.random.default_rng(23)
+    lens, q_lens = [37, 130, 700, 64, 65, 200], [37, 5, 100, 64, 65, 200]
+    c = paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16)
+    tiles, row = [], 0
+    for r, (L, n) in enumerate(zip(lens, q_lens)):
+        tiles += [(r, row + q0, min(64, n - q0), L - n + q0) for q0 in range(0, n, 64)]
+        row += n
+    out = torch.zeros(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(tiles, np.int32), torch.int32), heads, kv_heads, d, window, scale)
+    ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(len(lens))])
+    close(out, ref, BF16, "prefill attention")
+
+
+def test_prefill_attention_far_key():
+    rng = np.random.default_rng(29)
+    heads, kv_heads, d, bs, L, far = 6, 2, 64, 16, 700, 3
+    c = paged_case(rng, [L], [40], heads, kv_heads, d, bs, torch.bfloat16, scale_key=far)
+    out = torch.zeros(40, heads * d, device=DEV, dtype=torch.bfloat16)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    for window in (None, L - far, L - far - 1):
+        ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array([[0, 0, 40, L - 40]], np.int32), torch.int32),
+                                heads, kv_heads, d, window, scale)
+        close(out, pm.attention(c["q"][0], c["k"][0], c["v"][0], heads, kv_heads, d, window), BF16, f"far key, window {window}")
+
+
 @pytest.mark.parametrize("dtype,exact", [(torch.float32, True), (torch.bfloat16, False)])
 def test_attention_far_key_and_window_edge(dtype, exact):
     """One far key among hundreds carries the weight: dropping it, or any page of
