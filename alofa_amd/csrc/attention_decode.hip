@@ -34,7 +34,7 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
     int64_t q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ rows, int heads, int kv_heads, int d,
-    int block_size, int window, float scale, int n_splits) {
+    int bs_shift, int window, float scale, int n_splits) {
   extern __shared__ float lds[];  // [kpi][d]: one head's weighted value sums of every lane group
   const int group = heads / kv_heads;
   const int chunks = (group + GC - 1) / GC;
@@ -52,7 +52,7 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
   const int begin = lo + split * per_split;
   const int end = (begin + per_split < p + 1) ? begin + per_split : p + 1;
   const int32_t* table = block_table + static_cast<int64_t>(req_of_token[t]) * max_blocks;
-  const int64_t head_stride = static_cast<int64_t>(block_size) * d;
+  const int64_t head_stride = static_cast<int64_t>(d) << bs_shift;   // pages hold a power of two of tokens
 
   {
     const int h0 = (blockIdx.y % chunks) * GC;
@@ -77,8 +77,8 @@ __global__ void __launch_bounds__(64) attention_decode_kernel(
 
     auto fetch = [&](int j, uint4& k0, uint4& k1, uint4& v0, uint4& v1) {
       if (active && j < end) {
-        const int64_t blk = table[j / block_size];
-        const int64_t base = (blk * kv_heads + hk) * head_stride + static_cast<int64_t>(j % block_size) * d + part * 16;
+        const int64_t blk = table[j >> bs_shift];
+        const int64_t base = (blk * kv_heads + hk) * head_stride + static_cast<int64_t>(j & ((1 << bs_shift) - 1)) * d + part * 16;
         const uint4* kp = reinterpret_cast<const uint4*>(k_cache + base);
         const uint4* vp = reinterpret_cast<const uint4*>(v_cache + base);
         k0 = kp[0]; k1 = kp[1]; v0 = vp[0]; v1 = vp[1];
@@ -215,7 +215,10 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
   ALOFA_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention_decode: head size %d must be 16..256 in steps of 16", d);
-  ALOFA_REQUIRE(block_size > 0 && max_blocks > 0 && window >= 0, "attention_decode: block_size=%d max_blocks=%d window=%d", block_size, max_blocks, window);
+  ALOFA_REQUIRE(block_size > 0 && (block_size & (block_size - 1)) == 0 && max_blocks > 0 && window >= 0,
+                "attention_decode: block_size=%d must be a power of two; max_blocks=%d window=%d", block_size, max_blocks, window);
+  int bs_shift = 0;
+  while ((1 << bs_shift) < block_size) ++bs_shift;
   ALOFA_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || partial), "attention_decode: n_splits=%d (1..%d) needs scratch when above 1", n_splits, kMaxSplits);
   ALOFA_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_decode: q rows must be 16-byte aligned");
   const int group = heads / kv_heads;
@@ -228,7 +231,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
     attention_decode_kernel<GC><<<grid, 64, lds, stream>>>(                                                               \
         static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                          \
         static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, max_blocks, req_of_token,  \
-        positions, rows, heads, kv_heads, d, block_size, window, scale, n_splits);                                        \
+        positions, rows, heads, kv_heads, d, bs_shift, window, scale, n_splits);                                          \
   }
   if (gc == 1) ALOFA_DECODE(1)
   else if (gc == 2) ALOFA_DECODE(2)

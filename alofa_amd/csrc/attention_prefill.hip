@@ -3,19 +3,19 @@
 //
 // A block of four wavefronts serves 64 consecutive query rows of one request
 // and one query head; every wave owns 16 rows. The visible keys are walked in
-// tiles of 32 that start at absolute multiples of 32, so the order of additions
+// tiles of 64 that start at absolute multiples of 64, so the order of additions
 // for a row is the same however the prompt was cut into steps. Per tile the
-// block stages the keys [32, d] and the values transposed [d, 32] in LDS.
+// block stages the keys [64, d] and the values transposed [d, 64] in LDS.
 //
 // Both products are taken transposed, so that one lane's data stays with one
 // query row throughout (v_mfma_f32_16x16x32_bf16; lane l: A row and B column
 // l % 16, D column l % 16 and rows 4 * (l / 16) .. + 3):
 //   S^T[key, q] = K[key, :] . Q[q, :]      A = keys from LDS, B = queries (registers)
 //   O^T[c, q] += V^T[c, key] * P^T[key, q]  A = values^T from LDS, B = weights (registers)
-// After the first product lane l holds, for query l % 16, the scores of keys
-// 4 g + r and 16 + 4 g + r (g = l / 16, r = 0..3); these eight are exactly the
-// reduction slots of the second product when the values are read in the same
-// order, so the weights never leave their registers.
+// After the first product of a 32-key half lane l holds, for query l % 16, the
+// scores of keys 4 g + r and 16 + 4 g + r (g = l / 16, r = 0..3); these eight are
+// exactly the reduction slots of the second product when the values are read in
+// the same order, so the weights never leave their registers.
 // Scores, the running maximum, the weights and their sum are float; the
 // weights are rounded to bfloat16 only as MFMA operands.
 // Cache layout: [block, kv_head, slot_in_block, d].
@@ -29,7 +29,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BQ = 64;    // query rows per block
-constexpr int BKV = 32;   // keys per tile
+constexpr int BKV = 64;   // keys per tile
 constexpr int KPAD = 8, VPAD = 8;
 
 // tiles: int32 [n_tiles, 4] = (request index, first row in the packed batch, rows (<= 64), position of the first row)
@@ -37,7 +37,7 @@ template <int DT>  // DT = d / 16
 __global__ void __launch_bounds__(256) attention_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
-    int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int block_size, int window,
+    int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int bs_shift, int window,
     float scale) {
   constexpr int d = DT * 16;
   constexpr int DS = (d + 31) / 32;           // steps of 32 along d in the first product
@@ -47,7 +47,8 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
 
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int c16 = lane % 16, g = lane / 16;
-  const int32_t* tile = tiles + 4 * blockIdx.x;
+  // later tiles of a prompt see more keys: they are started first so that the short ones fill the tail
+  const int32_t* tile = tiles + 4 * (gridDim.x - 1 - blockIdx.x);
   const int req = tile[0], row0 = tile[1], n_rows = tile[2], pos0 = tile[3];
   const int head = blockIdx.y, hk = head / (heads / kv_heads);
   const int32_t* table = block_table + static_cast<int64_t>(req) * max_blocks;
@@ -70,6 +71,7 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
 #pragma unroll
   for (int nt = 0; nt < DT; ++nt) o[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -FLT_MAX, l = 0.f;
+  const float scale2 = scale * 1.44269504088896340736f;   // scores in units of log2(e)
 
   // keys the block needs: from the first key its first row sees to the last row's own position
   const int last_pos = pos0 + n_rows - 1;
@@ -88,8 +90,9 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
       if (c < kChunks) {
         const int key = t * BKV + c / (d / 8), ch = (c % (d / 8)) * 8;
         if (key <= last_pos && key >= first_key) {
-          const int64_t blk = table[key / block_size];
-          const int64_t base = ((blk * kv_heads + hk) * block_size + key % block_size) * static_cast<int64_t>(d) + ch;
+          // pages hold a power of two of tokens: block = key >> shift, slot = key & mask
+          const int64_t blk = table[key >> bs_shift];
+          const int64_t base = ((((blk * kv_heads + hk) << bs_shift) + (key & ((1 << bs_shift) - 1))) * d) + ch;
           k_reg[j] = *reinterpret_cast<const uint4*>(k_cache + base);
           v_reg[j] = *reinterpret_cast<const uint4*>(v_cache + base);
         }
@@ -120,10 +123,10 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
     __syncthreads();
     if (t < t_end) fetch(t + 1);
 
-    // S^T for the two 16-key halves of the tile
-    f32x4 s[2];
+    // S^T for the four 16-key quarters of the tile
+    f32x4 s[4];
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
+    for (int kt = 0; kt < 4; ++kt) {
       s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ds = 0; ds < DS; ++ds) {
@@ -133,41 +136,60 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
         s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kv), qf[ds], s[kt], 0, 0, 0);
       }
     }
-    // scale, mask, running maximum
-    float p[8];
-    bool seen[8];
+    // scale, mask, running maximum. Scores are kept in units of log2(e) so that the
+    // weights are single exp2 instructions; tiles that every row of the block sees
+    // whole (all but the last one or two) skip the masking.
+    float p[16];
     float tile_max = -FLT_MAX;
+    const bool whole = t * BKV + BKV - 1 <= pos0 && (window <= 0 || t * BKV > last_pos - window);
+    if (whole) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int key = t * BKV + (i / 4) * 16 + g * 4 + i % 4;
-      seen[i] = key <= my_pos && (window <= 0 || key > my_pos - window);
-      p[i] = s[i / 4][i % 4] * scale;
-      if (seen[i]) tile_max = fmaxf(tile_max, p[i]);
+      for (int i = 0; i < 16; ++i) {
+        p[i] = s[i / 4][i % 4] * scale2;
+        tile_max = fmaxf(tile_max, p[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = t * BKV + (i / 4) * 16 + g * 4 + i % 4;
+        const bool seen = key <= my_pos && (window <= 0 || key > my_pos - window);
+        p[i] = seen ? s[i / 4][i % 4] * scale2 : -FLT_MAX;
+        tile_max = fmaxf(tile_max, p[i]);
+      }
     }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
     const float m_new = fmaxf(m, tile_max);
-    const float corr = __expf(m - m_new);   // 1 while nothing was seen yet (both -FLT_MAX)
+    const float corr = __builtin_amdgcn_exp2f(m - m_new);    // 1 while nothing was seen yet (both -FLT_MAX)
     m = m_new;
     float sum = 0.f;
+    // a masked score is -FLT_MAX: its weight is 0 unless the row has seen nothing yet
+    // (m_new is then -FLT_MAX too), which the second test catches
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      p[i] = seen[i] ? __expf(p[i] - m_new) : 0.f;
+    for (int i = 0; i < 16; ++i) {
+      p[i] = (p[i] > -FLT_MAX) ? __builtin_amdgcn_exp2f(p[i] - m_new) : 0.f;
       sum += p[i];
     }
     l = l * corr + sum;   // this lane's share of the row's sum; the four lanes of a row meet at the end
-    bf16x8 pf;
+    bf16x8 pf[2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) pf[i] = static_cast<__bf16>(p[i]);
-    // O^T += V^T P^T
+    for (int half = 0; half < 2; ++half) {
+      const uint4 w = make_uint4(pack_bf16x2(p[8 * half], p[8 * half + 1]), pack_bf16x2(p[8 * half + 2], p[8 * half + 3]),
+                                 pack_bf16x2(p[8 * half + 4], p[8 * half + 5]), pack_bf16x2(p[8 * half + 6], p[8 * half + 7]));
+      pf[half] = __builtin_bit_cast(bf16x8, w);
+    }
+    // O^T += V^T P^T, one MFMA per 32-key half
 #pragma unroll
     for (int nt = 0; nt < DT; ++nt) {
       o[nt] *= corr;
       const bf16_t* vrow = &Vt[(nt * 16 + c16) * VROW];
-      const uint2 lo = *reinterpret_cast<const uint2*>(vrow + g * 4);
-      const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16 + g * 4);
-      const uint4 vv = make_uint4(lo.x, lo.y, hi.x, hi.y);
-      o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf, o[nt], 0, 0, 0);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow + half * 32 + g * 4);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + half * 32 + 16 + g * 4);
+        const uint4 vv = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf[half], o[nt], 0, 0, 0);
+      }
     }
   }
 
@@ -179,8 +201,8 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
 #pragma unroll
     for (int nt = 0; nt < DT; ++nt) {
       uint2 w;
-      w.x = static_cast<uint32_t>(f32_to_bf16(o[nt][0] * inv)) | (static_cast<uint32_t>(f32_to_bf16(o[nt][1] * inv)) << 16);
-      w.y = static_cast<uint32_t>(f32_to_bf16(o[nt][2] * inv)) | (static_cast<uint32_t>(f32_to_bf16(o[nt][3] * inv)) << 16);
+      w.x = pack_bf16x2(o[nt][0] * inv, o[nt][1] * inv);
+      w.y = pack_bf16x2(o[nt][2] * inv, o[nt][3] * inv);
       *reinterpret_cast<uint2*>(dst + nt * 16 + g * 4) = w;
     }
   }
@@ -201,14 +223,17 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
   ALOFA_REQUIRE(n_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_prefill: tiles=%d heads=%d kv_heads=%d (kv_heads must divide heads)", n_tiles, heads, kv_heads);
   ALOFA_REQUIRE(alofa_attention_prefill_supports(d), "attention_prefill: head size %d is not built (16, 32, 48, 64, 96, 128, 256 are)", d);
-  ALOFA_REQUIRE(block_size > 0 && max_blocks > 0 && window >= 0, "attention_prefill: block_size=%d max_blocks=%d window=%d", block_size, max_blocks, window);
+  ALOFA_REQUIRE(block_size > 0 && (block_size & (block_size - 1)) == 0 && max_blocks > 0 && window >= 0,
+                "attention_prefill: block_size=%d must be a power of two; max_blocks=%d window=%d", block_size, max_blocks, window);
+  int bs_shift = 0;
+  while ((1 << bs_shift) < block_size) ++bs_shift;
   ALOFA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
                 "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
   dim3 grid(n_tiles, heads);
 #define ALOFA_PREFILL(DT)                                                                                                 \
   attention_prefill_kernel<DT><<<grid, 256, 0, stream>>>(                                                                 \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
-      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, block_size, window, scale)
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
   switch (d / 16) {
     case 1: ALOFA_PREFILL(1); break;
     case 2: ALOFA_PREFILL(2); break;

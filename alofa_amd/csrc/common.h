@@ -20,13 +20,16 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
   return __uint_as_float(static_cast<uint32_t>(v) << 16);
 }
 
-// round to nearest, ties to even; NaN stays NaN
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<bf16_t>(u >> 16);
+// two floats to a pair of bfloat16 (a in the low half), round to nearest even:
+// the hardware conversion v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return static_cast<bf16_t>(pack_bf16x2(f, 0.f) & 0xffffu); }
 
 template <typename T> __device__ __forceinline__ float load_f32(const T* p);
 template <> __device__ __forceinline__ float load_f32<float>(const float* p) { return *p; }

@@ -1,9 +1,11 @@
 // Matrix products for many rows (prompt portions), bfloat16 on MFMA:
 // out[m, n] = sum_k A[m, k] * W[n, k].
 //
-// A block of four wavefronts computes a 128 x 128 tile of the output; every
-// wave owns a 64 x 64 quarter as 2 x 2 tiles of v_mfma_f32_32x32x16_bf16. Per
-// step of 32 along K the block stages a 128 x 32 slab of A and of W in LDS
+// A block of four wavefronts (2 x 2) computes a 128 x 128 tile of the output,
+// every wave a 64 x 64 quarter as 2 x 2 tiles of v_mfma_f32_32x32x16_bf16; for
+// outputs too small to fill the chip with such tiles the block computes 64 x 64
+// (one MFMA tile per wave). Per step of 64 along K the block stages a slab of A
+// and of W in LDS
 // (16-byte loads along K; rows are padded by 8 elements so that the fragment
 // reads fall on distinct banks), while the next slab is already on its way from
 // memory into registers. Accumulation is float; each output element has one
@@ -25,15 +27,18 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 enum MfmaEpilogue : int { kMfStore = 0, kMfResidual = 1, kMfSwiglu = 2 };
 
-constexpr int TM = 128, TN = 128, TK = 32, PAD = 8;
+constexpr int TK = 64, PAD = 8;
 constexpr int kRow = TK + PAD;  // LDS row length in elements
 
-template <int kEpilogue, typename TO>
+// WT: MFMA tiles per wave along each of m and n (2: 128 x 128 block tile, 1: 64 x 64)
+template <int kEpilogue, typename TO, int WT>
 __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, int64_t ldo,
                                                         const bf16_t* __restrict__ A, int64_t lda,
                                                         const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                                         int64_t ldw, const float* __restrict__ bias, int M, int N,
                                                         int K) {
+  constexpr int TM = 64 * WT, TN = 64 * WT;
+  static_assert(kEpilogue != kMfSwiglu || WT == 2, "the swiglu epilogue needs two column tiles per wave");
   __shared__ __attribute__((aligned(16))) bf16_t As[TM * kRow];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[TN * kRow];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -41,14 +46,17 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
   constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * kOutCols;
 
-  // global -> register staging: 512 chunks of 16 bytes per slab, two per thread
-  const int c_row[2] = {tid / 4, (tid + 256) / 4};
-  const int c_k = (tid % 4) * 8;
-  const bf16_t* a_src[2];
-  const bf16_t* w_src[2];
-  bool a_ok[2], w_ok[2];
+  // global -> register staging: TM * 8 chunks of 16 bytes per slab, NC per thread
+  constexpr int NC = WT * 2;
+  int c_row[NC];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < NC; ++j) c_row[j] = (tid + 256 * j) / 8;
+  const int c_k = (tid % 8) * 8;
+  const bf16_t* a_src[NC];
+  const bf16_t* w_src[NC];
+  bool a_ok[NC], w_ok[NC];
+#pragma unroll
+  for (int j = 0; j < NC; ++j) {
     const int m = m0 + c_row[j];
     a_ok[j] = m < M;
     a_src[j] = A + static_cast<int64_t>(a_ok[j] ? m : 0) * lda + c_k;
@@ -64,26 +72,26 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
     w_src[j] = base + static_cast<int64_t>(w_ok[j] ? n : 0) * ldw + c_k;
   }
 
-  f32x16 acc[2][2];
+  f32x16 acc[WT][WT];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < WT; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < WT; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  uint4 a_reg[2], w_reg[2];
+  uint4 a_reg[NC], w_reg[NC];
   auto fetch = [&](int k0) {
     const bool k_ok = k0 + c_k < K;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NC; ++j) {
       a_reg[j] = (k_ok && a_ok[j]) ? *reinterpret_cast<const uint4*>(a_src[j] + k0) : make_uint4(0, 0, 0, 0);
       w_reg[j] = (k_ok && w_ok[j]) ? *reinterpret_cast<const uint4*>(w_src[j] + k0) : make_uint4(0, 0, 0, 0);
     }
   };
   auto stage = [&]() {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NC; ++j) {
       *reinterpret_cast<uint4*>(&As[c_row[j] * kRow + c_k]) = a_reg[j];
       *reinterpret_cast<uint4*>(&Ws[c_row[j] * kRow + c_k]) = w_reg[j];
     }
@@ -91,12 +99,12 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 
   // rows of the fragments this lane reads
   const int frag_row = lane % 32, frag_k = (lane / 32) * 8;
-  int a_off[2], w_off[2];
+  int a_off[WT], w_off[WT];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    a_off[i] = (wm * 64 + i * 32 + frag_row) * kRow + frag_k;
+  for (int i = 0; i < WT; ++i) {
+    a_off[i] = (wm * 32 * WT + i * 32 + frag_row) * kRow + frag_k;
     // swiglu: tile 0 = gate rows of this wave's 32 columns, tile 1 = the up rows of the same columns
-    w_off[i] = ((kEpilogue == kMfSwiglu) ? (i * 64 + wn * 32 + frag_row) : (wn * 64 + i * 32 + frag_row)) * kRow + frag_k;
+    w_off[i] = ((kEpilogue == kMfSwiglu) ? (i * 64 + wn * 32 + frag_row) : (wn * 32 * WT + i * 32 + frag_row)) * kRow + frag_k;
   }
 
   fetch(0);
@@ -107,31 +115,31 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
     if (k0 + TK < K) fetch(k0 + TK);
 #pragma unroll
     for (int ks = 0; ks < TK; ks += 16) {
-      bf16x8 a[2], w[2];
+      bf16x8 a[WT], w[WT];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < WT; ++i) {
         a[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&As[a_off[i] + ks]));
         w[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Ws[w_off[i] + ks]));
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < WT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < WT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
     }
   }
 
   // epilogue
   const int col = lane % 32, row_base = (lane / 32) * 4;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < WT; ++i) {
 #pragma unroll
-    for (int j = 0; j < ((kEpilogue == kMfSwiglu) ? 1 : 2); ++j) {
-      const int n = (kEpilogue == kMfSwiglu) ? n0 + wn * 32 + col : n0 + wn * 64 + j * 32 + col;
+    for (int j = 0; j < ((kEpilogue == kMfSwiglu) ? 1 : WT); ++j) {
+      const int n = (kEpilogue == kMfSwiglu) ? n0 + wn * 32 + col : n0 + wn * 32 * WT + j * 32 + col;
       if (n >= N) continue;
       const float b = (bias && kEpilogue == kMfStore) ? bias[n] : 0.f;
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm * 64 + i * 32 + 8 * (e / 4) + row_base + e % 4;
+        const int m = m0 + wm * 32 * WT + i * 32 + 8 * (e / 4) + row_base + e % 4;
         if (m >= M) continue;
         TO* dst = out + static_cast<int64_t>(m) * ldo + n;
         if (kEpilogue == kMfStore) {
@@ -140,7 +148,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
           store_f32(dst, load_f32(dst) + acc[i][j][e]);
         } else {
           const float g = acc[i][0][e];
-          store_f32(dst, g / (1.f + __expf(-g)) * acc[i][1][e]);
+          store_f32(dst, g / (1.f + __expf(-g)) * acc[i][WT - 1][e]);
         }
       }
     }
@@ -150,11 +158,21 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 template <int kEpilogue, typename TO>
 static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                        const float* bias, int M, int N, int K, hipStream_t stream) {
-  constexpr int cols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
-  dim3 grid((N + cols - 1) / cols, (M + TM - 1) / TM);
-  gemm_mfma_kernel<kEpilogue, TO><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
-                                                             static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2),
-                                                             ldw, bias, M, N, K);
+  // big tiles when they fill the chip (about two blocks per compute unit), small ones otherwise
+  const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
+  if (kEpilogue == kMfSwiglu || big_blocks >= 512) {
+    constexpr int cols = (kEpilogue == kMfSwiglu) ? 64 : 128;
+    dim3 grid((N + cols - 1) / cols, (M + 127) / 128);
+    gemm_mfma_kernel<kEpilogue, TO, 2><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
+                                                                  static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2),
+                                                                  ldw, bias, M, N, K);
+  } else {
+    constexpr int kE = (kEpilogue == kMfSwiglu) ? kMfStore : kEpilogue;   // (never taken for swiglu)
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    gemm_mfma_kernel<kE, TO, 1><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
+                                                           static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw,
+                                                           bias, M, N, K);
+  }
   return check_launch("gemm_mfma");
 }
 

@@ -257,7 +257,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     if req_of_token.shape[0] != T or positions.shape[0] != T:
         raise AlofaError("shape_mismatch", "one request index and one position per token")
     if (not exact and q.dtype is torch.bfloat16 and max_q_len is not None and max_q_len <= DECODE_MAX_Q and d % 16 == 0
-            and _rows("q", q) % 8 == 0 and q.data_ptr() % 16 == 0):
+            and _rows("q", q) % 8 == 0 and q.data_ptr() % 16 == 0 and bs & (bs - 1) == 0):
         attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
                          max_context or 1 << 30, scratch)
         return
@@ -277,6 +277,8 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
     check_cache("v_cache", v_cache, kv_heads, d)
     if k_cache.shape != v_cache.shape or k_cache.dtype is not torch.bfloat16 or v_cache.dtype is not torch.bfloat16:
         raise AlofaError("shape_mismatch", "caches must agree with each other and be bfloat16")
+    if bs & (bs - 1):
+        raise AlofaError("unsupported", "the bfloat16 attention kernels take pages of a power of two of tokens", f"block_size={bs}")
     _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
     if _rows("q", q) % 8 or q.data_ptr() % 16 or _rows("out", out) % 4 or out.data_ptr() % 8:
         raise AlofaError("alignment", "attention rows must be 16-byte aligned", f"q_stride={_rows('q', q)} out_stride={_rows('out', out)}")
