@@ -21,7 +21,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum SkinnyEpilogue : int { kSkStore = 0, kSkResidual = 1, kSkSwiglu = 2 };
 
-constexpr int kUnroll = 4;
 
 __device__ __forceinline__ bf16x8 load_frag(const bf16_t* __restrict__ p, bool ok) {
   uint4 v = make_uint4(0, 0, 0, 0);
@@ -31,7 +30,8 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* __restrict__ p, bool o
 
 // MT: 16-row tiles of A; NT: 16-column tiles per block (kSkSwiglu: tile 0 is the
 // gate matrix, tile 1 the up matrix, same columns); TO: float or bf16_t.
-template <int MT, int NT, int kWaves, int kEpilogue, typename TO>
+// kUnroll: steps of 32 along K whose loads are in flight together (twice that with the prefetch).
+template <int MT, int NT, int kWaves, int kEpilogue, typename TO, int kUnroll>
 __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
     const bf16_t* __restrict__ W2, int64_t ldw, const float* __restrict__ bias, int M, int N, int K) {
@@ -143,7 +143,8 @@ template <int MT, int NT, int kWaves, int kEpilogue, typename TO>
 static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                          const float* bias, int M, int N, int K, hipStream_t stream) {
   constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
-  gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO><<<(N + cols - 1) / cols, kWaves * 64, 0, stream>>>(
+  constexpr int unroll = (MT >= 4) ? 2 : 4;   // many row tiles: fewer steps in flight, or registers run out
+  gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, unroll><<<(N + cols - 1) / cols, kWaves * 64, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
       static_cast<const bf16_t*>(W2), ldw, bias, M, N, K);
   return check_launch("gemm_skinny");
@@ -152,16 +153,17 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
 template <int kEpilogue, typename TO>
 static int dispatch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                            const float* bias, int M, int N, int K, hipStream_t stream) {
-  // few columns: one 16-column tile per block and eight waves along K keep more of the chip busy
+  // few columns: one 16-column tile per block and eight waves along K keep more of the chip busy;
+  // many columns and many rows: four column tiles per block, so that the rows are read less often
   const bool narrow = (kEpilogue != kSkSwiglu) && N <= 4096;
-#define ALOFA_SKINNY(MT)                                                                                              \
+#define ALOFA_SKINNY(MT, WIDE)                                                                                        \
   if (kEpilogue == kSkSwiglu)                                                                                         \
     return launch_skinny<MT, 2, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);               \
   if (narrow) return launch_skinny<MT, 1, 8, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);     \
-  return launch_skinny<MT, 2, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
-  if (M <= 16) { ALOFA_SKINNY(1) }
-  if (M <= 32) { ALOFA_SKINNY(2) }
-  ALOFA_SKINNY(4)
+  return launch_skinny<MT, WIDE, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+  if (M <= 16) { ALOFA_SKINNY(1, 2) }
+  if (M <= 32) { ALOFA_SKINNY(2, 4) }
+  ALOFA_SKINNY(4, 4)
 #undef ALOFA_SKINNY
 }
 

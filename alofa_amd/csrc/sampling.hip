@@ -39,6 +39,54 @@ __global__ void __launch_bounds__(kPickThreads) argmax_kernel(int32_t* __restric
   }
 }
 
+// Two-stage form for long rows: kArgmaxChunks blocks per row each find the first
+// maximum of a contiguous chunk, then one wave per row takes the first maximum of
+// the chunks in chunk order (a lower chunk holds lower indices, so ties still go
+// to the lowest index).
+constexpr int kArgmaxChunks = 64;
+
+__global__ void __launch_bounds__(256) argmax_chunk_kernel(float* __restrict__ part_v, int32_t* __restrict__ part_i,
+                                                           const float* __restrict__ logits, int64_t stride, int vocab) {
+  __shared__ float best_v[4];
+  __shared__ int best_i[4];
+  const int r = blockIdx.y, chunk = blockIdx.x;
+  const int per = (vocab + kArgmaxChunks - 1) / kArgmaxChunks;
+  const int lo = chunk * per, hi = (lo + per < vocab) ? lo + per : vocab;
+  const float* row = logits + static_cast<int64_t>(r) * stride;
+  float bv = -FLT_MAX;
+  int bi = vocab;
+  for (int i = lo + threadIdx.x; i < hi; i += 256) {
+    const float v = row[i];
+    if (v > bv) { bv = v; bi = i; }
+  }
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, kWave);
+    const int oi = __shfl_xor(bi, off, kWave);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if (threadIdx.x % kWave == 0) { best_v[threadIdx.x / kWave] = bv; best_i[threadIdx.x / kWave] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
+    part_v[r * kArgmaxChunks + chunk] = bv;
+    part_i[r * kArgmaxChunks + chunk] = bi;
+  }
+}
+
+__global__ void __launch_bounds__(kWave) argmax_final_kernel(int32_t* __restrict__ out, const float* __restrict__ part_v,
+                                                             const int32_t* __restrict__ part_i, int vocab) {
+  const int r = blockIdx.x;
+  float bv = part_v[r * kArgmaxChunks + threadIdx.x];
+  int bi = part_i[r * kArgmaxChunks + threadIdx.x];
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, kWave);
+    const int oi = __shfl_xor(bi, off, kWave);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if (threadIdx.x == 0) out[r] = bi < vocab ? bi : 0;
+}
+
 __global__ void __launch_bounds__(kPickThreads) sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits,
                                                               int64_t stride, int vocab,
                                                               const double* __restrict__ temperature,
@@ -88,11 +136,20 @@ __global__ void __launch_bounds__(kPickThreads) sample_kernel(int32_t* __restric
 
 using namespace alofa;
 
-extern "C" int alofa_argmax(int32_t* out, const float* logits, int64_t stride, int rows, int vocab,
+// scratch: rows * 64 floats followed by rows * 64 int32 for long rows (null: one block per row)
+extern "C" int alofa_argmax(int32_t* out, const float* logits, int64_t stride, int rows, int vocab, void* scratch,
                             hipStream_t stream) {
   ALOFA_REQUIRE(rows > 0 && vocab > 0 && stride >= vocab, "argmax: rows=%d vocab=%d stride=%lld", rows, vocab, static_cast<long long>(stride));
-  argmax_kernel<<<rows, kPickThreads, 0, stream>>>(out, logits, stride, vocab);
-  return check_launch("argmax");
+  if (scratch == nullptr) {
+    argmax_kernel<<<rows, kPickThreads, 0, stream>>>(out, logits, stride, vocab);
+    return check_launch("argmax");
+  }
+  float* part_v = static_cast<float*>(scratch);
+  int32_t* part_i = reinterpret_cast<int32_t*>(part_v + static_cast<int64_t>(rows) * kArgmaxChunks);
+  argmax_chunk_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(part_v, part_i, logits, stride, vocab);
+  if (check_launch("argmax_chunk")) return 1;
+  argmax_final_kernel<<<rows, kWave, 0, stream>>>(out, part_v, part_i, vocab);
+  return check_launch("argmax_final");
 }
 
 extern "C" int alofa_sample(int32_t* out, const float* logits, int64_t stride, int rows, int vocab,

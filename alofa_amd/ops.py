@@ -333,7 +333,9 @@ def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
     _gpu("out", out, torch.int32, 1), _gpu("logits", logits, torch.float32, 2), _contig("out", out)
     if out.shape[0] != logits.shape[0]:
         raise AlofaError("shape_mismatch", "one choice per row")
-    _call("alofa_argmax", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(logits.shape[0]), _I(logits.shape[1]), _stream())
+    # long rows are searched by 64 blocks each, through a small scratch (values, then indices)
+    scratch = torch.empty(2 * 64 * logits.shape[0], dtype=torch.float32, device=logits.device) if logits.shape[1] >= 8192 else None
+    _call("alofa_argmax", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(logits.shape[0]), _I(logits.shape[1]), _ptr(scratch), _stream())
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor) -> None:

@@ -304,6 +304,13 @@ def test_argmax_and_sample():
     out = torch.empty(5, dtype=torch.int32, device=DEV)
     ops().argmax(out, t(logits))
     assert out.tolist() == [pm.argmax(r) for r in logits] and out[1].item() == 7 and out[2].item() == 0
+    big = rng.standard_normal((3, 151936)).astype(np.float32)       # long rows take the two-stage search
+    big[0, [150000, 2400, 77000]] = 11.0
+    big[1, :] = 2.0
+    big[2, 151935] = 12.0
+    outb = torch.empty(3, dtype=torch.int32, device=DEV)
+    ops().argmax(outb, t(big))
+    assert outb.tolist() == [2400, 0, 151935]
     rows = np.repeat(logits[:1], 64, axis=0)
     temps = np.full(64, 0.8)
     us = np.array([ps.SplitMix64(3).next_uniform() for _ in range(1)] + list(rng.random(61)) + [0.0, 0.9999999999999999])
