@@ -120,6 +120,7 @@ def main():
     ap.add_argument("--layers", type=int, default=QWEN25_05B["num_hidden_layers"], help="fewer layers than the configuration has, where memory or time needs it")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (--gpus must be 1)")
@@ -131,6 +132,11 @@ def main():
     cfg = dict(QWEN25_05B, num_hidden_layers=args.layers)
     with tempfile.TemporaryDirectory() as d:
         write_random_model(cfg, d, seed=20260918)
+        if args.only_prefill:
+            pt = measure_prefill(d, cfg, args.dtype, 2048)
+            print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
+                                          "frac": round(prefill_flops(cfg, 2048) / pt / PEAK_FLOPS[args.dtype], 4)}}))
+            return 0
         ms, ctx_lens = measure_decode(d, cfg, args.dtype, args.batch, args.steps, args.warmup)
         value = args.batch / ms
         dbytes = 2 if args.dtype == "bfloat16" else 4
