@@ -9,6 +9,15 @@
 // the result is the same on every run and for every batch the row is part of
 // (M only selects how many 16-row tiles are computed).
 //
+// With few output columns the blocks are too few to pull the weights at speed,
+// so K is also split across blocks (blockIdx.y): every block leaves its partial
+// tiles in a workspace and bumps a counter of its column tile; the block that
+// arrives last adds the partial tiles in split order (not in arrival order, so
+// the sum is the same on every run), runs the epilogue and puts the counter
+// back to zero. Nobody waits for anybody. The workspace is uncached device
+// memory: what one block wrote is what another reads, whichever die they run
+// on, without flushing caches; fences only order the accesses within a block.
+//
 // Operand layout of v_mfma_f32_16x16x32_bf16, lane l: A holds row l % 16,
 // B holds column l % 16, both the 8 reduction indices 8 * (l / 16) .. + 7 of
 // the step; D holds column l % 16, rows 4 * (l / 16) .. + 3.
@@ -34,8 +43,10 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* __restrict__ p, bool o
 template <int MT, int NT, int kWaves, int kEpilogue, typename TO, int kUnroll>
 __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
-    const bf16_t* __restrict__ W2, int64_t ldw, const float* __restrict__ bias, int M, int N, int K) {
+    const bf16_t* __restrict__ W2, int64_t ldw, const float* __restrict__ bias, int M, int N, int K,
+    f32x4* __restrict__ ws, int* __restrict__ counters) {
   __shared__ f32x4 red[kWaves][MT * NT][64];
+  __shared__ int last_block;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int r = lane % 16, g = lane / 16;
   constexpr int kColsPerBlock = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
@@ -65,14 +76,18 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int n_steps = (K + 31) / 32;  // steps of 32 along K; this wave takes steps wave, wave + kWaves, ...
+  // steps of 32 along K: this block takes a contiguous share, this wave every kWaves-th step of it
+  const int all_steps = (K + 31) / 32, k_splits = gridDim.y;
+  const int per_split = (all_steps + k_splits - 1) / k_splits;
+  const int first_step = blockIdx.y * per_split;
+  const int n_steps = (first_step + per_split < all_steps) ? first_step + per_split : all_steps;
   bf16x8 a_cur[kUnroll][MT], w_cur[kUnroll][NT], a_nxt[kUnroll][MT], w_nxt[kUnroll][NT];
 
   auto load = [&](bf16x8 (&a)[kUnroll][MT], bf16x8 (&w)[kUnroll][NT], int first) {
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       const int k = (first + u * kWaves) * 32 + g * 8;
-      const bool k_ok = k < K;
+      const bool k_ok = k < K && first + u * kWaves < n_steps;
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) w[u][nt] = load_frag(w_row[nt] + k, k_ok && w_ok[nt]);
 #pragma unroll
@@ -80,8 +95,8 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     }
   };
 
-  load(a_cur, w_cur, wave);
-  for (int s = wave; s < n_steps; s += kUnroll * kWaves) {
+  load(a_cur, w_cur, first_step + wave);
+  for (int s = first_step + wave; s < n_steps; s += kUnroll * kWaves) {
     if (s + kUnroll * kWaves < n_steps) load(a_nxt, w_nxt, s + kUnroll * kWaves);
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
@@ -105,19 +120,46 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     for (int nt = 0; nt < NT; ++nt) red[wave][mt * NT + nt][lane] = acc[mt][nt];
   __syncthreads();
 
-  // tiles are shared out among the waves; each adds the partial sums in wave order
+  if (k_splits > 1) {
+    // this block's tiles (its waves added in wave order) go to the workspace; the last block to arrive goes on
+    f32x4* mine = ws + (static_cast<int64_t>(blockIdx.x) * k_splits + blockIdx.y) * (MT * NT * 64);
+    for (int tile = wave; tile < MT * NT; tile += kWaves) {
+      f32x4 sum = red[0][tile][lane];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) sum += red[w][tile][lane];
+      mine[tile * 64 + lane] = sum;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // this wave's tiles have left before the block is counted
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const int arrived = atomicAdd(&counters[blockIdx.x], 1);
+      last_block = arrived == k_splits - 1;
+      if (last_block) atomicExch(&counters[blockIdx.x], 0);
+    }
+    __syncthreads();
+    if (!last_block) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  }
+  const f32x4* parts = ws + static_cast<int64_t>(blockIdx.x) * k_splits * (MT * NT * 64);
+
+  // tiles are shared out among the waves; each adds the partial sums in wave (or split) order
   constexpr int kOutTiles = (kEpilogue == kSkSwiglu) ? MT : MT * NT;
   for (int tile = wave; tile < kOutTiles; tile += kWaves) {
     const int mt = (kEpilogue == kSkSwiglu) ? tile : tile / NT;
     const int nt = (kEpilogue == kSkSwiglu) ? 0 : tile % NT;
-    f32x4 sum = red[0][mt * NT + nt][lane];
+    f32x4 sum, up = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (k_splits > 1) {
+      sum = parts[(mt * NT + nt) * 64 + lane];
+      for (int ks = 1; ks < k_splits; ++ks) sum += parts[(ks * MT * NT + mt * NT + nt) * 64 + lane];
+    } else {
+      sum = red[0][mt * NT + nt][lane];
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) sum += red[w][mt * NT + nt][lane];
-    f32x4 up = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (kEpilogue == kSkSwiglu) {
-      up = red[0][mt * NT + 1][lane];
+      for (int w = 1; w < kWaves; ++w) sum += red[w][mt * NT + nt][lane];
+      if (kEpilogue == kSkSwiglu) {
+        up = red[0][mt * NT + 1][lane];
 #pragma unroll
-      for (int w = 1; w < kWaves; ++w) up += red[w][mt * NT + 1][lane];
+        for (int w = 1; w < kWaves; ++w) up += red[w][mt * NT + 1][lane];
+      }
     }
     const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
     if (n >= N) continue;
@@ -139,14 +181,36 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   }
 }
 
+// Workspace of the cross-block K split: partial tiles and one zeroed counter per column tile, in
+// uncached device memory that the library allocates once per process and never frees. Every call
+// leaves the counters zero. Calls that overlap on one GPU (two streams) would race on it.
+struct SkinnyWorkspace {
+  f32x4* tiles;
+  int64_t tile_floats;
+  int* counters;
+  int n_counters;
+};
+static SkinnyWorkspace g_ws = {nullptr, 0, nullptr, 0};
+constexpr int64_t kWsTileFloats = 4 << 20;   // 16 MB
+constexpr int kWsCounters = 8192;
+
 template <int MT, int NT, int kWaves, int kEpilogue, typename TO>
 static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                          const float* bias, int M, int N, int K, hipStream_t stream) {
   constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
-  constexpr int unroll = (MT >= 4) ? 2 : 4;   // many row tiles: fewer steps in flight, or registers run out
-  gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, unroll><<<(N + cols - 1) / cols, kWaves * 64, 0, stream>>>(
+  const int col_tiles = (N + cols - 1) / cols;
+  // split K across blocks while the column tiles alone leave most of the chip idle
+  int k_splits = 1;
+  if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr) {
+    const int steps = (K + 31) / 32;
+    while (k_splits < 8 && col_tiles * k_splits * 2 <= 512 && steps / (k_splits * 2) >= kWaves / 2) k_splits *= 2;
+    if (col_tiles > g_ws.n_counters || static_cast<int64_t>(col_tiles) * k_splits * MT * NT * 256 > g_ws.tile_floats) k_splits = 1;
+  }
+  // loads in flight: many for one row tile (latency is all there is), fewer as row tiles take the registers
+  constexpr int unroll = (MT >= 4) ? 2 : 4;
+  gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, unroll><<<dim3(col_tiles, k_splits), kWaves * 64, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
-      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K);
+      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, g_ws.tiles, g_ws.counters);
   return check_launch("gemm_skinny");
 }
 
@@ -170,6 +234,21 @@ static int dispatch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, c
 }  // namespace alofa
 
 using namespace alofa;
+
+// Allocates the workspace of the cross-block K split (once; later calls do nothing). Without it K
+// is split inside blocks only. Not to be called under graph capture.
+extern "C" int alofa_gemm_skinny_workspace_init() {
+  if (g_ws.tiles != nullptr) return 0;
+  void* tiles = nullptr;
+  void* counters = nullptr;
+  hipError_t e = hipExtMallocWithFlags(&tiles, kWsTileFloats * sizeof(float), hipDeviceMallocUncached);
+  if (e == hipSuccess) e = hipExtMallocWithFlags(&counters, kWsCounters * sizeof(int), hipDeviceMallocUncached);
+  if (e == hipSuccess) e = hipMemset(counters, 0, kWsCounters * sizeof(int));
+  if (e == hipSuccess) e = hipDeviceSynchronize();
+  ALOFA_REQUIRE(e == hipSuccess, "gemm_skinny_workspace_init: %s", hipGetErrorString(e));
+  g_ws = {static_cast<f32x4*>(tiles), kWsTileFloats, static_cast<int*>(counters), kWsCounters};
+  return 0;
+}
 
 // bfloat16 A [M, K] (M <= 64) and W [N, K] (W2 for the swiglu epilogue); K a multiple of 8,
 // rows 16-byte aligned. Epilogues: 0 store (+ bias) as o_dtype, 1 add to the float residual, 2 swiglu.
