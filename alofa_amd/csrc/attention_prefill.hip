@@ -32,7 +32,9 @@ constexpr int BQ = 64;    // query rows per block
 constexpr int BKV = 64;   // keys per tile
 constexpr int KPAD = 8, VPAD = 8;
 
-// tiles: int32 [n_tiles, 4] = (request index, first row in the packed batch, rows (<= 64), position of the first row)
+// tiles: int32 [n_blocks, 2, 4]: a block serves up to two runs of rows, one after the other, each
+// (request index, first row in the packed batch, rows (<= 64; 0: none), position of the first row). The caller
+// pairs long runs with short ones so that blocks carry about the same number of key tiles.
 template <int DT>  // DT = d / 16
 __global__ void __launch_bounds__(256) attention_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
@@ -47,10 +49,12 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
 
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int c16 = lane % 16, g = lane / 16;
-  // later tiles of a prompt see more keys: they are started first so that the short ones fill the tail
-  const int32_t* tile = tiles + 4 * (gridDim.x - 1 - blockIdx.x);
-  const int req = tile[0], row0 = tile[1], n_rows = tile[2], pos0 = tile[3];
   const int head = blockIdx.y, hk = head / (heads / kv_heads);
+  for (int part = 0; part < 2; ++part) {
+  const int32_t* tile = tiles + 8 * blockIdx.x + 4 * part;
+  const int req = tile[0], row0 = tile[1], n_rows = tile[2], pos0 = tile[3];
+  if (n_rows <= 0) break;     // uniform over the block
+  __syncthreads();            // the first run's last tile has been read by every wave
   const int32_t* table = block_table + static_cast<int64_t>(req) * max_blocks;
 
   // this lane's query row and its fragments of Q
@@ -107,10 +111,13 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
         const int key = c / (d / 8), ch = (c % (d / 8)) * 8;
         *reinterpret_cast<uint4*>(&Ks[key * KROW + ch]) = k_reg[j];
         const uint32_t w[4] = {v_reg[j].x, v_reg[j].y, v_reg[j].z, v_reg[j].w};
+        // rows ch..ch+7 of V^T; groups of four keys are permuted within a row by the row's
+        // chunk number, so that the lanes of a wave (eight chunks of the same keys) hit different banks
+        const int skey = key ^ (((ch >> 3) & 7) << 2);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          Vt[(ch + 2 * e) * VROW + key] = static_cast<bf16_t>(w[e] & 0xffffu);
-          Vt[(ch + 2 * e + 1) * VROW + key] = static_cast<bf16_t>(w[e] >> 16);
+          Vt[(ch + 2 * e) * VROW + skey] = static_cast<bf16_t>(w[e] & 0xffffu);
+          Vt[(ch + 2 * e + 1) * VROW + skey] = static_cast<bf16_t>(w[e] >> 16);
         }
       }
     }
@@ -183,10 +190,11 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
     for (int nt = 0; nt < DT; ++nt) {
       o[nt] *= corr;
       const bf16_t* vrow = &Vt[(nt * 16 + c16) * VROW];
+      const int sw = ((nt * 2 + (c16 >> 3)) & 7) << 2;   // this row's permutation of its four-key groups
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const uint2 lo = *reinterpret_cast<const uint2*>(vrow + half * 32 + g * 4);
-        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + half * 32 + 16 + g * 4);
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow + ((half * 32 + g * 4) ^ sw));
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + ((half * 32 + 16 + g * 4) ^ sw));
         const uint4 vv = make_uint4(lo.x, lo.y, hi.x, hi.y);
         o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf[half], o[nt], 0, 0, 0);
       }
@@ -206,6 +214,7 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
       *reinterpret_cast<uint2*>(dst + nt * 16 + g * 4) = w;
     }
   }
+  }  // runs of this block
 }
 
 }  // namespace alofa

@@ -80,20 +80,23 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  uint4 a_reg[NC], w_reg[NC];
-  auto fetch = [&](int k0) {
+  // PF slabs are on their way from memory while another is being multiplied: two for the small
+  // tiles (their loop is short and latency shows), one for the big ones (registers are scarcer)
+  constexpr int PF = (WT == 1) ? 2 : 1;
+  uint4 a_reg[PF][NC], w_reg[PF][NC];
+  auto fetch = [&](uint4 (&a)[NC], uint4 (&w)[NC], int k0) {
     const bool k_ok = k0 + c_k < K;
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-      a_reg[j] = (k_ok && a_ok[j]) ? *reinterpret_cast<const uint4*>(a_src[j] + k0) : make_uint4(0, 0, 0, 0);
-      w_reg[j] = (k_ok && w_ok[j]) ? *reinterpret_cast<const uint4*>(w_src[j] + k0) : make_uint4(0, 0, 0, 0);
+      a[j] = (k_ok && a_ok[j]) ? *reinterpret_cast<const uint4*>(a_src[j] + k0) : make_uint4(0, 0, 0, 0);
+      w[j] = (k_ok && w_ok[j]) ? *reinterpret_cast<const uint4*>(w_src[j] + k0) : make_uint4(0, 0, 0, 0);
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](const uint4 (&a)[NC], const uint4 (&w)[NC]) {
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-      *reinterpret_cast<uint4*>(&As[c_row[j] * kRow + c_k]) = a_reg[j];
-      *reinterpret_cast<uint4*>(&Ws[c_row[j] * kRow + c_k]) = w_reg[j];
+      *reinterpret_cast<uint4*>(&As[c_row[j] * kRow + c_k]) = a[j];
+      *reinterpret_cast<uint4*>(&Ws[c_row[j] * kRow + c_k]) = w[j];
     }
   };
 
@@ -106,13 +109,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
     // swiglu: tile 0 = gate rows of this wave's 32 columns, tile 1 = the up rows of the same columns
     w_off[i] = ((kEpilogue == kMfSwiglu) ? (i * 64 + wn * 32 + frag_row) : (wn * 32 * WT + i * 32 + frag_row)) * kRow + frag_k;
   }
-
-  fetch(0);
-  for (int k0 = 0; k0 < K; k0 += TK) {
-    __syncthreads();          // the previous slab has been read by every wave
-    stage();
-    __syncthreads();
-    if (k0 + TK < K) fetch(k0 + TK);
+  auto multiply = [&]() {
 #pragma unroll
     for (int ks = 0; ks < TK; ks += 16) {
       bf16x8 a[WT], w[WT];
@@ -125,6 +122,21 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
       for (int i = 0; i < WT; ++i)
 #pragma unroll
         for (int j = 0; j < WT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+#pragma unroll
+  for (int p = 0; p < PF; ++p) fetch(a_reg[p], w_reg[p], p * TK);
+  for (int k0 = 0; k0 < K; k0 += PF * TK) {
+#pragma unroll
+    for (int p = 0; p < PF; ++p) {
+      if (k0 + p * TK < K) {    // uniform over the block
+        __syncthreads();        // the previous slab has been read by every wave
+        stage(a_reg[p], w_reg[p]);
+        __syncthreads();
+        fetch(a_reg[p], w_reg[p], k0 + (p + PF) * TK);
+        multiply();
+      }
     }
   }
 

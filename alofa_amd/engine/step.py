@@ -13,6 +13,7 @@ from typing import Optional
 import numpy as np
 import torch
 
+from .. import ops
 from ..cache.manager import CacheManager
 from ..errors import AlofaError
 
@@ -220,7 +221,7 @@ class StepFunction:
         if ctx.n_short < T:
             tiles = [(i, s.row0 + q0, min(TILE_ROWS, s.n - q0), s.pos0 + q0)
                      for i, s in enumerate(spans) if s.n > SHORT for q0 in range(0, s.n, TILE_ROWS)]
-            ctx.long_tiles = torch.tensor(tiles, dtype=torch.int32, device=dev)
+            ctx.long_tiles = torch.tensor(ops.pair_tiles(tiles), dtype=torch.int32, device=dev)
             if ctx.n_short:
                 ctx.short_rows = torch.tensor([r for s in spans if s.n <= SHORT for r in range(s.row0, s.row0 + s.n)],
                                               dtype=torch.int32, device=dev)
@@ -298,7 +299,7 @@ class StepFunction:
                 logits = self.model.logits(ctx, hidden, buf["rows"])
                 torch.cuda.current_stream().synchronize()
                 graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
+                with torch.cuda.graph(graph), ops.stream_scope():
                     hidden = self.model.forward(ctx, buf["ids"])
                     captured = self.model.logits(ctx, hidden, buf["rows"])
                 if captured.data_ptr() != logits.data_ptr():
@@ -318,10 +319,11 @@ class StepFunction:
         """Run the step. Returns float32 logits [wanted, vocab] on the device in
         the order of the entries and of their ``want`` lists, or None when nothing
         is wanted. The buffer is re-used by the next step."""
-        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-            return self._run_decode_graph(entries)
-        ctx, ids, rows = self.begin(entries)
-        hidden = self.model.forward(ctx, ids)
-        logits = self.model.logits(ctx, hidden, rows) if rows is not None else None
-        self.finish(ctx)
-        return logits
+        with ops.stream_scope():
+            if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+                return self._run_decode_graph(entries)
+            ctx, ids, rows = self.begin(entries)
+            hidden = self.model.forward(ctx, ids)
+            logits = self.model.logits(ctx, hidden, rows) if rows is not None else None
+            self.finish(ctx)
+            return logits

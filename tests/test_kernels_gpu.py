@@ -256,7 +256,9 @@ def test_prefill_attention(heads, kv_heads, d, bs, window):
         row += n
     out = torch.zeros(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
     scale = float(np.float32(1) / np.sqrt(np.float32(d)))
-    ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(tiles, np.int32), torch.int32), heads, kv_heads, d, window, scale)
+    paired = ops().pair_tiles(tiles, window)
+    assert sorted(tuple(r) for b in paired for r in b if r[2]) == sorted(tiles) and len(paired) == (len(tiles) + 1) // 2
+    ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(paired, np.int32), torch.int32), heads, kv_heads, d, window, scale)
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(len(lens))])
     close(out, ref, BF16, "prefill attention")
 
@@ -268,7 +270,7 @@ def test_prefill_attention_far_key():
     out = torch.zeros(40, heads * d, device=DEV, dtype=torch.bfloat16)
     scale = float(np.float32(1) / np.sqrt(np.float32(d)))
     for window in (None, L - far, L - far - 1):
-        ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array([[0, 0, 40, L - 40]], np.int32), torch.int32),
+        ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array([[[0, 0, 40, L - 40], [0, 0, 0, 0]]], np.int32), torch.int32),
                                 heads, kv_heads, d, window, scale)
         close(out, pm.attention(c["q"][0], c["k"][0], c["v"][0], heads, kv_heads, d, window), BF16, f"far key, window {window}")
 
