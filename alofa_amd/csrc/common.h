@@ -70,6 +70,21 @@ __device__ __forceinline__ T block_sum(T v, T* scratch) {
   return total;
 }
 
+// ---- workspace ---------------------------------------------------------------
+// Scratch for kernels whose blocks hand partial results to one another (the K split of the
+// few-rows product): `tiles` for the partial results and zeroed counters, in uncached device memory, so that what one block wrote is what another
+// reads, whichever die they run on, without flushing caches. The library allocates it once
+// per process (alofa_workspace_init) and never frees it. Every kernel leaves its counters
+// zero. Kernels that use it must not overlap on one GPU (one stream at a time).
+struct Workspace {
+  float* tiles;
+  int64_t tile_floats;
+  int* counters;
+  int n_counters;
+};
+constexpr int kGemmCounters = 4096;   // counters the few-rows product may use
+const Workspace& workspace();
+
 // ---- error channel ---------------------------------------------------------
 
 void set_error(const char* fmt, ...);

@@ -15,8 +15,7 @@
 // arrives last adds the partial tiles in split order (not in arrival order, so
 // the sum is the same on every run), runs the epilogue and puts the counter
 // back to zero. Nobody waits for anybody. The workspace is uncached device
-// memory: what one block wrote is what another reads, whichever die they run
-// on, without flushing caches; fences only order the accesses within a block.
+// memory (common.h), so fences only have to order the accesses within a block.
 //
 // Operand layout of v_mfma_f32_16x16x32_bf16, lane l: A holds row l % 16,
 // B holds column l % 16, both the 8 reduction indices 8 * (l / 16) .. + 7 of
@@ -181,19 +180,6 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   }
 }
 
-// Workspace of the cross-block K split: partial tiles and one zeroed counter per column tile, in
-// uncached device memory that the library allocates once per process and never frees. Every call
-// leaves the counters zero. Calls that overlap on one GPU (two streams) would race on it.
-struct SkinnyWorkspace {
-  f32x4* tiles;
-  int64_t tile_floats;
-  int* counters;
-  int n_counters;
-};
-static SkinnyWorkspace g_ws = {nullptr, 0, nullptr, 0};
-constexpr int64_t kWsTileFloats = 4 << 20;   // 16 MB
-constexpr int kWsCounters = 8192;
-
 template <int MT, int NT, int kWaves, int kEpilogue, typename TO>
 static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                          const float* bias, int M, int N, int K, hipStream_t stream) {
@@ -201,16 +187,17 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
   const int col_tiles = (N + cols - 1) / cols;
   // split K across blocks while the column tiles alone leave most of the chip idle
   int k_splits = 1;
+  const Workspace& g_ws = workspace();
   if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr) {
     const int steps = (K + 31) / 32;
     while (k_splits < 8 && col_tiles * k_splits * 2 <= 512 && steps / (k_splits * 2) >= kWaves / 2) k_splits *= 2;
-    if (col_tiles > g_ws.n_counters || static_cast<int64_t>(col_tiles) * k_splits * MT * NT * 256 > g_ws.tile_floats) k_splits = 1;
+    if (col_tiles > kGemmCounters || static_cast<int64_t>(col_tiles) * k_splits * MT * NT * 256 > g_ws.tile_floats) k_splits = 1;
   }
   // loads in flight: many for one row tile (latency is all there is), fewer as row tiles take the registers
   constexpr int unroll = (MT >= 4) ? 2 : 4;
   gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, unroll><<<dim3(col_tiles, k_splits), kWaves * 64, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
-      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, g_ws.tiles, g_ws.counters);
+      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters);
   return check_launch("gemm_skinny");
 }
 
@@ -234,21 +221,6 @@ static int dispatch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, c
 }  // namespace alofa
 
 using namespace alofa;
-
-// Allocates the workspace of the cross-block K split (once; later calls do nothing). Without it K
-// is split inside blocks only. Not to be called under graph capture.
-extern "C" int alofa_gemm_skinny_workspace_init() {
-  if (g_ws.tiles != nullptr) return 0;
-  void* tiles = nullptr;
-  void* counters = nullptr;
-  hipError_t e = hipExtMallocWithFlags(&tiles, kWsTileFloats * sizeof(float), hipDeviceMallocUncached);
-  if (e == hipSuccess) e = hipExtMallocWithFlags(&counters, kWsCounters * sizeof(int), hipDeviceMallocUncached);
-  if (e == hipSuccess) e = hipMemset(counters, 0, kWsCounters * sizeof(int));
-  if (e == hipSuccess) e = hipDeviceSynchronize();
-  ALOFA_REQUIRE(e == hipSuccess, "gemm_skinny_workspace_init: %s", hipGetErrorString(e));
-  g_ws = {static_cast<f32x4*>(tiles), kWsTileFloats, static_cast<int*>(counters), kWsCounters};
-  return 0;
-}
 
 // bfloat16 A [M, K] (M <= 64) and W [N, K] (W2 for the swiglu epilogue); K a multiple of 8,
 // rows 16-byte aligned. Epilogues: 0 store (+ bias) as o_dtype, 1 add to the float residual, 2 swiglu.

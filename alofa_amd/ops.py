@@ -130,17 +130,17 @@ SKINNY_MAX_ROWS = 64
 SWIGLU = 2
 
 
-_skinny_workspace_ready = False
+_workspace_ready = False
 
 
-def _lend_skinny_workspace(device) -> None:
-    """Once per process: the library allocates the workspace of the skinny
-    kernel's K split across blocks. It is never moved, so captured graphs keep
-    valid pointers. One stream at a time may run these kernels."""
-    global _skinny_workspace_ready
-    if not _skinny_workspace_ready:
-        _call("alofa_gemm_skinny_workspace_init")
-        _skinny_workspace_ready = True
+def _ensure_workspace(device) -> None:
+    """Once per process: the library allocates its workspace (partial results that
+    blocks hand to one another). It is never moved, so captured graphs keep valid
+    pointers. One stream at a time may run the kernels that use it."""
+    global _workspace_ready
+    if not _workspace_ready:
+        _call("alofa_workspace_init")
+        _workspace_ready = True
 
 
 def _mfma_operands(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -169,7 +169,7 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
     if add_to_out and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the residual stream is float32", f"out={out.dtype}")
     if not exact and _mfma_operands(a, w):
-        _lend_skinny_workspace(a.device)
+        _ensure_workspace(a.device)
         # few rows: the weight-streaming kernel; many rows: the tiled one
         _call("alofa_gemm_skinny" if M <= SKINNY_MAX_ROWS else "alofa_gemm_mfma", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
               _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(None if add_to_out else bias), _I(M), _I(N), _I(K),
