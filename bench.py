@@ -20,7 +20,7 @@ sys.path.insert(0, str(ROOT))
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-# BASELINE.json configs[2]: Qwen2.5-0.5B layer sizes
+# Qwen2.5-0.5B layer sizes (the benchmark configuration)
 QWEN25_05B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 24, "hidden_size": 896,
     "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,

@@ -45,6 +45,14 @@ TINY = {
         "sliding_window": 40, "max_window_layers": 1,
         "max_position_embeddings": 512,
     },
+    # wider: head size 128, groups of four, a width the 128-wide tiles do not divide
+    "D": {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+        "num_hidden_layers": 2, "hidden_size": 1024, "num_attention_heads": 8,
+        "num_key_value_heads": 2, "intermediate_size": 2840, "vocab_size": 3001,
+        "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+        "use_sliding_window": False, "max_position_embeddings": 1024,
+    },
 }
 
 

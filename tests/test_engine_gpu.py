@@ -15,7 +15,7 @@ from helpers import (assert_close, bound, bulk_and_tail, collect, mixed, plain_l
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": 100, "B": 150, "C": 190}
+LENGTHS = {"A": 100, "B": 150, "C": 190, "D": 300}
 
 
 @pytest.fixture(scope="module")
@@ -102,6 +102,17 @@ def test_first_tokens_of_a_sequence(replayers, tiny_dirs, name, dtype):
     assert_close(collect(replayers(name, dtype), whole("f", ids[:1]))["f"], ref[:1], dtype, "one token")
     assert_close(collect(replayers(name, dtype), bulk_and_tail("g", ids, tail=4))["g"], ref, dtype, "token by token from the first")
     assert_close(collect(replayers(name, dtype), whole("h", ids[:2]))["h"], ref[:2], dtype, "two tokens")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_wider_model_in_every_cutting(replayers, tiny_dirs, dtype):
+    """Head size 128, four query heads per key head, 300 tokens: the large-tile kernels with ragged edges."""
+    ids = ids_of("D")
+    ref = plain_logits(tiny_dirs["D"], tuple(ids))
+    r = replayers("D", dtype, 1024)
+    assert_close(collect(r, whole("w", ids))["w"], ref, dtype, "D whole")
+    assert_close(collect(r, bulk_and_tail("t", ids))["t"], ref, dtype, "D bulk+tail")
+    assert_close(collect(r, portions("p", ids, sizes=(70, 2, 130, 9, 33, 2)))["p"], ref, dtype, "D portions")
 
 
 @pytest.mark.parametrize("block_size", [16, 32, 64])
