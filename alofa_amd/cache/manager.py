@@ -14,14 +14,20 @@ after the window has passed the block. Pages come back when a request ends and
 when a window has passed them, and the pool hands them out again at once.
 
 Beside the tables lies a slot per request for state of fixed size (one tensor
-per entry whose mixer asks for it), zeroed when the request is admitted."""
+per entry whose mixer asks for it), zeroed when the request is admitted.
+
+The counting is done by the C++ host runtime (csrc/host/host.cpp); this class
+is its face and owns the device tensors."""
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass
 from typing import Optional
 
+import numpy as np
 import torch
 
+from ..csrc import hostlib
 from ..errors import AlofaError
 from .pool import BlockPool
 
@@ -37,40 +43,36 @@ class Group:
     pool: BlockPool
 
 
-class _Request:
-    __slots__ = ("slot", "length", "tables", "first_held")
-
-    def __init__(self, slot: int, n_groups: int):
-        self.slot = slot
-        self.length = 0                              # tokens written so far
-        self.tables = [[] for _ in range(n_groups)]  # logical block -> physical or -1
-        self.first_held = [0] * n_groups             # lowest logical block still held
-
-
 class CacheManager:
-    """Host-side accounting (integers only) plus, when ``device`` is given, the
-    bytes: K and V per owning entry as [blocks, kv_heads, block_size, head_dim]
-    and one state tensor per entry that needs one."""
+    """Accounting (integers only, in the C++ host runtime) plus, when ``device``
+    is given, the bytes: K and V per owning entry as [blocks, kv_heads,
+    block_size, head_dim] and one state tensor per entry that needs one."""
 
     def __init__(self, cache_needs: list, state_needs: list, n_blocks: int, block_size: int = 16,
                  max_requests: int = 64, device=None, dtype=torch.bfloat16):
         if block_size <= 0 or max_requests <= 0:
             raise AlofaError("invalid_argument", "block_size and max_requests must be positive", f"block_size={block_size} max_requests={max_requests}")
+        if n_blocks <= 0:
+            raise AlofaError("invalid_argument", "a pool needs at least one block", f"n_blocks={n_blocks}")
         self.block_size = block_size
         self.max_requests = max_requests
-        self.groups: list = []
+        windows: list = []
+        entries: list = []
         self.group_of_entry: dict = {}
         for i, need in enumerate(cache_needs):
             if need is None:
                 continue
-            g = next((k for k, grp in enumerate(self.groups) if grp.window == need.window), None)
-            if g is None:
-                self.groups.append(Group(need.window, [], BlockPool(n_blocks)))
-                g = len(self.groups) - 1
-            self.groups[g].entries.append(i)
+            if need.window not in windows:
+                windows.append(need.window)
+                entries.append([])
+            g = windows.index(need.window)
+            entries[g].append(i)
             self.group_of_entry[i] = g
-        self.requests: dict = {}
-        self.free_slots = list(range(max_requests - 1, -1, -1))
+        self._lib = hostlib.lib()
+        self._h = ctypes.c_void_p(self._lib.alofa_cache_new(len(windows), hostlib.long_array([-1 if w is None else w for w in windows]),
+                                                             n_blocks, block_size, max_requests))
+        self.groups = [Group(w, entries[g], BlockPool(0, _borrowed=self._lib.alofa_cache_pool(self._h, g))) for g, w in enumerate(windows)]
+        self.requests: dict = {}      # request key -> its slot
         self.needs = list(cache_needs)
         self.state_needs = list(state_needs)
         self.k: dict = {}
@@ -87,15 +89,19 @@ class CacheManager:
                 if need is not None:
                     self.state[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
 
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self.groups = []
+            self._lib.alofa_cache_free(self._h)
+            self._h = None
+
     # ------------------------------------------------------------- requests
     def admit(self, req) -> int:
         """Take a request slot (the lowest free one) and zero its state."""
         if req in self.requests:
             raise AlofaError("invalid_argument", "duplicate request id", f"request={req}")
-        if not self.free_slots:
-            raise AlofaError("capacity", "no request slot is free", f"max_requests={self.max_requests}")
-        slot = self.free_slots.pop()
-        self.requests[req] = _Request(slot, len(self.groups))
+        slot = hostlib.check(self._lib.alofa_cache_admit(self._h))
+        self.requests[req] = slot
         for t in self.state.values():
             t[slot].zero_()
         return slot
@@ -103,121 +109,113 @@ class CacheManager:
     def has(self, req) -> bool:
         return req in self.requests
 
-    def _get(self, req) -> _Request:
+    def slot(self, req) -> int:
         if req not in self.requests:
             raise AlofaError("invalid_argument", "no such request", f"request={req}")
         return self.requests[req]
 
-    def length(self, req) -> int:
-        return self._get(req).length
+    @property
+    def free_slots(self) -> list:
+        """Only its length is meaningful: how many request slots are free."""
+        return [None] * self._lib.alofa_cache_n_free_slots(self._h)
 
-    def slot(self, req) -> int:
-        return self._get(req).slot
+    def length(self, req) -> int:
+        return hostlib.check(self._lib.alofa_cache_length(self._h, self.slot(req)))
 
     def blocks_needed(self, req, target: int) -> list:
         """New pages per group that growing ``req`` to ``target`` tokens takes."""
-        r = self._get(req)
-        return [max(0, blocks_for(target, self.block_size) - len(r.tables[g])) for g in range(len(self.groups))]
+        out = hostlib.int_array(len(self.groups))
+        hostlib.check(self._lib.alofa_cache_blocks_needed(self._h, self.slot(req), ctypes.c_int64(target), out))
+        return list(out)[:len(self.groups)]
 
     def reserve(self, req, target: int) -> None:
         """Hold pages for the positions up to ``target`` (exclusive) in every
         group. Either all pages are taken or none (capacity error)."""
-        r = self._get(req)
-        if target < r.length:
-            raise AlofaError("invalid_argument", "a request cannot shrink", f"request={req} length={r.length} target={target}")
-        need = self.blocks_needed(req, target)
-        for g, grp in enumerate(self.groups):
-            if need[g] > grp.pool.n_free:
-                raise AlofaError("capacity", "kv block pool is exhausted",
-                                 f"request={req} group={g} need={need[g]} free={grp.pool.n_free}")
-        for g, grp in enumerate(self.groups):
-            for _ in range(need[g]):
-                r.tables[g].append(grp.pool.alloc_one())
+        hostlib.check(self._lib.alofa_cache_reserve(self._h, self.slot(req), ctypes.c_int64(target)))
 
     def commit(self, req, target: int) -> list:
         """The tokens up to ``target`` are written. Pages that every later query
         has passed (window groups) go back to the pool; returns them per group."""
-        r = self._get(req)
-        if target < r.length or any(blocks_for(target, self.block_size) > len(t) for t in r.tables):
-            raise AlofaError("invalid_argument", "commit beyond what was reserved", f"request={req} length={r.length} target={target}")
-        r.length = target
-        freed = [[] for _ in self.groups]
-        for g, grp in enumerate(self.groups):
-            if grp.window is None:
-                continue
-            # the next query stands at position `target` and sees keys >= target - window + 1
-            first_needed = max(0, target - grp.window + 1) // self.block_size
-            for b in range(r.first_held[g], min(first_needed, len(r.tables[g]))):
-                if r.tables[g][b] >= 0:
-                    grp.pool.release(r.tables[g][b])
-                    freed[g].append(r.tables[g][b])
-                    r.tables[g][b] = -1
-            r.first_held[g] = max(r.first_held[g], min(first_needed, len(r.tables[g])))
-        return freed
+        G = len(self.groups)
+        cap = max(1, target // self.block_size + 2)
+        freed, counts = hostlib.int_array(G * cap), hostlib.int_array(G)
+        hostlib.check(self._lib.alofa_cache_commit(self._h, self.slot(req), ctypes.c_int64(target), freed, cap, counts))
+        return [[freed[g * cap + i] for i in range(counts[g])] for g in range(G)]
 
     def free(self, req) -> None:
         """The request ends: every page it holds and its state slot are given back."""
-        r = self._get(req)
-        for g, grp in enumerate(self.groups):
-            for b in r.tables[g]:
-                if b >= 0:
-                    grp.pool.release(b)
-        self.free_slots.append(r.slot)
+        hostlib.check(self._lib.alofa_cache_drop(self._h, self.slot(req)))
         del self.requests[req]
 
     def share_prefix(self, src, dst, n_tokens: int) -> int:
         """Let ``dst`` (fresh, empty) hold the whole blocks of ``src``'s first
         ``n_tokens`` tokens as well, by reference count; returns the tokens
-        shared. Only groups that keep every key can share."""
-        s, d = self._get(src), self._get(dst)
-        if d.length != 0 or any(d.tables[g] for g in range(len(self.groups))):
-            raise AlofaError("invalid_argument", "only an empty request can take a shared prefix", f"request={dst}")
-        if any(grp.window is not None for grp in self.groups) or any(n is not None for n in self.state_needs):
+        shared. Only groups that keep every key can share; state cannot be shared."""
+        if any(n is not None for n in self.state_needs):
             return 0
-        n_blocks = min(n_tokens, s.length) // self.block_size
-        for g, grp in enumerate(self.groups):
-            for b in s.tables[g][:n_blocks]:
-                grp.pool.retain(b)
-                d.tables[g].append(b)
-        d.length = n_blocks * self.block_size
-        return d.length
+        return hostlib.check(self._lib.alofa_cache_share_prefix(self._h, self.slot(src), self.slot(dst), ctypes.c_int64(n_tokens)))
 
     # ------------------------------------------------------------- lookups
     def table(self, req, group: int) -> list:
-        return self._get(req).tables[group]
+        n = hostlib.check(self._lib.alofa_cache_table_len(self._h, self.slot(req), group))
+        out = hostlib.int_array(n)
+        hostlib.check(self._lib.alofa_cache_table(self._h, self.slot(req), group, out, max(1, n)))
+        return list(out)[:n]
 
     def slots(self, req, group: int, start: int, n: int) -> list:
         """Physical slot (block * block_size + offset) of positions start..start+n-1."""
-        t = self._get(req).tables[group]
-        bs = self.block_size
-        out = []
-        for p in range(start, start + n):
-            b = t[p // bs] if p // bs < len(t) else -1
-            if b < 0:
-                raise AlofaError("capacity", "no page is held for this position", f"request={req} group={group} position={p}")
-            out.append(b * bs + p % bs)
-        return out
+        out = hostlib.long_array(n)
+        hostlib.check(self._lib.alofa_cache_slots(self._h, self.slot(req), group, ctypes.c_int64(start), n, out))
+        return list(out)[:n]
 
     def max_blocks(self) -> int:
-        return max((len(t) for r in self.requests.values() for t in r.tables), default=0)
+        return self._lib.alofa_cache_max_blocks(self._h)
+
+    # ------------------------------------------------------ steps, as arrays
+    def plan_step(self, slots: np.ndarray, n_tokens: np.ndarray, max_positions: int, width: Optional[int] = None):
+        """Lay one step out: entry i brings ``n_tokens[i]`` tokens of the request
+        in ``slots[i]``. Pages are taken for all entries or for none. Returns
+        (pos0 [n] int64, positions [T] int32, req_of_token [T] int32, tables
+        [groups, n, width] int32 with -1 where no page is held, row_slots
+        [groups, T] int64)."""
+        n = int(slots.shape[0])
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        n_tokens = np.ascontiguousarray(n_tokens, dtype=np.int32)
+        ip = ctypes.POINTER(ctypes.c_int)
+        if width is None:
+            width = hostlib.check(self._lib.alofa_cache_step_width(self._h, n, slots.ctypes.data_as(ip), n_tokens.ctypes.data_as(ip)))
+        T, G = int(n_tokens.sum()), len(self.groups)
+        pos0 = np.empty(n, dtype=np.int64)
+        positions = np.empty(T, dtype=np.int32)
+        req_of_token = np.empty(T, dtype=np.int32)
+        tables = np.empty((G, n, width), dtype=np.int32)
+        row_slots = np.empty((G, T), dtype=np.int64)
+        lp = ctypes.POINTER(ctypes.c_int64)
+        hostlib.check(self._lib.alofa_cache_plan_step(
+            self._h, n, slots.ctypes.data_as(ip), n_tokens.ctypes.data_as(ip), ctypes.c_int64(max_positions), width,
+            pos0.ctypes.data_as(lp), positions.ctypes.data_as(ip), req_of_token.ctypes.data_as(ip), tables.ctypes.data_as(ip),
+            row_slots.ctypes.data_as(lp), ctypes.c_int64(T)))
+        return pos0, positions, req_of_token, tables, row_slots
+
+    def plan_step_into(self, slots: np.ndarray, n_tokens: np.ndarray, max_positions: int, pos0: np.ndarray, positions: np.ndarray,
+                       req_of_token: np.ndarray, tables: np.ndarray, row_slots: np.ndarray) -> None:
+        """``plan_step`` into arrays the caller keeps (contiguous; tables [groups, n, width])."""
+        ip, lp = ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int64)
+        hostlib.check(self._lib.alofa_cache_plan_step(
+            self._h, int(slots.shape[0]), slots.ctypes.data_as(ip), n_tokens.ctypes.data_as(ip), ctypes.c_int64(max_positions),
+            int(tables.shape[2]), pos0.ctypes.data_as(lp), positions.ctypes.data_as(ip), req_of_token.ctypes.data_as(ip),
+            tables.ctypes.data_as(ip), row_slots.ctypes.data_as(lp), ctypes.c_int64(positions.shape[0])))
+
+    def commit_step(self, slots: np.ndarray, n_tokens: np.ndarray) -> None:
+        """The step's tokens are written: lengths advance, pages a window has passed go back."""
+        ip = ctypes.POINTER(ctypes.c_int)
+        hostlib.check(self._lib.alofa_cache_commit_step(self._h, int(slots.shape[0]), slots.ctypes.data_as(ip), n_tokens.ctypes.data_as(ip)))
 
     # ---------------------------------------------------------- invariants
     def check(self) -> None:
         """No page lost, held twice without a count, or freed twice: per group the
-        references in all tables equal the pool's counts, and free + used = all."""
-        for g, grp in enumerate(self.groups):
-            counts = [0] * grp.pool.n_blocks
-            for r in self.requests.values():
-                for b in r.tables[g]:
-                    if b >= 0:
-                        counts[b] += 1
-            if counts != grp.pool.refcnt:
-                raise AlofaError("invalid_argument", "tables and pool disagree on who holds which page", f"group={g}")
-            free = sorted(grp.pool.free_stack)
-            if len(set(free)) != len(free) or any(grp.pool.refcnt[b] != 0 for b in free):
-                raise AlofaError("double_free", "a page is on the free stack twice or while held", f"group={g}")
-            if len(free) + sum(1 for c in counts if c > 0) != grp.pool.n_blocks:
-                raise AlofaError("invalid_argument", "a page is neither free nor held", f"group={g}")
-        slots = [r.slot for r in self.requests.values()]
-        if len(set(slots)) != len(slots) or set(slots) & set(self.free_slots) or len(slots) + len(self.free_slots) != self.max_requests:
+        references in all tables equal the pool's counts, and free + used = all;
+        request slots are neither lost nor held twice."""
+        hostlib.check(self._lib.alofa_cache_check(self._h))
+        if len(set(self.requests.values())) != len(self.requests) or len(self.requests) + len(self.free_slots) != self.max_requests:
             raise AlofaError("invalid_argument", "request slots are lost or held twice")

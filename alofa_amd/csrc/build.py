@@ -1,5 +1,5 @@
 """Builds the HIP sources of this folder into one shared library for gfx950
-and loads it. The library's file name carries a hash of the sources and flags,
+and the C++ host runtime (host/) into another, and loads them. The library's file name carries a hash of the sources and flags,
 so a stale build is never loaded: when no file of the current hash exists, it
 is compiled at the first call (a line is printed for every file meanwhile)."""
 from __future__ import annotations
@@ -41,6 +41,75 @@ def _hash() -> str:
 
 def _lib_name() -> str:
     return f"libalofa_hip_{_hash()}.so"
+
+
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+_host = None
+
+
+def host_sources() -> list:
+    return sorted((HERE / "host").glob("*.cpp"))
+
+
+def _host_name() -> str:
+    h = hashlib.sha256(" ".join(HOST_FLAGS).encode())
+    for p in host_sources():
+        h.update(p.name.encode())
+        h.update(p.read_bytes())
+    return f"libalofa_host_{h.hexdigest()[:12]}.so"
+
+
+def find_built_host():
+    for d in _candidate_dirs():
+        if (d / _host_name()).is_file():
+            return d / _host_name()
+    return None
+
+
+def build_host(force: bool = False) -> Path:
+    """Compile the host runtime (plain C++, no GPU code) with the system compiler."""
+    if not force:
+        found = find_built_host()
+        if found:
+            return found
+    cxx = next((c for c in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++")) if c), None)
+    if cxx is None:
+        raise AlofaError("not_initialized", "no C++ compiler was found; the host runtime cannot be built")
+    target_dir = next((d for d in _candidate_dirs() if _writable(d)), None)
+    if target_dir is None:
+        raise AlofaError("io", "no writable folder for the built library", f"tried={[str(d) for d in _candidate_dirs()]}")
+    out = target_dir / _host_name()
+    tmp = target_dir / (out.name + f".tmp{os.getpid()}")
+    _say(f"compiling the host runtime into {target_dir}")
+    r = subprocess.run([cxx, *HOST_FLAGS, "-o", str(tmp), *map(str, host_sources())], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise AlofaError("io", "compiling the host runtime failed", r.stderr[-4000:])
+    os.replace(tmp, out)
+    for old in target_dir.glob("libalofa_host_*.so"):
+        if old != out:
+            try:
+                old.unlink()
+            except OSError:
+                pass
+    return out
+
+
+def load_host() -> ctypes.CDLL:
+    """The host runtime (pool, cache accounting, scheduler); built first when missing."""
+    global _host
+    if _host is None:
+        path = find_built_host() or build_host()
+        try:
+            _host = ctypes.CDLL(str(path))
+        except OSError as e:
+            raise AlofaError("not_initialized", "the host runtime cannot be loaded", f"path={path} reason={e}") from None
+        c = ctypes
+        _host.alofa_host_last_error.restype = c.c_char_p
+        for name in ("alofa_pool_new", "alofa_cache_new", "alofa_cache_pool", "alofa_sched_new"):
+            getattr(_host, name).restype = c.c_void_p
+        for name in ("alofa_cache_length", "alofa_sched_scalar"):
+            getattr(_host, name).restype = c.c_int64
+    return _host
 
 
 def _candidate_dirs() -> list:

@@ -75,6 +75,7 @@ class StepContext:
         self.n_short = sum(s.n for s in spans if s.n <= SHORT)
         self.short_rows: Optional[torch.Tensor] = None
         self.long_tiles: Optional[torch.Tensor] = None
+        self.entry_slots = self.entry_tokens = None   # request slot and token count per entry, as arrays
         self.positions: torch.Tensor = None
         self.req_of_token: torch.Tensor = None
         self._tables: list = []
@@ -149,28 +150,29 @@ class StepFunction:
 
     # ----------------------------------------------------------------- run
     def plan(self, entries: list):
-        """Check a batch and lay out its rows (host only, nothing is changed)."""
+        """Check a batch (host only, nothing is changed). Returns (request slots, tokens per
+        entry, all token ids) as arrays."""
         if not entries:
             raise AlofaError("invalid_argument", "a step needs at least one entry")
         vocab = self.model.spec.vocab_size
-        spans, seen, row = [], set(), 0
-        for e in entries:
-            if e.request in seen:
-                raise AlofaError("invalid_argument", "a request appears twice in one step", f"request={e.request}")
-            seen.add(e.request)
-            n = len(e.tokens)
-            if n == 0:
-                raise AlofaError("invalid_argument", "an entry brings no tokens", f"request={e.request}")
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise AlofaError("out_of_range", "token id outside the vocabulary", f"request={e.request} token={t} vocab={vocab}")
+        n_tokens = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=len(entries))
+        if n_tokens.min() <= 0:
+            raise AlofaError("invalid_argument", "an entry brings no tokens", f"request={entries[int(n_tokens.argmin())].request}")
+        slots = np.fromiter((self.cache.slot(e.request) for e in entries), dtype=np.int32, count=len(entries))
+        ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=int(n_tokens.sum()))
+        if ids.min() < 0 or ids.max() >= vocab:
+            raise AlofaError("out_of_range", "token id outside the vocabulary", f"vocab={vocab} min={ids.min()} max={ids.max()}")
+        for e, n in zip(entries, n_tokens):
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise AlofaError("out_of_range", "wanted place outside the entry's tokens", f"request={e.request} want={w} tokens={n}")
-            pos0 = self.cache.length(e.request)
-            if pos0 + n > self.n_positions:
-                raise AlofaError("capacity", "the request would pass the context bound", f"request={e.request} length={pos0 + n} bound={self.n_positions}")
-            spans.append(Span(e.request, self.cache.slot(e.request), row, n, pos0))
+        return slots, n_tokens, ids.astype(np.int32)
+
+    @staticmethod
+    def _spans(entries: list, slots, n_tokens, pos0) -> list:
+        spans, row = [], 0
+        for e, slot, n, p in zip(entries, slots.tolist(), n_tokens.tolist(), pos0.tolist()):
+            spans.append(Span(e.request, slot, row, n, p))
             row += n
         return spans
 
@@ -178,43 +180,21 @@ class StepFunction:
         """Take the pages the entries need and lay the step out on the device.
         Returns (context, token ids [T] int32, wanted rows or None). Either every
         entry gets its pages or nothing is changed (capacity error)."""
-        spans = self.plan(entries)
+        slots, n_tokens, ids = self.plan(entries)
         cache = self.cache
-        need = [0] * len(cache.groups)
-        for s in spans:
-            for g, n in enumerate(cache.blocks_needed(s.request, s.pos0 + s.n)):
-                need[g] += n
-        for g, grp in enumerate(cache.groups):
-            if need[g] > grp.pool.n_free:
-                raise AlofaError("capacity", "kv block pool is exhausted", f"group={g} need={need[g]} free={grp.pool.n_free}")
-        for s in spans:
-            cache.reserve(s.request, s.pos0 + s.n)
-        T = sum(s.n for s in spans)
-        ids = np.empty(T, dtype=np.int32)
-        positions = np.empty(T, dtype=np.int32)
-        req_of_token = np.empty(T, dtype=np.int32)
-        want_rows = []
-        for i, (e, s) in enumerate(zip(entries, spans)):
-            ids[s.row0:s.row0 + s.n] = np.asarray(e.tokens, dtype=np.int32)
-            positions[s.row0:s.row0 + s.n] = np.arange(s.pos0, s.pos0 + s.n, dtype=np.int32)
-            req_of_token[s.row0:s.row0 + s.n] = i
-            want_rows.extend(s.row0 + int(w) for w in e.want)
+        pos0, positions, req_of_token, tables, row_slots = cache.plan_step(slots, n_tokens, self.n_positions)
+        spans = self._spans(entries, slots, n_tokens, pos0)
+        T = int(positions.shape[0])
+        want_rows = [s.row0 + int(w) for e, s in zip(entries, spans) for w in e.want]
         ctx = StepContext(self, spans, positions)
-        max_blocks = max(1, cache.max_blocks())
+        ctx.entry_slots, ctx.entry_tokens = slots, n_tokens
         n_groups = len(cache.groups)
-        tables = np.full((n_groups, len(spans), max_blocks), -1, dtype=np.int32)
-        slots = np.empty((n_groups, T), dtype=np.int64)
-        for g in range(n_groups):
-            for i, s in enumerate(spans):
-                t = cache.table(s.request, g)
-                tables[g, i, :len(t)] = t
-                slots[g, s.row0:s.row0 + s.n] = cache.slots(s.request, g, s.pos0, s.n)
         dev = self.device
         ids_d = torch.from_numpy(ids).to(dev)
         ctx.positions = torch.from_numpy(positions).to(dev)
         ctx.req_of_token = torch.from_numpy(req_of_token).to(dev)
         tables_d = torch.from_numpy(tables).to(dev)
-        slots_d = torch.from_numpy(slots).to(dev)
+        slots_d = torch.from_numpy(row_slots).to(dev)
         ctx._tables = [tables_d[g] for g in range(n_groups)]
         ctx._slots = [slots_d[g] for g in range(n_groups)]
         rows = torch.tensor(want_rows, dtype=torch.int32, device=dev) if want_rows else None
@@ -230,8 +210,7 @@ class StepFunction:
     def finish(self, ctx: StepContext) -> None:
         """The step's tokens are written: lengths advance and pages that a window
         has passed go back to the pool."""
-        for s in ctx.spans:
-            self.cache.commit(s.request, s.pos0 + s.n)
+        self.cache.commit_step(ctx.entry_slots, ctx.entry_tokens)
         self.steps_run += 1
         self.rows_run += ctx.tokens
 
@@ -260,30 +239,18 @@ class StepFunction:
         return self._graph_buffers[B]
 
     def _run_decode_graph(self, entries: list) -> torch.Tensor:
-        spans = self.plan(entries)
+        slots, n_tokens, ids = self.plan(entries)
         cache = self.cache
-        need = [0] * len(cache.groups)
-        for s in spans:
-            for g, n in enumerate(cache.blocks_needed(s.request, s.pos0 + 1)):
-                need[g] += n
-        for g, grp in enumerate(cache.groups):
-            if need[g] > grp.pool.n_free:
-                raise AlofaError("capacity", "kv block pool is exhausted", f"group={g} need={need[g]} free={grp.pool.n_free}")
-        for s in spans:
-            cache.reserve(s.request, s.pos0 + 1)
-        B = len(spans)
+        B = len(entries)
         buf = self._decode_buffers(B)
         buf["copied"].synchronize()                      # the last copy out of the host block is done
-        buf["h_tables"].fill(-1)
-        for i, (e, s) in enumerate(zip(entries, spans)):
-            buf["h_ids"][i] = e.tokens[0]
-            buf["h_pos"][i] = s.pos0
-            for g in range(len(cache.groups)):
-                t = cache.table(s.request, g)
-                buf["h_tables"][g, i, :len(t)] = t
-                buf["h_slots"][g, i] = cache.slots(s.request, g, s.pos0, 1)[0]
-        positions = buf["h_pos"].copy()
-        ctx = StepContext(self, spans, positions)
+        pos0 = np.empty(B, dtype=np.int64)
+        # the layout goes straight into the pinned block that is copied to the device in one piece
+        cache.plan_step_into(slots, n_tokens, self.n_positions, pos0, buf["h_pos"], buf["h_req"], buf["h_tables"], buf["h_slots"])
+        buf["h_ids"][:] = ids
+        spans = self._spans(entries, slots, n_tokens, pos0)
+        ctx = StepContext(self, spans, buf["h_pos"].copy())
+        ctx.entry_slots, ctx.entry_tokens = slots, n_tokens
         ctx.positions, ctx.req_of_token = buf["positions"], buf["req_of_token"]
         ctx._tables = [buf["tables"][g] for g in range(len(cache.groups))]
         ctx._slots = [buf["slots"][g] for g in range(len(cache.groups))]
