@@ -15,7 +15,8 @@
 // arrives last adds the partial tiles in split order (not in arrival order, so
 // the sum is the same on every run), runs the epilogue and puts the counter
 // back to zero. Nobody waits for anybody. The workspace is uncached device
-// memory (common.h), so fences only have to order the accesses within a block.
+// memory (common.h): a block's partial tiles are in memory once its stores have
+// been acknowledged, which every wave waits for before the block is counted.
 //
 // Operand layout of v_mfma_f32_16x16x32_bf16, lane l: A holds row l % 16,
 // B holds column l % 16, both the 8 reduction indices 8 * (l / 16) .. + 7 of
@@ -29,6 +30,14 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum SkinnyEpilogue : int { kSkStore = 0, kSkResidual = 1, kSkSwiglu = 2 };
 
+
+// A partial sum leaves for the workspace at device scope: written through to memory, past this
+// die's L2, where blocks on every die find it.
+__device__ __forceinline__ void store_partial(f32x4* p, f32x4 v) {
+  float* f = reinterpret_cast<float*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) __hip_atomic_store(f + i, v[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ bf16x8 load_frag(const bf16_t* __restrict__ p, bool ok) {
   uint4 v = make_uint4(0, 0, 0, 0);
@@ -126,9 +135,13 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
       f32x4 sum = red[0][tile][lane];
 #pragma unroll
       for (int w = 1; w < kWaves; ++w) sum += red[w][tile][lane];
-      mine[tile * 64 + lane] = sum;
+      store_partial(mine + tile * 64 + lane, sum);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // this wave's tiles have left before the block is counted
+    // Every wave waits until its partial sums have been performed in memory; only then may the
+    // block be counted. A release fence of workgroup scope does not wait for stores to memory (the
+    // counter could overtake them), and one of device scope would write this die's whole L2 back.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (threadIdx.x == 0) {
       const int arrived = atomicAdd(&counters[blockIdx.x], 1);

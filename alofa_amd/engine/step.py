@@ -108,6 +108,8 @@ class StepFunction:
         self.n_positions = int(n_positions)
         self.device = model.rt.device
         self._scratch: dict = {}
+        self._eager_scratch = self._scratch      # buffers of steps that run kernel by kernel
+        self._retired: list = []                 # outgrown buffers that captured graphs may still use
         self._identity: dict = {}
         self.cache_entry = [i if e.cache_of is None else e.cache_of for i, e in enumerate(model.order)]
         needs = model.cache_needs()
@@ -137,6 +139,11 @@ class StepFunction:
         key = (name, dtype)
         buf = self._scratch.get(key)
         if buf is None or buf.numel() < n:
+            if buf is not None and self._scratch is not self._eager_scratch:
+                # a captured graph may hold this buffer's address (graphs of one batch size share
+                # buffers, and a longer context needs more room for attention's partial results):
+                # it is kept for good, so that replays of the older graph write where nothing else lives
+                self._retired.append(buf)
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._scratch[key] = buf
         return buf[:n].view(shape)

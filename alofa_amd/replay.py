@@ -35,8 +35,9 @@ class Replayer:
         n_blocks = max(1, (int(max_tokens) + block_size - 1) // block_size)
         self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), n_blocks, block_size,
                                   max_requests=8, device=self.model.rt.device, dtype=self.model.rt.dtype)
-        self.fn = StepFunction(self.model, self.cache,
-                               n_positions=min(self.model.spec.max_positions, max(int(max_tokens), 64)))
+        # the position table is as long as a request can get here, not the checkpoint's
+        # max_position_embeddings, which the reference does not read (qwen.mojo:849)
+        self.fn = StepFunction(self.model, self.cache, n_positions=max(int(max_tokens), 64))
 
     def step(self, rec: dict):
         """Run one step record; returns float32 logits [wanted, vocab] as a NumPy

@@ -53,6 +53,15 @@ TINY = {
         "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
         "use_sliding_window": False, "max_position_embeddings": 1024,
     },
+    # one wide head (size 144: nine lanes share a key in decoding, no tiled prefill kernel), an odd
+    # feed-forward width; decoding needs partial results whose room grows with the context
+    "E": {
+        "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+        "num_hidden_layers": 3, "hidden_size": 144, "num_attention_heads": 1,
+        "num_key_value_heads": 1, "intermediate_size": 57, "vocab_size": 903,
+        "rope_theta": 500000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+        "use_sliding_window": False, "max_position_embeddings": 64,
+    },
 }
 
 

@@ -15,7 +15,7 @@ from helpers import (assert_close, bound, bulk_and_tail, collect, mixed, plain_l
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": 100, "B": 150, "C": 190, "D": 300}
+LENGTHS = {"A": 100, "B": 150, "C": 190, "D": 300, "E": 160}
 
 
 @pytest.fixture(scope="module")
@@ -68,7 +68,7 @@ def test_portions_of_changing_size(replayers, tiny_dirs, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "E"])
 def test_mixed_requests_with_pages_used_again(tiny_dirs, name, dtype):
     from alofa_amd.replay import Replayer
     vocab, top = TINY[name]["vocab_size"], LENGTHS[name]
@@ -113,6 +113,51 @@ def test_wider_model_in_every_cutting(replayers, tiny_dirs, dtype):
     assert_close(collect(r, whole("w", ids))["w"], ref, dtype, "D whole")
     assert_close(collect(r, bulk_and_tail("t", ids))["t"], ref, dtype, "D bulk+tail")
     assert_close(collect(r, portions("p", ids, sizes=(70, 2, 130, 9, 33, 2)))["p"], ref, dtype, "D portions")
+
+
+def random_config(rnd):
+    """A Qwen2 configuration drawn at random: head sizes in steps of 16 up to 256, any head and
+    group counts, widths and vocabularies that are no powers of two, windows on some layers."""
+    kv = int(rnd.choice([1, 1, 2, 3, 4]))
+    heads = kv * int(rnd.choice([1, 2, 3, 4, 5, 7, 8]))
+    d = int(rnd.choice([16, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 256]))
+    if heads * d > 1536:
+        d = int(rnd.choice([16, 32, 48]))
+    layers = int(rnd.integers(1, 4))
+    cfg = dict(architectures=["Qwen2ForCausalLM"], num_hidden_layers=layers, hidden_size=heads * d, num_attention_heads=heads,
+               num_key_value_heads=kv, intermediate_size=int(rnd.choice([int(rnd.integers(8, 600)), 8 * int(rnd.integers(2, 80))])),
+               vocab_size=int(rnd.integers(50, 1500)), rms_norm_eps=float(rnd.choice([1e-6, 1e-5, 3e-4])),
+               rope_theta=float(rnd.choice([1e4, 1e6, 5e5])), tie_word_embeddings=bool(rnd.random() < 0.5),
+               max_position_embeddings=512)
+    if rnd.random() < 0.4:
+        cfg.update(use_sliding_window=True, sliding_window=int(rnd.integers(8, 90)), max_window_layers=int(rnd.integers(0, layers)))
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at random, mixed requests and decoding one by one, in both dtypes.
+    (Such a sweep found a captured graph that kept a freed buffer and a counter that overtook
+    the partial sums it counted.)"""
+    from alofa_amd.replay import Replayer
+    from alofa_amd.weights import write_random_model
+    rnd = np.random.default_rng(7000 + seed)
+    cfg = random_config(rnd)
+    write_random_model(cfg, tmp_path, seed=seed)
+    top = int(rnd.integers(70, 200))
+    requests = {f"r{i}": random_ids(100 + i, n, cfg["vocab_size"]) for i, n in enumerate([top, 41, max(34, top - 37), 64, 35])}
+    ref = {k: plain_logits(tmp_path, tuple(v)) for k, v in requests.items()}
+    what = " ".join(f"{k}={v}" for k, v in cfg.items() if k != "architectures")
+    for dtype in DTYPES:
+        steps, peak = mixed(requests, seed=seed)
+        r = Replayer(tmp_path, dtype, peak)
+        got = collect(r, steps)
+        r.cache.check()
+        for k in requests:
+            assert_close(got[k], ref[k], dtype, f"[{what}] {dtype} mixed {k}")
+        r = Replayer(tmp_path, dtype, 256)
+        assert_close(collect(r, bulk_and_tail("x", requests["r0"]))["x"], ref["r0"], dtype, f"[{what}] {dtype} bulk+tail")
+        assert_close(collect(r, portions("y", requests["r0"]))["y"], ref["r0"], dtype, f"[{what}] {dtype} portions")
 
 
 @pytest.mark.parametrize("block_size", [16, 32, 64])

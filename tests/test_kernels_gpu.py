@@ -108,6 +108,28 @@ def test_gemm_bf16(M, N, K):
     close(outw, pm.linear(a, w32, b), BF16, "f32 weight")
 
 
+def test_gemm_split_over_blocks_is_repeatable():
+    """Few rows and few columns: K is split over blocks that hand partial sums to the last one
+    to arrive. The additions are in a fixed order, so every run gives the same bits; a partial
+    sum that was not yet in memory when it was read would show as a difference. Two products
+    of different shapes alternate, so that what the workspace held before is never the answer."""
+    rng = np.random.default_rng(40)
+    cases = []
+    for M, N, K in [(3, 1082, 672), (3, 864, 672), (5, 672, 288), (2, 144, 2048)]:
+        a = t(bf(rng.standard_normal((M, K)).astype(np.float32)), torch.bfloat16)
+        w = t(bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1), torch.bfloat16)
+        out = torch.empty(M, N, device=DEV)
+        ops().gemm(out, a, w)
+        cases.append((a, w, out, out.clone()))
+        close(out, pm.linear(a.float().cpu().numpy(), w.float().cpu().numpy()), 1e-4, f"{M}x{N}x{K}")
+    differing = torch.zeros((), dtype=torch.int64, device=DEV)
+    for _ in range(1500):
+        for a, w, out, first in cases:
+            ops().gemm(out, a, w)
+            differing += (out != first).sum()
+    assert int(differing) == 0
+
+
 def test_gemm_takes_a_strided_view():
     rng = np.random.default_rng(4)
     big = rng.standard_normal((6, 300)).astype(np.float32)
