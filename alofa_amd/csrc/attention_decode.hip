@@ -190,11 +190,16 @@ __global__ void __launch_bounds__(64) attention_merge_kernel(bf16_t* __restrict_
   const float big = wave_max(m);
   const float e = __expf(m - big);
   const float total = wave_sum(l * e);
-  for (int c = lane; c < d; c += 64) {
+  // every lane takes part in every round, so that the weights can be read from all 64 lanes
+  for (int c0 = 0; c0 < d; c0 += 64) {
+    const int c = c0 + lane;
     float acc = 0.f;
 #pragma unroll 8
-    for (int s = 0; s < n_splits; ++s) acc += src[s * (d + 2) + 2 + c] * __shfl(e, s, 64);
-    store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
+    for (int s = 0; s < n_splits; ++s) {
+      const float w = __shfl(e, s, 64);
+      if (c < d) acc += src[s * (d + 2) + 2 + c] * w;
+    }
+    if (c < d) store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
   }
 }
 

@@ -95,6 +95,29 @@ def test_long_decoding(replayers, tiny_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_long_context(tiny_dirs, name, dtype):
+    """2,300 tokens: many key tiles per query tile in the prompt, then decoding whose keys are
+    shared out among many splits; a second request joins for the decoding."""
+    from alofa_amd.replay import Replayer
+    vocab = TINY[name]["vocab_size"]
+    ids, other = random_ids(21, 2300, vocab), random_ids(22, 700, vocab)
+    ref, ref_other = plain_logits(tiny_dirs[name], tuple(ids)), plain_logits(tiny_dirs[name], tuple(other))
+    r = Replayer(tiny_dirs[name], dtype, round64(2300) + round64(700))
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ids[:1500], "want": list(range(1500))}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": ids[1500:2268], "want": list(range(768))},
+                                     {"id": "b", "tokens": other[:690], "want": list(range(690))}], "end": []}]
+    for i in range(32):
+        entries = [{"id": "a", "tokens": [ids[2268 + i]], "want": [0]}]
+        if i < 10:
+            entries.append({"id": "b", "tokens": [other[690 + i]], "want": [0]})
+        steps.append({"step": 2 + i, "entries": entries, "end": ["b"] if i == 9 else []})
+    got = collect(r, steps)
+    assert_close(got["a"], ref, dtype, f"{name} long a")
+    assert_close(got["b"], ref_other, dtype, f"{name} long b")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_first_tokens_of_a_sequence(replayers, tiny_dirs, name, dtype):
     ids = ids_of(name, seed=9, n=5)

@@ -264,6 +264,26 @@ def test_decode_attention(heads, kv_heads, d, bs, window):
                               max_q_len=4, max_context=700)
 
 
+@pytest.mark.parametrize("heads,kv_heads,d", [(5, 1, 80), (2, 2, 96), (3, 1, 64)])
+def test_decode_attention_with_many_splits(heads, kv_heads, d):
+    """One token over 5,000 keys: the keys are shared out among 64 splits, and all of them count
+    (head sizes between 64 and 128 combine channels 64.. in a second round of the lanes)."""
+    rng = np.random.default_rng(18)
+    lens, q_lens = [5000, 3000], [1, 2]
+    c = paged_case(rng, lens, q_lens, heads, kv_heads, d, 16, torch.bfloat16)
+    out = torch.empty(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    o = ops()
+    assert o.decode_splits(sum(q_lens), kv_heads, d, 8192) == 64
+    scratch = torch.empty(o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, 8192, None), device=DEV)
+    o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, None, scale, False,
+                      max_q_len=2, max_context=8192, scratch=scratch)
+    ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, None) for r in range(2)])
+    # random keys give almost even weights, so the result is small: compare at its own scale
+    err = np.abs(out.float().cpu().numpy() - ref).max()
+    assert err <= 1e-2 * np.abs(ref).max(), f"{err} vs {np.abs(ref).max()}"
+
+
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 96, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (3, 1, 32, 64)])
 @pytest.mark.parametrize("window", [None, 21, 300])
 def test_prefill_attention(heads, kv_heads, d, bs, window):
