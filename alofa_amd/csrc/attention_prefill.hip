@@ -1,11 +1,13 @@
 // Paged causal grouped-query attention for prompt portions, bfloat16 on MFMA,
 // with a running softmax so that no score matrix is ever stored.
 //
-// A block of four wavefronts serves 64 consecutive query rows of one request
-// and one query head; every wave owns 16 rows. The visible keys are walked in
-// tiles of 64 that start at absolute multiples of 64, so the order of additions
-// for a row is the same however the prompt was cut into steps. Per tile the
-// block stages the keys [64, d] and the values transposed [d, 64] in LDS.
+// A block serves 64 consecutive query rows of one request and one query head
+// with TEAMS teams of four wavefronts; within a team every wave owns 16 rows.
+// The visible keys are walked in tiles of 64 that start at absolute multiples
+// of 64; the teams take the tiles in turn (a row's chain of dependent tiles is
+// TEAMS times shorter, and the teams' waves fill one another's stalls) and
+// their running states meet in LDS at the end, combined in team order. Per
+// tile a team stages the keys [64, d] and the values transposed [d, 64] in LDS.
 //
 // Both products are taken transposed, so that one lane's data stays with one
 // query row throughout (v_mfma_f32_16x16x32_bf16; lane l: A row and B column
@@ -35,8 +37,8 @@ constexpr int KPAD = 8, VPAD = 8;
 // tiles: int32 [n_blocks, 2, 4]: a block serves up to two runs of rows, one after the other, each
 // (request index, first row in the packed batch, rows (<= 64; 0: none), position of the first row). The caller
 // pairs long runs with short ones so that blocks carry about the same number of key tiles.
-template <int DT>  // DT = d / 16
-__global__ void __launch_bounds__(256) attention_prefill_kernel(
+template <int DT, int TEAMS>  // DT = d / 16
+__global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
     int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int bs_shift, int window,
@@ -44,10 +46,16 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
   constexpr int d = DT * 16;
   constexpr int DS = (d + 31) / 32;           // steps of 32 along d in the first product
   constexpr int KROW = d + KPAD, VROW = BKV + VPAD;
-  __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * KROW];
-  __shared__ __attribute__((aligned(16))) bf16_t Vt[d * VROW];
+  // per team: its key tile and its transposed value tile; at the end the same room takes the team's
+  // running state (per lane its maximum, its sum and its 4 * DT channels)
+  constexpr int kStageBytes = (BKV * KROW + d * VROW) * 2, kStateBytes = 256 * (4 * DT + 2) * 4;
+  constexpr int kTeamBytes = ((kStageBytes > kStateBytes ? kStageBytes : kStateBytes) + 15) / 16 * 16;
+  __shared__ __attribute__((aligned(16))) char team_room[TEAMS * kTeamBytes];
+  const int team = threadIdx.x / 256;
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(team_room + team * kTeamBytes);
+  bf16_t* Vt = Ks + BKV * KROW;
 
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int tid = threadIdx.x % 256, wave = tid / 64, lane = tid % 64;
   const int c16 = lane % 16, g = lane / 16;
   const int head = blockIdx.y, hk = head / (heads / kv_heads);
   for (int part = 0; part < 2; ++part) {
@@ -123,12 +131,15 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
     }
   };
 
-  fetch(t_begin);
-  for (int t = t_begin; t <= t_end; ++t) {
+  if (t_begin + team <= t_end) fetch(t_begin + team);
+  for (int t0 = t_begin; t0 <= t_end; t0 += TEAMS) {     // uniform over the block
+    const int t = t0 + team;
+    const bool mine = t <= t_end;
     __syncthreads();      // the previous tile has been read by every wave
-    stage();
+    if (mine) stage();
     __syncthreads();
-    if (t < t_end) fetch(t + 1);
+    if (!mine) continue;
+    if (t + TEAMS <= t_end) fetch(t + TEAMS);
 
     // S^T for the four 16-key quarters of the tile
     f32x4 s[4];
@@ -203,7 +214,36 @@ __global__ void __launch_bounds__(256) attention_prefill_kernel(
 
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
-  if (row_ok) {
+  if (TEAMS > 1) {
+    // the other teams leave their states where their tiles were; team 0 adds them in team order
+    __syncthreads();      // every tile has been read
+    float* state = reinterpret_cast<float*>(team_room + team * kTeamBytes) + tid * (4 * DT + 2);
+    if (team > 0) {
+      state[0] = m;
+      state[1] = l;
+#pragma unroll
+      for (int nt = 0; nt < DT; ++nt) *reinterpret_cast<f32x4*>(state + 2 + 4 * nt) = o[nt];
+    }
+    __syncthreads();
+    if (team == 0) {
+      float big = m;
+#pragma unroll
+      for (int k = 1; k < TEAMS; ++k) big = fmaxf(big, state[k * (kTeamBytes / 4)]);
+      const float e0 = __builtin_amdgcn_exp2f(m - big);
+      l *= e0;
+#pragma unroll
+      for (int nt = 0; nt < DT; ++nt) o[nt] *= e0;
+#pragma unroll
+      for (int k = 1; k < TEAMS; ++k) {
+        const float* other = state + k * (kTeamBytes / 4);
+        const float e = __builtin_amdgcn_exp2f(other[0] - big);
+        l += other[1] * e;
+#pragma unroll
+        for (int nt = 0; nt < DT; ++nt) o[nt] += *reinterpret_cast<const f32x4*>(other + 2 + 4 * nt) * e;
+      }
+    }
+  }
+  if (row_ok && team == 0) {
     const float inv = 1.f / l;
     bf16_t* dst = out + static_cast<int64_t>(row0 + my_row) * out_stride + static_cast<int64_t>(head) * d;
 #pragma unroll
@@ -239,8 +279,9 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
   ALOFA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
                 "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
   dim3 grid(n_tiles, heads);
+  // teams per block: as many as the registers and LDS of a compute unit hold at this head size
 #define ALOFA_PREFILL(DT)                                                                                                 \
-  attention_prefill_kernel<DT><<<grid, 256, 0, stream>>>(                                                                 \
+  attention_prefill_kernel<DT, (DT <= 4 ? 4 : DT <= 8 ? 2 : 1)><<<grid, 256 * (DT <= 4 ? 4 : DT <= 8 ? 2 : 1), 0, stream>>>( \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
       static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
   switch (d / 16) {
