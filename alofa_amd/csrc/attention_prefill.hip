@@ -175,8 +175,7 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
         tile_max = fmaxf(tile_max, p[i]);
       }
     }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    tile_max = rows_max(tile_max);     // over the four lanes that share the query row
     const float m_new = fmaxf(m, tile_max);
     const float corr = __builtin_amdgcn_exp2f(m - m_new);    // 1 while nothing was seen yet (both -FLT_MAX)
     m = m_new;
@@ -212,8 +211,7 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
     }
   }
 
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
+  l = rows_sum(l);
   if (TEAMS > 1) {
     // the other teams leave their states where their tiles were; team 0 adds them in team order
     __syncthreads();      // every tile has been read

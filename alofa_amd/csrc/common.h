@@ -40,18 +40,81 @@ template <> __device__ __forceinline__ void store_f32<float>(float* p, float v) 
 template <> __device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
 // ---- reductions ------------------------------------------------------------
+// Sums and maxima over the 64 lanes of a wavefront ride on data-parallel-primitive moves between
+// neighbouring lanes (no trip through LDS): a scan within each row of 16 lanes (shifts by 1, 2, 4, 8),
+// then row 0's total into row 1 and row 2's into row 3, then the lower half's total into the upper half;
+// lane 63 holds the result, which every lane reads. The order of the additions is fixed.
+
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ float dpp_move(float identity, float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(__float_as_uint(identity), __float_as_uint(v), kCtrl, kRowMask, 0xf, false));
+}
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ double dpp_move(double identity, double v) {
+  const uint64_t i = __builtin_bit_cast(uint64_t, identity), x = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = __builtin_amdgcn_update_dpp(static_cast<uint32_t>(i), static_cast<uint32_t>(x), kCtrl, kRowMask, 0xf, false);
+  const uint32_t hi = __builtin_amdgcn_update_dpp(static_cast<uint32_t>(i >> 32), static_cast<uint32_t>(x >> 32), kCtrl, kRowMask, 0xf, false);
+  return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
+}
+__device__ __forceinline__ float read_lane(float v, int lane) {
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
+}
+__device__ __forceinline__ double read_lane(double v, int lane) {
+  const uint64_t x = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = __builtin_amdgcn_readlane(static_cast<uint32_t>(x), lane), hi = __builtin_amdgcn_readlane(static_cast<uint32_t>(x >> 32), lane);
+  return __builtin_bit_cast(double, (static_cast<uint64_t>(hi) << 32) | lo);
+}
+
+constexpr int kRowShr1 = 0x111, kRowShr2 = 0x112, kRowShr4 = 0x114, kRowShr8 = 0x118, kRowBcast15 = 0x142, kRowBcast31 = 0x143;
 
 template <typename T>
 __device__ __forceinline__ T wave_sum(T v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+  v += dpp_move<kRowShr1, 0xf>(T(0), v);
+  v += dpp_move<kRowShr2, 0xf>(T(0), v);
+  v += dpp_move<kRowShr4, 0xf>(T(0), v);
+  v += dpp_move<kRowShr8, 0xf>(T(0), v);
+  v += dpp_move<kRowBcast15, 0xa>(T(0), v);
+  v += dpp_move<kRowBcast31, 0xc>(T(0), v);
+  return read_lane(v, 63);
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+  constexpr float lowest = -3.402823466e+38f;
+  v = fmaxf(v, dpp_move<kRowShr1, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<kRowShr2, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<kRowShr4, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<kRowShr8, 0xf>(lowest, v));
+  v = fmaxf(v, dpp_move<kRowBcast15, 0xa>(lowest, v));
+  v = fmaxf(v, dpp_move<kRowBcast31, 0xc>(lowest, v));
+  return read_lane(v, 63);
+}
+
+// The four lanes l, l ^ 16, l ^ 32, l ^ 48 (one of each row of 16) meet: the rows are swapped in pairs,
+// then the halves of the wavefront, by the lane-swap instructions; every lane gets the result.
+__device__ __forceinline__ float rows_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// v of lane l ^ 1, l ^ 2 (within a quad of lanes) and l ^ 8 (within a row of 16), without LDS
+__device__ __forceinline__ float lane_xor1(float v) { return dpp_move<0xB1, 0xf>(0.f, v); }   // quad_perm [1,0,3,2]
+__device__ __forceinline__ float lane_xor2(float v) { return dpp_move<0x4E, 0xf>(0.f, v); }   // quad_perm [2,3,0,1]
+__device__ __forceinline__ float lane_xor8(float v) { return dpp_move<0x128, 0xf>(0.f, v); }  // row_ror:8
+
+// What this wavefront's lanes wrote to LDS is seen by its other lanes afterwards (LDS serves a
+// wavefront's accesses in program order; the fences keep the compiler from moving them).
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // Sum over a block of kThreads (a multiple of 64) in a fixed tree, so the

@@ -253,13 +253,18 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
 DECODE_MAX_Q = 4          # requests with at most this many query tokens use the decode kernel
 
 
+def decode_waves(d: int) -> int:
+    """Waves of a decode attention block; each takes a share of the keys (the kernel's own rule)."""
+    return 8 if d <= 128 else 4
+
+
 def decode_splits(tokens: int, kv_heads: int, d: int, max_context: int) -> int:
-    """Shares of the keys per (token, key head): enough waves to fill the chip,
-    but at least eight rounds of keys each."""
+    """Parts the keys of a (token, key head) are cut into beyond the waves of a block: none while a
+    wave has at most about eight rounds of keys; more for long contexts, while the chip has room."""
     keys_per_round = 64 // (d // 16)
-    by_chip = -(-2048 // max(1, tokens * kv_heads))
-    by_length = max(1, max_context // (8 * keys_per_round))
-    return max(1, min(64, by_chip, by_length))
+    by_length = -(-max_context // (keys_per_round * decode_waves(d) * 8))
+    by_chip = max(1, 1024 // max(1, tokens * kv_heads))
+    return max(1, min(64, by_length, by_chip))
 
 
 def decode_scratch_floats(tokens: int, heads: int, kv_heads: int, d: int, max_context: int, window: Optional[int]) -> int:

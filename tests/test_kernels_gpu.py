@@ -236,48 +236,52 @@ def test_paged_attention(heads, kv_heads, d, bs, dtype, exact, window):
 
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 80, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (18, 2, 32, 64)])
 @pytest.mark.parametrize("window", [None, 21, 300])
-def test_decode_attention(heads, kv_heads, d, bs, window):
+@pytest.mark.parametrize("bucket", [700, 8192])
+def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
     """The kernel for few query tokens per request: single tokens and short
-    portions, contexts from one key to many pages (several splits), groups of
-    1 to 9 heads per key head, head sizes whose lanes-per-key is no power of two."""
+    portions, contexts from one key to many pages, groups of 1 to 9 heads per
+    key head, head sizes whose lanes-per-key is no power of two. ``bucket`` is the
+    context bound the launch is shaped for: the waves of one block share the keys
+    out, and for the larger bound several blocks do, whose states a second kernel combines."""
     rng = np.random.default_rng(17)
     lens, q_lens = [1, 37, 700, 64, 333], [1, 2, 1, 4, 3]
     c = paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16)
     out = torch.empty(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
     scale = float(np.float32(1) / np.sqrt(np.float32(d)))
     o = ops()
-    scratch = torch.empty(max(1, o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, 700, window)), device=DEV)
+    scratch = torch.empty(max(1, o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, bucket, window)), device=DEV)
     o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, False,
-                      max_q_len=4, max_context=700, scratch=scratch)
+                      max_q_len=4, max_context=bucket, scratch=scratch)
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(5)])
     close(out, ref, BF16, "decode attention")
     if (heads, d, window) == (14, 64, None):
-        assert o.decode_splits(sum(q_lens), kv_heads, d, 700) == 5                       # several splits are really in play
-    one = torch.empty(1, heads * d, device=DEV, dtype=torch.bfloat16)        # one split, one token
+        assert o.decode_splits(sum(q_lens), kv_heads, d, bucket) == (1 if bucket == 700 else 8)   # several parts are really in play
+    one = torch.empty(1, heads * d, device=DEV, dtype=torch.bfloat16)        # one token that sees one key
     o.paged_attention(one, c["qcat"][:1], c["kc"], c["vc"], c["table"], c["req"][:1], c["pos"][:1], heads, kv_heads, d, window, scale, False,
                       max_q_len=1, max_context=1)
     close(one, ref[:1], BF16, "decode attention, first token")
-    if o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, 700, window):
+    if o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, bucket, window):
         from alofa_amd.errors import AlofaError
         with pytest.raises(AlofaError):                                          # needed scratch is demanded, not allocated behind the back
             o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, False,
-                              max_q_len=4, max_context=700)
+                              max_q_len=4, max_context=bucket)
 
 
 @pytest.mark.parametrize("heads,kv_heads,d", [(5, 1, 80), (2, 2, 96), (3, 1, 64)])
 def test_decode_attention_with_many_splits(heads, kv_heads, d):
-    """One token over 5,000 keys: the keys are shared out among 64 splits, and all of them count
-    (head sizes between 64 and 128 combine channels 64.. in a second round of the lanes)."""
+    """One token over 5,000 keys, the launch shaped for a far longer context: the keys are shared out
+    among 64 parts, and all of them count (head sizes between 64 and 128 combine channels 64.. in a
+    second round of the lanes)."""
     rng = np.random.default_rng(18)
     lens, q_lens = [5000, 3000], [1, 2]
     c = paged_case(rng, lens, q_lens, heads, kv_heads, d, 16, torch.bfloat16)
     out = torch.empty(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
     scale = float(np.float32(1) / np.sqrt(np.float32(d)))
     o = ops()
-    assert o.decode_splits(sum(q_lens), kv_heads, d, 8192) == 64
-    scratch = torch.empty(o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, 8192, None), device=DEV)
+    assert o.decode_splits(sum(q_lens), kv_heads, d, 65536) == 64
+    scratch = torch.empty(o.decode_scratch_floats(sum(q_lens), heads, kv_heads, d, 65536, None), device=DEV)
     o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, None, scale, False,
-                      max_q_len=2, max_context=8192, scratch=scratch)
+                      max_q_len=2, max_context=65536, scratch=scratch)
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, None) for r in range(2)])
     # random keys give almost even weights, so the result is small: compare at its own scale
     err = np.abs(out.float().cpu().numpy() - ref).max()
