@@ -258,18 +258,22 @@ def decode_waves(d: int) -> int:
     return 8 if d <= 128 else 4
 
 
-def decode_splits(tokens: int, kv_heads: int, d: int, max_context: int) -> int:
-    """Parts the keys of a (token, key head) are cut into beyond the waves of a block: none while a
-    wave has at most about eight rounds of keys; more for long contexts, while the chip has room."""
-    keys_per_round = 64 // (d // 16)
-    by_length = -(-max_context // (keys_per_round * decode_waves(d) * 8))
-    by_chip = max(1, 1024 // max(1, tokens * kv_heads))
+def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
+    """Parts the keys of a (token, key head) are cut into beyond the waves of a block. None while a
+    wave has at most eight rounds of keys. Longer contexts: down to about four rounds a wave, but
+    only until the blocks fill the chip (a block's fixed cost is paid once per part)."""
+    keys_per_round, waves = 64 // (d // 16), decode_waves(d)
+    if max_context <= keys_per_round * waves * 8:
+        return 1
+    blocks = tokens * kv_heads * -(-(heads // kv_heads) // 4)
+    by_length = -(-max_context // (keys_per_round * waves * 4))
+    by_chip = max(1, 256 // max(1, blocks))
     return max(1, min(64, by_length, by_chip))
 
 
 def decode_scratch_floats(tokens: int, heads: int, kv_heads: int, d: int, max_context: int, window: Optional[int]) -> int:
     """Floats of scratch the decode kernel needs for these sizes (0: none)."""
-    n = decode_splits(tokens, kv_heads, d, min(max_context, window or max_context))
+    n = decode_splits(tokens, heads, kv_heads, d, min(max_context, window or max_context))
     return tokens * heads * n * (d + 2) if n > 1 else 0
 
 
@@ -340,7 +344,7 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     if rows is not None:
         _gpu("rows", rows, torch.int32, 1), _contig("rows", rows)
         n_tok = rows.shape[0]
-    n_splits = decode_splits(n_tok, kv_heads, d, min(max_context, window or max_context))
+    n_splits = decode_splits(n_tok, heads, kv_heads, d, min(max_context, window or max_context))
     floats = n_tok * heads * n_splits * (d + 2) if n_splits > 1 else 0
     if floats and (scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous()):
         raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")
