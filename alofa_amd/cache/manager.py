@@ -45,8 +45,9 @@ class Group:
 
 class CacheManager:
     """Accounting (integers only, in the C++ host runtime) plus, when ``device``
-    is given, the bytes: K and V per owning entry as [blocks, kv_heads,
-    block_size, head_dim] and one state tensor per entry that needs one."""
+    is given, the bytes: per owning entry K as [blocks, kv_heads, block_size,
+    head_dim] and V transposed as [blocks, kv_heads, head_dim, block_size], and
+    one state tensor per entry that needs one."""
 
     def __init__(self, cache_needs: list, state_needs: list, n_blocks: int, block_size: int = 16,
                  max_requests: int = 64, device=None, dtype=torch.bfloat16):
@@ -82,9 +83,10 @@ class CacheManager:
         if device is not None:
             for i, need in enumerate(cache_needs):
                 if need is not None:
-                    shape = (n_blocks, need.kv_heads, block_size, need.head_dim)
-                    self.k[i] = torch.zeros(shape, dtype=dtype, device=device)
-                    self.v[i] = torch.zeros(shape, dtype=dtype, device=device)
+                    # values lie transposed, [channel][slot]: consecutive keys of a channel are contiguous,
+                    # the order in which the matrix cores reduce over keys
+                    self.k[i] = torch.zeros((n_blocks, need.kv_heads, block_size, need.head_dim), dtype=dtype, device=device)
+                    self.v[i] = torch.zeros((n_blocks, need.kv_heads, need.head_dim, block_size), dtype=dtype, device=device)
             for i, need in enumerate(state_needs):
                 if need is not None:
                     self.state[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)

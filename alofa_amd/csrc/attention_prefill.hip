@@ -20,7 +20,8 @@
 // the same order, so the weights never leave their registers.
 // Scores, the running maximum, the weights and their sum are float; the
 // weights are rounded to bfloat16 only as MFMA operands.
-// Cache layout: [block, kv_head, slot_in_block, d].
+// Cache layout: keys [block, kv_head, slot_in_block, d], values transposed [block, kv_head, d, slot_in_block]:
+// eight consecutive keys of a channel are one 16-byte load, staged as they are.
 #include "common.h"
 
 #include <float.h>
@@ -90,7 +91,7 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
   const int first_key = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
   const int t_begin = first_key / BKV, t_end = last_pos / BKV;     // inclusive
 
-  // staging: chunks of 8 channels; the block moves 32 * d / 8 chunks of K and of V per tile
+  // staging: 16-byte chunks, 64 * d / 8 of K (eight channels of a key) and as many of V^T (eight keys of a channel)
   constexpr int kChunks = BKV * d / 8;
   constexpr int kPerThread = (kChunks + 255) / 256;
   uint4 k_reg[kPerThread], v_reg[kPerThread];
@@ -106,7 +107,23 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
           const int64_t blk = table[key >> bs_shift];
           const int64_t base = ((((blk * kv_heads + hk) << bs_shift) + (key & ((1 << bs_shift) - 1))) * d) + ch;
           k_reg[j] = *reinterpret_cast<const uint4*>(k_cache + base);
-          v_reg[j] = *reinterpret_cast<const uint4*>(v_cache + base);
+        }
+        // keys key0 .. key0 + 7 of channel c / 8 (one page: pages hold at least eight tokens)
+        const int key0 = t * BKV + (c % 8) * 8, channel = c / 8;
+        if (key0 <= last_pos && key0 + 7 >= first_key) {
+          const int64_t blk = table[key0 >> bs_shift];
+          const int64_t base = (((blk * kv_heads + hk) * d + channel) << bs_shift) + (key0 & ((1 << bs_shift) - 1));
+          uint4 v = *reinterpret_cast<const uint4*>(v_cache + base);
+          // what lies beyond the visible keys is not data: it is cleared, so that a weight of zero times it is zero
+          const int lo_e = first_key - key0, hi_e = last_pos - key0 + 1;   // elements lo_e .. hi_e - 1 are visible
+          if (lo_e > 0 || hi_e < 8) {
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (e < lo_e || e >= hi_e) w[e / 2] &= (e % 2) ? 0x0000ffffu : 0xffff0000u;
+            v = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+          v_reg[j] = v;
         }
       }
     }
@@ -118,15 +135,12 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
       if (c < kChunks) {
         const int key = c / (d / 8), ch = (c % (d / 8)) * 8;
         *reinterpret_cast<uint4*>(&Ks[key * KROW + ch]) = k_reg[j];
-        const uint32_t w[4] = {v_reg[j].x, v_reg[j].y, v_reg[j].z, v_reg[j].w};
-        // rows ch..ch+7 of V^T; groups of four keys are permuted within a row by the row's
-        // chunk number, so that the lanes of a wave (eight chunks of the same keys) hit different banks
-        const int skey = key ^ (((ch >> 3) & 7) << 2);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          Vt[(ch + 2 * e) * VROW + skey] = static_cast<bf16_t>(w[e] & 0xffffu);
-          Vt[(ch + 2 * e + 1) * VROW + skey] = static_cast<bf16_t>(w[e] >> 16);
-        }
+        // row c / 8 of V^T, keys 8 (c % 8) .. + 7. Groups of four keys are permuted within a row by the row's
+        // number / 8, so that lanes reading rows r and r + 8 hit different banks: the two groups of this chunk
+        // stay in their 16 bytes and change places when that number is odd.
+        const int sw = ((c / 8) >> 3) & 7;
+        const uint4 v = (sw & 1) ? make_uint4(v_reg[j].z, v_reg[j].w, v_reg[j].x, v_reg[j].y) : v_reg[j];
+        *reinterpret_cast<uint4*>(&Vt[(c / 8) * VROW + ((((c % 8) * 2) ^ (sw & 6)) << 2)]) = v;
       }
     }
   };
@@ -270,8 +284,8 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
   ALOFA_REQUIRE(n_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_prefill: tiles=%d heads=%d kv_heads=%d (kv_heads must divide heads)", n_tiles, heads, kv_heads);
   ALOFA_REQUIRE(alofa_attention_prefill_supports(d), "attention_prefill: head size %d is not built (16, 32, 48, 64, 96, 128, 256 are)", d);
-  ALOFA_REQUIRE(block_size > 0 && (block_size & (block_size - 1)) == 0 && max_blocks > 0 && window >= 0,
-                "attention_prefill: block_size=%d must be a power of two; max_blocks=%d window=%d", block_size, max_blocks, window);
+  ALOFA_REQUIRE(block_size >= 8 && (block_size & (block_size - 1)) == 0 && max_blocks > 0 && window >= 0,
+                "attention_prefill: block_size=%d must be a power of two, at least 8; max_blocks=%d window=%d", block_size, max_blocks, window);
   int bs_shift = 0;
   while ((1 << bs_shift) < block_size) ++bs_shift;
   ALOFA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,

@@ -9,7 +9,7 @@
 // Acc in ascending key order per channel, and divided once at the end. The
 // order depends only on the key's position, so a row's result is the same
 // however the tokens were cut into steps and whichever pages hold them.
-// Cache layout: [block, kv_head, slot_in_block, d].
+// Cache layout: keys [block, kv_head, slot_in_block, d], values transposed [block, kv_head, d, slot_in_block].
 #include "common.h"
 
 #include <float.h>
@@ -65,11 +65,11 @@ __global__ void __launch_bounds__(64) attention_simple_kernel(
       z += e;
       const int jk = j0 + jj;
       const int64_t blk = table[jk / block_size];
-      const T* v = v_cache + ((blk * kv_heads + hk) * block_size + (jk % block_size)) * static_cast<int64_t>(d);
+      const T* v = v_cache + (blk * kv_heads + hk) * static_cast<int64_t>(d) * block_size + (jk % block_size);
 #pragma unroll
       for (int i = 0; i < kMaxHeadDim / kWave; ++i) {
         const int c = lane + i * kWave;
-        if (c < d) o[i] += e * static_cast<Acc>(load_f32(v + c));
+        if (c < d) o[i] += e * static_cast<Acc>(load_f32(v + static_cast<int64_t>(c) * block_size));
       }
     }
     __syncthreads();

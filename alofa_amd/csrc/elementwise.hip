@@ -47,7 +47,8 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(TO* __restrict__ out, cons
 // half-split pairing (j, j + d/2); queries are rotated in place, rotated keys
 // and plain values go to the token's cache slot. Products and the sum are
 // separate float operations (no fused multiply-add), as in a plain loop.
-// Cache layout: [block, kv_head, slot_in_block, d].
+// Cache layout: keys [block, kv_head, slot_in_block, d], values transposed [block, kv_head, d, slot_in_block]
+// (consecutive keys of one channel are contiguous: the order in which the matrix cores reduce over keys).
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t,
                                      const float* __restrict__ sin_t, const int32_t* __restrict__ positions,
@@ -85,7 +86,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, co
     const T* v = row + static_cast<int64_t>(heads + kv_heads) * d;
     for (int i = threadIdx.x; i < kv_heads * d; i += blockDim.x) {
       const int hk = i / d, c = i % d;
-      v_cache[((blk * kv_heads + hk) * block_size + off) * d + c] = v[i];
+      v_cache[((blk * kv_heads + hk) * d + c) * block_size + off] = v[i];      // values lie transposed: [channel][slot]
     }
   }
 }

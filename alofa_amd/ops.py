@@ -207,12 +207,23 @@ def swiglu(out: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, exact: bool 
 
 # ----------------------------------------------------- positions + cache write
 
-def check_cache(name: str, cache: torch.Tensor, kv_heads: int, d: int) -> int:
-    """A cache is [blocks, kv_heads, block_size, d], contiguous. Returns block_size."""
+def check_cache(name: str, cache: torch.Tensor, kv_heads: int, d: int, transposed: bool = False) -> int:
+    """A key cache is [blocks, kv_heads, block_size, d]; a value cache is transposed,
+    [blocks, kv_heads, d, block_size]. Contiguous. Returns block_size."""
     _gpu(name, cache, None, 4), _contig(name, cache)
-    if cache.shape[1] != kv_heads or cache.shape[3] != d:
+    want_d, bs = (cache.shape[2], cache.shape[3]) if transposed else (cache.shape[3], cache.shape[2])
+    if cache.shape[1] != kv_heads or want_d != d:
         raise AlofaError("shape_mismatch", "cache does not fit the heads", f"{name}={tuple(cache.shape)} kv_heads={kv_heads} d={d}")
-    return cache.shape[2]
+    return bs
+
+
+def check_caches(k_cache: torch.Tensor, v_cache: torch.Tensor, kv_heads: int, d: int) -> int:
+    """Key cache and (transposed) value cache of one layer; returns block_size."""
+    bs = check_cache("k_cache", k_cache, kv_heads, d)
+    if check_cache("v_cache", v_cache, kv_heads, d, transposed=True) != bs or k_cache.shape[0] != v_cache.shape[0] or k_cache.dtype is not v_cache.dtype:
+        raise AlofaError("shape_mismatch", "key and value caches must agree in blocks, block size and dtype",
+                         f"k_cache={tuple(k_cache.shape)} v_cache={tuple(v_cache.shape)}")
+    return bs
 
 
 def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
@@ -237,10 +248,9 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
         raise AlofaError("shape_mismatch", "one position per token", f"positions={tuple(positions.shape)} T={T}")
     bs = 0
     if write:
-        bs = check_cache("k_cache", k_cache, kv_heads, d)
-        check_cache("v_cache", v_cache, kv_heads, d)
-        if k_cache.shape != v_cache.shape or k_cache.dtype is not qkv.dtype or v_cache.dtype is not qkv.dtype:
-            raise AlofaError("shape_mismatch", "key and value caches must agree with each other and with qkv's dtype")
+        bs = check_caches(k_cache, v_cache, kv_heads, d)
+        if k_cache.dtype is not qkv.dtype:
+            raise AlofaError("shape_mismatch", "the caches must have qkv's dtype")
         _gpu("slots", slots, torch.int64, 1), _contig("slots", slots)
         if slots.shape[0] != T:
             raise AlofaError("shape_mismatch", "one cache slot per token", f"slots={tuple(slots.shape)} T={T}")
@@ -251,6 +261,7 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, posit
 # ----------------------------------------------------------------- attention
 
 DECODE_MAX_Q = 4          # requests with at most this many query tokens use the decode kernel
+MIN_FAST_PAGE = 8         # the bfloat16 attention kernels load eight keys of a value channel at once
 
 
 def decode_waves(d: int) -> int:
@@ -260,13 +271,13 @@ def decode_waves(d: int) -> int:
 
 def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
     """Parts the keys of a (token, key head) are cut into beyond the waves of a block. None while a
-    wave has at most eight rounds of keys. Longer contexts: down to about four rounds a wave, but
+    wave has at most eight steps of 32 keys. Longer contexts: down to about four steps a wave, but
     only until the blocks fill the chip (a block's fixed cost is paid once per part)."""
-    keys_per_round, waves = 64 // (d // 16), decode_waves(d)
-    if max_context <= keys_per_round * waves * 8:
+    waves = decode_waves(d)
+    if max_context <= 32 * waves * 8:
         return 1
-    blocks = tokens * kv_heads * -(-(heads // kv_heads) // 4)
-    by_length = -(-max_context // (keys_per_round * waves * 4))
+    blocks = tokens * kv_heads * -(-(heads // kv_heads) // 16)
+    by_length = -(-max_context // (32 * waves * 4))
     by_chip = max(1, 256 // max(1, blocks))
     return max(1, min(64, by_length, by_chip))
 
@@ -293,17 +304,16 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         raise AlofaError("shape_mismatch", "attention rows do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} heads={heads} d={d}")
     if d % 2 or d > MAX_HEAD_DIM or d <= 0:
         raise AlofaError("unsupported", f"head size must be even and at most {MAX_HEAD_DIM}", f"head_dim={d}")
-    bs = check_cache("k_cache", k_cache, kv_heads, d)
-    check_cache("v_cache", v_cache, kv_heads, d)
-    if k_cache.shape != v_cache.shape or k_cache.dtype is not q.dtype or v_cache.dtype is not q.dtype:
-        raise AlofaError("shape_mismatch", "caches must agree with each other and with q's dtype")
+    bs = check_caches(k_cache, v_cache, kv_heads, d)
+    if k_cache.dtype is not q.dtype:
+        raise AlofaError("shape_mismatch", "the caches must have q's dtype")
     _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
     _gpu("req_of_token", req_of_token, torch.int32, 1), _contig("req_of_token", req_of_token)
     _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
     if req_of_token.shape[0] != T or positions.shape[0] != T:
         raise AlofaError("shape_mismatch", "one request index and one position per token")
     if (not exact and q.dtype is torch.bfloat16 and max_q_len is not None and max_q_len <= DECODE_MAX_Q and d % 16 == 0
-            and _rows("q", q) % 8 == 0 and q.data_ptr() % 16 == 0 and bs & (bs - 1) == 0):
+            and _rows("q", q) % 8 == 0 and q.data_ptr() % 16 == 0 and bs >= MIN_FAST_PAGE and bs & (bs - 1) == 0):
         attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
                          max_context or 1 << 30, scratch)
         return
@@ -319,12 +329,11 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
         raise AlofaError("shape_mismatch", "attention rows do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} heads={heads} d={d}")
     if d % 16 or not 16 <= d <= MAX_HEAD_DIM or kv_heads <= 0 or heads % kv_heads:
         raise AlofaError("unsupported", "head size 16..256 in steps of 16, kv_heads dividing heads", f"head_dim={d} heads={heads} kv_heads={kv_heads}")
-    bs = check_cache("k_cache", k_cache, kv_heads, d)
-    check_cache("v_cache", v_cache, kv_heads, d)
-    if k_cache.shape != v_cache.shape or k_cache.dtype is not torch.bfloat16 or v_cache.dtype is not torch.bfloat16:
-        raise AlofaError("shape_mismatch", "caches must agree with each other and be bfloat16")
-    if bs & (bs - 1):
-        raise AlofaError("unsupported", "the bfloat16 attention kernels take pages of a power of two of tokens", f"block_size={bs}")
+    bs = check_caches(k_cache, v_cache, kv_heads, d)
+    if k_cache.dtype is not torch.bfloat16:
+        raise AlofaError("shape_mismatch", "the caches must be bfloat16")
+    if bs < MIN_FAST_PAGE or bs & (bs - 1):
+        raise AlofaError("unsupported", f"the bfloat16 attention kernels take pages of a power of two of tokens, at least {MIN_FAST_PAGE}", f"block_size={bs}")
     _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
     if _rows("q", q) % 8 or q.data_ptr() % 16 or _rows("out", out) % 4 or out.data_ptr() % 8:
         raise AlofaError("alignment", "attention rows must be 16-byte aligned", f"q_stride={_rows('q', q)} out_stride={_rows('out', out)}")

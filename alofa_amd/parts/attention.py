@@ -86,7 +86,7 @@ class GQAAttention(Mixer):
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
         attn = ctx.scratch("attn", (T, self.heads * self.d), self.rt.dtype)
         common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
-        pow2_pages = kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
+        pow2_pages = kv.k.shape[2] >= ops.MIN_FAST_PAGE and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
         fast_prefill = self.d in ops.PREFILL_HEAD_DIMS
         if exact or not pow2_pages or (ctx.long_tiles is not None and not fast_prefill):
             # the exact path, and page or head sizes the bfloat16 kernels are not built for

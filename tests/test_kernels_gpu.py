@@ -169,14 +169,14 @@ def test_rope_and_cache_write(heads, kv_heads, d, bs, dtype):
     slots = rng.permutation(n_blocks * bs)[:T]
     dev = t(qkv, dtype)
     kc = torch.full((n_blocks, kv_heads, bs, d), 7.0, device=DEV, dtype=dtype)
-    vc = torch.full((n_blocks, kv_heads, bs, d), 7.0, device=DEV, dtype=dtype)
+    vc = torch.full((n_blocks, kv_heads, d, bs), 7.0, device=DEV, dtype=dtype)       # values lie transposed: [channel][slot]
     ops().rope_kv_write(dev, t(cos[:, :d // 2]), t(sin[:, :d // 2]), t(pos.astype(np.int32), torch.int32), heads, kv_heads, d,
                         t(slots.astype(np.int64), torch.int64), kc, vc)
     rel = EXACT if dtype is torch.float32 else BF16
     q_ref = pm.rope_apply(qkv[:, :heads * d], cos, sin, pos, d)
     k_ref = pm.rope_apply(qkv[:, heads * d:(heads + kv_heads) * d], cos, sin, pos, d)
     close(dev[:, :heads * d], q_ref, rel, "q in place")
-    kc_h, vc_h = kc.float().cpu().numpy(), vc.float().cpu().numpy()
+    kc_h, vc_h = kc.float().cpu().numpy(), vc.float().cpu().numpy().transpose(0, 1, 3, 2)
     written = np.zeros((n_blocks, bs), bool)
     for i, s in enumerate(slots):
         written[s // bs, s % bs] = True
@@ -215,6 +215,7 @@ def paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, dtype, scale_key=None)
         ks.append(k), vs.append(v), qs.append(q)
         pos.extend(range(L - q_lens[r], L))
         req.extend([r] * q_lens[r])
+    vc = vc.transpose(0, 1, 3, 2)      # the value cache is [block, kv_head, channel, slot]
     return dict(k=ks, v=vs, q=qs, kc=t(kc, dtype), vc=t(vc, dtype), table=t(table, torch.int32),
                 pos=t(np.array(pos, np.int32), torch.int32), req=t(np.array(req, np.int32), torch.int32),
                 qcat=t(np.concatenate(qs), dtype))
@@ -234,7 +235,7 @@ def test_paged_attention(heads, kv_heads, d, bs, dtype, exact, window):
     close(out, ref, 2e-6 if exact else BF16, "paged attention")
 
 
-@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 80, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (18, 2, 32, 64)])
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 80, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (18, 2, 32, 64), (20, 1, 32, 16)])
 @pytest.mark.parametrize("window", [None, 21, 300])
 @pytest.mark.parametrize("bucket", [700, 8192])
 def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
@@ -255,7 +256,7 @@ def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(5)])
     close(out, ref, BF16, "decode attention")
     if (heads, d, window) == (14, 64, None):
-        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == (1 if bucket == 700 else 5)   # several parts are really in play
+        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == (1 if bucket == 700 else 8)   # several parts are really in play
     one = torch.empty(1, heads * d, device=DEV, dtype=torch.bfloat16)        # one token that sees one key
     o.paged_attention(one, c["qcat"][:1], c["kc"], c["vc"], c["table"], c["req"][:1], c["pos"][:1], heads, kv_heads, d, window, scale, False,
                       max_q_len=1, max_context=1)
