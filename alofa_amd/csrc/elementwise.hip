@@ -29,6 +29,33 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(TO* __restrict__ out, cons
   __shared__ Acc scratch[4];
   const int r = blockIdx.x;
   const float* src = x + static_cast<int64_t>(rows ? rows[r] : r) * width;
+  TO* dst = out + static_cast<int64_t>(r) * width;
+  // rows of up to 256 * kKeep values stay in registers between the two passes, and their weights are on
+  // their way while the squares are summed; wider rows are read twice
+  constexpr int kKeep = 8;
+  if (width <= 256 * kKeep) {
+    float xs[kKeep], ws[kKeep];
+    Acc ss = 0;
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      xs[i] = c < width ? src[c] : 0.f;
+      ws[i] = c < width ? w[c] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {      // ascending c, as the strided loop below
+      const Acc v = static_cast<Acc>(xs[i]);
+      ss += v * v;
+    }
+    ss = block_sum<Acc, 256>(ss, scratch);
+    const Acc scale = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(width) + static_cast<Acc>(eps));
+#pragma unroll
+    for (int i = 0; i < kKeep; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (c < width) store_f32(dst + c, static_cast<float>(static_cast<Acc>(xs[i]) * scale * static_cast<Acc>(ws[i])));
+    }
+    return;
+  }
   Acc ss = 0;
   for (int c = threadIdx.x; c < width; c += 256) {
     Acc v = static_cast<Acc>(src[c]);
@@ -36,7 +63,6 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(TO* __restrict__ out, cons
   }
   ss = block_sum<Acc, 256>(ss, scratch);
   const Acc scale = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(width) + static_cast<Acc>(eps));
-  TO* dst = out + static_cast<int64_t>(r) * width;
   for (int c = threadIdx.x; c < width; c += 256)
     store_f32(dst + c, static_cast<float>(static_cast<Acc>(src[c]) * scale * static_cast<Acc>(w[c])));
 }

@@ -223,7 +223,7 @@ static int dispatch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, c
   const bool narrow = (kEpilogue != kSkSwiglu) && N <= 4096;
 #define ALOFA_SKINNY(MT, WIDE)                                                                                        \
   if (kEpilogue == kSkSwiglu)                                                                                         \
-    return launch_skinny<MT, 2, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);               \
+    return launch_skinny<MT, 2, (MT >= 4 ? 4 : 8), kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream); \
   if (narrow) return launch_skinny<MT, 1, 8, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);     \
   return launch_skinny<MT, WIDE, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
   if (M <= 16) { ALOFA_SKINNY(1, 2) }
