@@ -84,6 +84,27 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // What the epilogue adds (the bias, or the residual stream's old values) sets out now and has arrived when
+  // the sums are ready: this wave finishes tiles wave, wave + kWaves, ...
+  constexpr int kOutTiles = (kEpilogue == kSkSwiglu) ? MT : MT * NT;
+  constexpr int kMyTiles = (kOutTiles + kWaves - 1) / kWaves;
+  float add[kMyTiles][4];
+#pragma unroll
+  for (int it = 0; it < kMyTiles; ++it) {
+    const int tile = wave + it * kWaves;
+    const int mt = (kEpilogue == kSkSwiglu) ? tile : tile / NT, nt = (kEpilogue == kSkSwiglu) ? 0 : tile % NT;
+    const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = mt * 16 + g * 4 + i;
+      add[it][i] = 0.f;
+      if (tile < kOutTiles && n < N && m < M) {
+        if (kEpilogue == kSkStore && bias) add[it][i] = bias[n];
+        if (kEpilogue == kSkResidual) add[it][i] = load_f32(out + static_cast<int64_t>(m) * ldo + n);
+      }
+    }
+  }
+
   // steps of 32 along K: this block takes a contiguous share, this wave every kWaves-th step of it
   const int all_steps = (K + 31) / 32, k_splits = gridDim.y;
   const int per_split = (all_steps + k_splits - 1) / k_splits;
@@ -155,8 +176,10 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   const f32x4* parts = ws + static_cast<int64_t>(blockIdx.x) * k_splits * (MT * NT * 64);
 
   // tiles are shared out among the waves; each adds the partial sums in wave (or split) order
-  constexpr int kOutTiles = (kEpilogue == kSkSwiglu) ? MT : MT * NT;
-  for (int tile = wave; tile < kOutTiles; tile += kWaves) {
+#pragma unroll
+  for (int it = 0; it < kMyTiles; ++it) {
+    const int tile = wave + it * kWaves;
+    if (tile >= kOutTiles) break;
     const int mt = (kEpilogue == kSkSwiglu) ? tile : tile / NT;
     const int nt = (kEpilogue == kSkSwiglu) ? 0 : tile % NT;
     f32x4 sum, up = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -175,16 +198,15 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     }
     const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
     if (n >= N) continue;
-    const float b = (bias && kEpilogue == kSkStore) ? bias[n] : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = mt * 16 + g * 4 + i;
       if (m >= M) continue;
       TO* dst = out + static_cast<int64_t>(m) * ldo + n;
       if (kEpilogue == kSkStore) {
-        store_f32(dst, sum[i] + b);
+        store_f32(dst, sum[i] + add[it][i]);
       } else if (kEpilogue == kSkResidual) {
-        store_f32(dst, load_f32(dst) + sum[i]);
+        store_f32(dst, add[it][i] + sum[i]);
       } else {
         const float gv = sum[i];
         store_f32(dst, gv / (1.f + __expf(-gv)) * up[i]);
