@@ -30,8 +30,9 @@ enum MfmaEpilogue : int { kMfStore = 0, kMfResidual = 1, kMfSwiglu = 2 };
 constexpr int TK = 64, PAD = 8;
 constexpr int kRow = TK + PAD;  // LDS row length in elements
 
-// WT: MFMA tiles per wave along each of m and n (2: 128 x 128 block tile, 1: 64 x 64)
-template <int kEpilogue, typename TO, int WT>
+// WT: MFMA tiles per wave along each of m and n (2: 128 x 128 block tile, 1: 64 x 64).
+// PF: slabs on their way from memory while another is being multiplied.
+template <int kEpilogue, typename TO, int WT, int PF>
 __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, int64_t ldo,
                                                         const bf16_t* __restrict__ A, int64_t lda,
                                                         const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
@@ -80,23 +81,25 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // PF slabs are on their way from memory while another is being multiplied: two for the small
-  // tiles (their loop is short and latency shows), one for the big ones (registers are scarcer)
-  constexpr int PF = (WT == 1) ? 2 : 1;
   uint4 a_reg[PF][NC], w_reg[PF][NC];
   auto fetch = [&](uint4 (&a)[NC], uint4 (&w)[NC], int k0) {
+    // Every lane issues every load (from the row's start where the values are not wanted; zeros are put in
+    // their place at staging): with loads that are always issued the compiler can count them and wait for
+    // the oldest slab only, so that the later ones stay on their way.
+    const int koff = (k0 + c_k < K) ? k0 : -c_k;
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+      a[j] = *reinterpret_cast<const uint4*>(a_src[j] + koff);
+      w[j] = *reinterpret_cast<const uint4*>(w_src[j] + koff);
+    }
+  };
+  auto stage = [&](const uint4 (&a)[NC], const uint4 (&w)[NC], int k0) {
     const bool k_ok = k0 + c_k < K;
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-      a[j] = (k_ok && a_ok[j]) ? *reinterpret_cast<const uint4*>(a_src[j] + k0) : make_uint4(0, 0, 0, 0);
-      w[j] = (k_ok && w_ok[j]) ? *reinterpret_cast<const uint4*>(w_src[j] + k0) : make_uint4(0, 0, 0, 0);
-    }
-  };
-  auto stage = [&](const uint4 (&a)[NC], const uint4 (&w)[NC]) {
-#pragma unroll
-    for (int j = 0; j < NC; ++j) {
-      *reinterpret_cast<uint4*>(&As[c_row[j] * kRow + c_k]) = a[j];
-      *reinterpret_cast<uint4*>(&Ws[c_row[j] * kRow + c_k]) = w[j];
+      const uint32_t ka = 0u - static_cast<uint32_t>(k_ok && a_ok[j]), kw = 0u - static_cast<uint32_t>(k_ok && w_ok[j]);   // all ones or zero
+      *reinterpret_cast<uint4*>(&As[c_row[j] * kRow + c_k]) = make_uint4(a[j].x & ka, a[j].y & ka, a[j].z & ka, a[j].w & ka);
+      *reinterpret_cast<uint4*>(&Ws[c_row[j] * kRow + c_k]) = make_uint4(w[j].x & kw, w[j].y & kw, w[j].z & kw, w[j].w & kw);
     }
   };
 
@@ -132,7 +135,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
     for (int p = 0; p < PF; ++p) {
       if (k0 + p * TK < K) {    // uniform over the block
         __syncthreads();        // the previous slab has been read by every wave
-        stage(a_reg[p], w_reg[p]);
+        stage(a_reg[p], w_reg[p], k0 + p * TK);
         __syncthreads();
         fetch(a_reg[p], w_reg[p], k0 + (p + PF) * TK);
         multiply();
@@ -149,15 +152,25 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
       const int n = (kEpilogue == kMfSwiglu) ? n0 + wn * 32 + col : n0 + wn * 32 * WT + j * 32 + col;
       if (n >= N) continue;
       const float b = (bias && kEpilogue == kMfStore) ? bias[n] : 0.f;
+      const int m_first = m0 + wm * 32 * WT + i * 32 + row_base;      // element e: row m_first + 8 * (e / 4) + e % 4
+      TO* column = out + n;
+      float old[16];
+      if (kEpilogue == kMfResidual) {      // all sixteen old values set out before any is needed
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m_first + 8 * (e / 4) + e % 4;
+          old[e] = m < M ? load_f32(column + static_cast<int64_t>(m) * ldo) : 0.f;
+        }
+      }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int m = m0 + wm * 32 * WT + i * 32 + 8 * (e / 4) + row_base + e % 4;
+        const int m = m_first + 8 * (e / 4) + e % 4;
         if (m >= M) continue;
-        TO* dst = out + static_cast<int64_t>(m) * ldo + n;
+        TO* dst = column + static_cast<int64_t>(m) * ldo;
         if (kEpilogue == kMfStore) {
           store_f32(dst, acc[i][j][e] + b);
         } else if (kEpilogue == kMfResidual) {
-          store_f32(dst, load_f32(dst) + acc[i][j][e]);
+          store_f32(dst, old[e] + acc[i][j][e]);
         } else {
           const float g = acc[i][0][e];
           store_f32(dst, g / (1.f + __expf(-g)) * acc[i][WT - 1][e]);
@@ -170,20 +183,22 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 template <int kEpilogue, typename TO>
 static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                        const float* bias, int M, int N, int K, hipStream_t stream) {
-  // big tiles when they fill the chip (about two blocks per compute unit), small ones otherwise
+  // Big tiles (one slab ahead) when they fill the chip: about two blocks per compute unit, which hide one
+  // another's waits. Small tiles (two slabs ahead) otherwise: few big tiles, each alone on its compute
+  // unit, were slower here even with four slabs ahead.
   const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
   if (kEpilogue == kMfSwiglu || big_blocks >= 512) {
     constexpr int cols = (kEpilogue == kMfSwiglu) ? 64 : 128;
     dim3 grid((N + cols - 1) / cols, (M + 127) / 128);
-    gemm_mfma_kernel<kEpilogue, TO, 2><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
-                                                                  static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2),
-                                                                  ldw, bias, M, N, K);
+    gemm_mfma_kernel<kEpilogue, TO, 2, 1><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
+                                                                     static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2),
+                                                                     ldw, bias, M, N, K);
   } else {
     constexpr int kE = (kEpilogue == kMfSwiglu) ? kMfStore : kEpilogue;   // (never taken for swiglu)
     dim3 grid((N + 63) / 64, (M + 63) / 64);
-    gemm_mfma_kernel<kE, TO, 1><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
-                                                           static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw,
-                                                           bias, M, N, K);
+    gemm_mfma_kernel<kE, TO, 1, 2><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
+                                                              static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw,
+                                                              bias, M, N, K);
   }
   return check_launch("gemm_mfma");
 }
