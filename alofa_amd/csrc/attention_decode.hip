@@ -20,8 +20,8 @@
 // the weights are rounded to bfloat16 only as MFMA operands.
 //
 // The pages of a wave's share are read from the block table once, 64 at a time,
-// one per lane; keys and values of the next step are on their way while a step
-// is computed. At the end the waves' states meet in LDS and are combined in
+// one per lane; keys and values of the next two steps are on their way while a
+// step is computed. At the end the waves' states meet in LDS and are combined in
 // wave order. With several parts (long contexts) the blocks' states go to a
 // scratch buffer and a second kernel combines them in part order. The order of
 // additions depends only on the key range, the wave count and the part count,
@@ -90,66 +90,57 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   // lane x holds the page of logical block page_base + x; a step's keys lie within 64 pages of its first
   int page_base = (tile_begin << 4) >> bs_shift;
   const int last_page = p >> bs_shift;
+  // (pages that a window has passed read -1: they are never used, and 0 keeps every address inside the cache)
   int my_page = (tile_begin < tile_end && page_base + lane <= last_page) ? table[page_base + lane] : 0;
+  my_page = my_page < 0 ? 0 : my_page;
 
-  // operands of the step that starts at tile `tile` (two tiles): keys [tile][ds], values [tile][nt]
+  // Operands of the step that starts at tile `tile` (two tiles): keys [tile][ds], values [tile][nt]. Every
+  // lane issues every load, from the nearest visible key where its own is not visible (such scores are
+  // masked, such values cleared before use): with loads that are always issued the compiler can count
+  // them and wait for the oldest step only, so that two later steps stay on their way.
   struct Step {
     uint4 k[2][DS];
     uint2 v[2][DT];
   };
-  auto fetch = [&](int tile, Step& s) {
-    if (tile >= tile_end) return;                                      // uniform over the wave
-    if ((((((tile + 2) << 4) - 1)) >> bs_shift) - page_base >= 64) {       // uniform over the wave
+  const int lo4 = lo & ~3, p4 = p & ~3;
+  auto fetch = [&](int tile, Step& s) __attribute__((always_inline)) {
+    if ((((((tile + 2) << 4) - 1)) >> bs_shift) - page_base >= 64 && (tile << 4) <= p) {     // uniform over the wave
       page_base = (tile << 4) >> bs_shift;
       my_page = (page_base + lane <= last_page) ? table[page_base + lane] : 0;
+      my_page = my_page < 0 ? 0 : my_page;
     }
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
-      const bool tile_ok = tile + kt < tile_end;                       // uniform over the wave
-      // the key of this lane's row of K, and the first of this lane's four keys of V^T
-      const int key = ((tile + kt) << 4) + c16, key4 = ((tile + kt) << 4) + 4 * g;
-      const int kpage = ((tile_ok && key <= p ? key : tile << 4) >> bs_shift) - page_base;
-      const int vpage = ((tile_ok && key4 <= p ? key4 : tile << 4) >> bs_shift) - page_base;
-      const int64_t kblk = __shfl(my_page, kpage, 64), vblk = __shfl(my_page, vpage, 64);
+      // the key of this lane's row of K, and the first of this lane's four keys of V^T, brought into lo..p
+      int key = ((tile + kt) << 4) + c16, key4 = ((tile + kt) << 4) + 4 * g;
+      key = key < lo ? lo : (key > p ? p : key);
+      key4 = key4 < lo4 ? lo4 : (key4 > p4 ? p4 : key4);
+      // (a step past the end of the share may lie before the window of pages held in the lanes: its operands are not used)
+      const int kpage = (key >> bs_shift) - page_base, vpage = (key4 >> bs_shift) - page_base;
+      const int64_t kblk = __shfl(my_page, kpage < 0 ? 0 : (kpage > 63 ? 63 : kpage), 64);
+      const int64_t vblk = __shfl(my_page, vpage < 0 ? 0 : (vpage > 63 ? 63 : vpage), 64);
 #pragma unroll
       for (int ds = 0; ds < DS; ++ds) {
-        s.k[kt][ds] = make_uint4(0, 0, 0, 0);
         const int c = ds * 32 + g * 8;
-        if (tile_ok && key >= lo && key <= p && c < d)
-          s.k[kt][ds] = *reinterpret_cast<const uint4*>(k_cache + ((((kblk * kv_heads + hk) << bs_shift) + (key & bs_mask)) * d) + c);
+        s.k[kt][ds] = *reinterpret_cast<const uint4*>(k_cache + ((((kblk * kv_heads + hk) << bs_shift) + (key & bs_mask)) * d) + (c < d ? c : 0));
       }
 #pragma unroll
-      for (int nt = 0; nt < DT; ++nt) {
-        uint2 v = make_uint2(0, 0);
-        if (tile_ok && key4 + 3 >= lo && key4 <= p) {
-          v = *reinterpret_cast<const uint2*>(v_cache + ((((vblk * kv_heads + hk) * d + nt * 16 + c16) << bs_shift) + (key4 & bs_mask)));
-          // what lies beyond the visible keys is not data: it is cleared, so that a weight of zero times it is zero
-          const int lo_e = lo - key4, hi_e = p - key4 + 1;       // elements lo_e .. hi_e - 1 are visible
-          if (lo_e > 0 || hi_e < 4) {
-            if (0 < lo_e || 0 >= hi_e) v.x &= 0xffff0000u;
-            if (1 < lo_e || 1 >= hi_e) v.x &= 0x0000ffffu;
-            if (2 < lo_e || 2 >= hi_e) v.y &= 0xffff0000u;
-            if (3 < lo_e || 3 >= hi_e) v.y &= 0x0000ffffu;
-          }
-        }
-        s.v[kt][nt] = v;
-      }
+      for (int nt = 0; nt < DT; ++nt)
+        s.v[kt][nt] = *reinterpret_cast<const uint2*>(v_cache + ((((vblk * kv_heads + hk) * d + nt * 16 + c16) << bs_shift) + (key4 & bs_mask)));
     }
   };
 
-  Step cur, nxt;
-  fetch(tile_begin, cur);
-  for (int tile = tile_begin; tile < tile_end; tile += 2) {
-    fetch(tile + 2, nxt);
-
-    // S^T of the two tiles
+  // one step: the running state takes the two tiles from `tile` on (tiles past the share's end change nothing)
+  auto compute = [&](int tile, Step& st) __attribute__((always_inline)) {
+    // S^T of the two tiles (channels beyond d, in the last step of 32 of a head size that is no multiple of 32,
+    // meet zeros of Q)
     f32x4 s[2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ds = 0; ds < DS; ++ds)
-        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, cur.k[kt][ds]), qf[ds], s[kt], 0, 0, 0);
+        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, st.k[kt][ds]), qf[ds], s[kt], 0, 0, 0);
     }
     // scale, mask, running maximum; the four lanes of a head agree on the maximum
     float pw[8];
@@ -174,14 +165,56 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     l = l * corr + sum;   // this lane's share of the head's sum; the four lanes of a head meet at the end
     const uint4 w = make_uint4(pack_bf16x2(pw[0], pw[1]), pack_bf16x2(pw[2], pw[3]), pack_bf16x2(pw[4], pw[5]), pack_bf16x2(pw[6], pw[7]));
     const bf16x8 pf = __builtin_bit_cast(bf16x8, w);
+    // What lies beyond the visible keys is not data: it is cleared, so that a weight of zero times it is zero.
+    // (Within lo..p a weight of zero meets a visible key's values.)
+    uint32_t keep_x[2], keep_y[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const int key4 = ((tile + kt) << 4) + 4 * g;
+      const int lo_e = lo - key4, hi_e = p - key4 + 1;       // elements lo_e .. hi_e - 1 are visible
+      keep_x[kt] = ((0 < lo_e || 0 >= hi_e) ? 0u : 0x0000ffffu) | ((1 < lo_e || 1 >= hi_e) ? 0u : 0xffff0000u);
+      keep_y[kt] = ((2 < lo_e || 2 >= hi_e) ? 0u : 0x0000ffffu) | ((3 < lo_e || 3 >= hi_e) ? 0u : 0xffff0000u);
+    }
     // O^T += V^T P^T
 #pragma unroll
     for (int nt = 0; nt < DT; ++nt) {
       o[nt] *= corr;
-      const uint4 vv = make_uint4(cur.v[0][nt].x, cur.v[0][nt].y, cur.v[1][nt].x, cur.v[1][nt].y);
+      const uint4 vv = make_uint4(st.v[0][nt].x & keep_x[0], st.v[0][nt].y & keep_y[0], st.v[1][nt].x & keep_x[1], st.v[1][nt].y & keep_y[1]);
       o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf, o[nt], 0, 0, 0);
     }
-    cur = nxt;
+  };
+
+  // Three steps (two for large heads, whose operands fill the registers) are on their way or in work: each
+  // set of registers is filled again as soon as its step is done (no copies between sets: a copy would
+  // wait for the load).
+  constexpr bool kThree = DT <= 5;
+  constexpr int kStride = kThree ? 6 : 4;
+  Step s0, s1, s2;
+  int tile = tile_begin;
+  if (tile < tile_end) fetch(tile, s0);
+  if (tile + 2 < tile_end) fetch(tile + 2, s1);
+  if (kThree && tile + 4 < tile_end) fetch(tile + 4, s2);
+  // while every set has a further step to fetch: no branches, so that the waits are counted exactly
+  for (; tile + 2 * kStride - 2 < tile_end; tile += kStride) {
+    compute(tile, s0);
+    fetch(tile + kStride, s0);
+    compute(tile + 2, s1);
+    fetch(tile + 2 + kStride, s1);
+    if (kThree) {
+      compute(tile + 4, s2);
+      fetch(tile + 4 + kStride, s2);
+    }
+  }
+  // the last steps: nothing is fetched that no step will use (a wave ends only when its loads have come back)
+  for (; tile < tile_end; tile += kStride) {
+    compute(tile, s0);
+    if (tile + kStride < tile_end) fetch(tile + kStride, s0);
+    if (tile + 2 < tile_end) compute(tile + 2, s1);
+    if (tile + 2 + kStride < tile_end) fetch(tile + 2 + kStride, s1);
+    if (kThree) {
+      if (tile + 4 < tile_end) compute(tile + 4, s2);
+      if (tile + 4 + kStride < tile_end) fetch(tile + 4 + kStride, s2);
+    }
   }
   l = rows_sum(l);
 
