@@ -59,7 +59,7 @@ def sync():
     torch.cuda.synchronize()
 
 
-def measure_decode(model_dir, cfg, dtype, batch, steps, warmup, seed=0):
+def measure_decode(model_dir, cfg, dtype, batch, steps, warmup, seed=0, prompt=None):
     import numpy as np
     from alofa_amd import Engine
     rng = np.random.default_rng(seed)
@@ -67,8 +67,9 @@ def measure_decode(model_dir, cfg, dtype, batch, steps, warmup, seed=0):
     eng = Engine(model_dir, dtype=dtype, max_tokens=CONTEXT, max_batch=batch, kv_blocks=per_req * batch + 64,
                  block_size=BLOCK, token_budget=max(2048, batch), max_chunk=512, watermark_permille=1000)
     core = eng.core
+    prompt = PROMPT if prompt is None else prompt
     for r in range(batch):
-        core.submit(r + 1, [int(t) for t in rng.integers(0, cfg["vocab_size"], PROMPT)], CONTEXT - PROMPT)
+        core.submit(r + 1, [int(t) for t in rng.integers(0, cfg["vocab_size"], prompt)], CONTEXT - prompt)
     while not (core.last_action and len(core.last_action.decode) == batch and not core.last_action.prefill):
         core.tick()
     for _ in range(warmup):
@@ -162,6 +163,10 @@ def main():
             for b in (1, 64):
                 pms, _ = measure_decode(d, cfg, args.dtype, b, max(16, args.steps // 2), max(4, args.warmup // 2))
                 points[f"decode_b{b}"] = round(b / pms, 1)
+            # the same near the end of the context window (prompts of 3,840 tokens)
+            for b in (8, 64):
+                pms, _ = measure_decode(d, cfg, args.dtype, b, max(16, args.steps // 4), max(4, args.warmup // 4), prompt=CONTEXT - 256)
+                points[f"decode_b{b}_ctx{CONTEXT - 256}"] = round(b / pms, 1)
             out["points"] = points
     print(json.dumps(out))
     return 0
