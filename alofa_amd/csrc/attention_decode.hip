@@ -39,14 +39,48 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kMaxSplits = 64;
 constexpr int kHeadsPerBlock = 16;   // query heads of one key head that a block serves (the columns of a tile)
 
+// What the kernel needs to take the new token's projections as they come out of the fused query / key / value
+// product (kRope): q then points to rows [queries | keys | values] that are not yet rotated, one token per
+// request; the queries and the new key are rotated here by the token's position (half-split pairing,
+// cos / sin: [position, d / 2]), the new key and value are used from registers and written to the token's
+// cache slot by the one wave that owns the last tile of keys. Needs d a multiple of 64 (a channel and its
+// partner lie in the same lane's fragments).
+struct RopeArgs {
+  const float* cos_t;
+  const float* sin_t;
+  const int64_t* slots;
+};
+
+struct Pair8 {
+  uint4 lo, hi;
+};
+
+// a (low half) and b (high half) of eight pairs, rotated
+__device__ __forceinline__ Pair8 rotate8(uint4 lo, uint4 hi, float4 c_lo, float4 c_hi, float4 s_lo, float4 s_hi) {
+#pragma clang fp contract(off)
+  const uint32_t a[4] = {lo.x, lo.y, lo.z, lo.w}, b[4] = {hi.x, hi.y, hi.z, hi.w};
+  const float cs[8] = {c_lo.x, c_lo.y, c_lo.z, c_lo.w, c_hi.x, c_hi.y, c_hi.z, c_hi.w};
+  const float sn[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+  uint32_t ra[4], rb[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float a0 = __uint_as_float(a[i] << 16), a1 = __uint_as_float(a[i] & 0xffff0000u);
+    const float b0 = __uint_as_float(b[i] << 16), b1 = __uint_as_float(b[i] & 0xffff0000u);
+    ra[i] = pack_bf16x2(a0 * cs[2 * i] - b0 * sn[2 * i], a1 * cs[2 * i + 1] - b1 * sn[2 * i + 1]);
+    rb[i] = pack_bf16x2(b0 * cs[2 * i] + a0 * sn[2 * i], b1 * cs[2 * i + 1] + a1 * sn[2 * i + 1]);
+  }
+  return Pair8{make_uint4(ra[0], ra[1], ra[2], ra[3]), make_uint4(rb[0], rb[1], rb[2], rb[3])};
+}
+
 // DT = d / 16; NW: waves per block. blockIdx.y = key head * chunks + chunk of up to 16 heads of its group.
-template <int DT, int NW>
+template <int DT, int NW, bool kRope>
 __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ partial, const bf16_t* __restrict__ q,
-    int64_t q_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+    int64_t q_stride, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ rows, int heads, int kv_heads,
-    int bs_shift, int window, float scale) {
+    int bs_shift, int window, float scale, RopeArgs rope) {
+  static_assert(!kRope || DT % 4 == 0, "the rotation needs a channel and its partner in the same lane: d a multiple of 64");
   constexpr int d = DT * 16;
   constexpr int DS = (d + 31) / 32;            // steps of 32 along d in the first product
   // per wave and head: maximum, sum of weights, (two unused,) weighted value sums of the wave's share
@@ -79,6 +113,47 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     const int c = ds * 32 + g * 8;
     if (head_ok && c < d) v = *reinterpret_cast<const uint4*>(q + static_cast<int64_t>(t) * q_stride + static_cast<int64_t>(head) * d + c);
     qf[ds] = __builtin_bit_cast(bf16x8, v);
+  }
+
+  // the new token's key (this lane's channel slices, rotated) and value (channels 16 nt + c16), kRope only
+  uint4 new_k[DS];
+  uint32_t new_v[DT];
+  if constexpr (kRope) {
+    const bf16_t* row = q + static_cast<int64_t>(t) * q_stride;
+    const bf16_t* k_row = row + static_cast<int64_t>(heads + hk) * d;
+    const bf16_t* v_row = row + static_cast<int64_t>(heads + kv_heads + hk) * d;
+#pragma unroll
+    for (int ds = 0; ds < DS; ++ds) new_k[ds] = *reinterpret_cast<const uint4*>(k_row + ds * 32 + g * 8);
+#pragma unroll
+    for (int nt = 0; nt < DT; ++nt) new_v[nt] = v_row[nt * 16 + c16];
+    // pairs (c, c + d / 2): slices ds and ds + DS / 2 of this lane
+#pragma unroll
+    for (int ds = 0; ds < DS / 2; ++ds) {
+      const int64_t at = static_cast<int64_t>(p) * (d / 2) + ds * 32 + g * 8;
+      const float4 c_lo = *reinterpret_cast<const float4*>(rope.cos_t + at), c_hi = *reinterpret_cast<const float4*>(rope.cos_t + at + 4);
+      const float4 s_lo = *reinterpret_cast<const float4*>(rope.sin_t + at), s_hi = *reinterpret_cast<const float4*>(rope.sin_t + at + 4);
+      const Pair8 rq = rotate8(__builtin_bit_cast(uint4, qf[ds]), __builtin_bit_cast(uint4, qf[ds + DS / 2]), c_lo, c_hi, s_lo, s_hi);
+      qf[ds] = __builtin_bit_cast(bf16x8, rq.lo);
+      qf[ds + DS / 2] = __builtin_bit_cast(bf16x8, rq.hi);
+      const Pair8 rk = rotate8(new_k[ds], new_k[ds + DS / 2], c_lo, c_hi, s_lo, s_hi);
+      new_k[ds] = rk.lo;
+      new_k[ds + DS / 2] = rk.hi;
+    }
+    // the wave that owns the last tile of keys (in the first chunk of heads) writes the token's cache slot
+    if (h0 == 0 && tile_begin <= last && last < tile_end) {
+      const int64_t slot = rope.slots[t];
+      const int64_t blk = slot >> bs_shift, off = slot & bs_mask;
+      if (c16 == 0) {
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds)
+          *reinterpret_cast<uint4*>(k_cache + ((((blk * kv_heads + hk) << bs_shift) + off) * d) + ds * 32 + g * 8) = new_k[ds];
+      }
+      if (g == 0) {
+#pragma unroll
+        for (int nt = 0; nt < DT; ++nt)
+          v_cache[(((blk * kv_heads + hk) * d + nt * 16 + c16) << bs_shift) + off] = static_cast<bf16_t>(new_v[nt]);
+      }
+    }
   }
 
   f32x4 o[DT];
@@ -138,9 +213,19 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      // (kRope: the new token's key is not in the cache yet: its row of the last tile comes from the registers)
+      const bool new_row = kRope && tile + kt == last && c16 == (p & 15);
 #pragma unroll
-      for (int ds = 0; ds < DS; ++ds)
-        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, st.k[kt][ds]), qf[ds], s[kt], 0, 0, 0);
+      for (int ds = 0; ds < DS; ++ds) {
+        uint4 kf = st.k[kt][ds];
+        if constexpr (kRope) {      // (word by word: a choice between two whole operands would be made through memory)
+          kf.x = new_row ? new_k[ds].x : kf.x;
+          kf.y = new_row ? new_k[ds].y : kf.y;
+          kf.z = new_row ? new_k[ds].z : kf.z;
+          kf.w = new_row ? new_k[ds].w : kf.w;
+        }
+        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf), qf[ds], s[kt], 0, 0, 0);
+      }
     }
     // scale, mask, running maximum; the four lanes of a head agree on the maximum
     float pw[8];
@@ -179,7 +264,17 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
 #pragma unroll
     for (int nt = 0; nt < DT; ++nt) {
       o[nt] *= corr;
-      const uint4 vv = make_uint4(st.v[0][nt].x & keep_x[0], st.v[0][nt].y & keep_y[0], st.v[1][nt].x & keep_x[1], st.v[1][nt].y & keep_y[1]);
+      uint32_t vw[4] = {st.v[0][nt].x & keep_x[0], st.v[0][nt].y & keep_y[0], st.v[1][nt].x & keep_x[1], st.v[1][nt].y & keep_y[1]};
+      if constexpr (kRope) {
+        // the new token's value takes its place among this lane's four keys of the last tile
+#pragma unroll
+        for (int w2 = 0; w2 < 4; ++w2) {
+          const bool hit = tile + w2 / 2 == last && g == ((p & 15) >> 2) && ((p & 3) >> 1) == (w2 & 1);
+          const uint32_t ins = (p & 1) ? ((vw[w2] & 0x0000ffffu) | (new_v[nt] << 16)) : ((vw[w2] & 0xffff0000u) | new_v[nt]);
+          vw[w2] = hit ? ins : vw[w2];
+        }
+      }
+      const uint4 vv = make_uint4(vw[0], vw[1], vw[2], vw[3]);
       o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf, o[nt], 0, 0, 0);
     }
   };
@@ -290,11 +385,14 @@ extern "C" int64_t alofa_attention_decode_scratch(int tokens, int heads, int d, 
   return n_splits > 1 ? static_cast<int64_t>(tokens) * heads * n_splits * (d + 2) : 0;
 }
 
+// cos_t, sin_t, slots: null for queries that are rotated and a cache that is written already; else (see RopeArgs)
+// q holds rows [queries | keys | values] of one new token per request.
 extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
-                                      const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                      void* k_cache, void* v_cache, const int32_t* block_table,
                                       int max_blocks, const int32_t* req_of_token, const int32_t* positions,
                                       const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
-                                      float scale, int n_splits, hipStream_t stream) {
+                                      float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
+                                      hipStream_t stream) {
   ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
   ALOFA_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention_decode: head size %d must be 16..256 in steps of 16", d);
@@ -305,30 +403,44 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   ALOFA_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || partial), "attention_decode: n_splits=%d (1..%d) needs scratch when above 1", n_splits, kMaxSplits);
   ALOFA_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_decode: q rows must be 16-byte aligned");
   ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 8 == 0, "attention_decode: caches must be 16-byte aligned");
+  const bool fused = cos_t != nullptr;
+  ALOFA_REQUIRE(!fused || (sin_t && slots && d % 64 == 0 && q_stride >= static_cast<int64_t>(heads + 2 * kv_heads) * d),
+                "attention_decode: the rotary variant needs sin, slots, rows of queries, keys and values, and a head size in steps of 64 (d=%d)", d);
+  ALOFA_REQUIRE(!fused || (reinterpret_cast<uintptr_t>(cos_t) % 16 == 0 && reinterpret_cast<uintptr_t>(sin_t) % 16 == 0), "attention_decode: cos and sin must be 16-byte aligned");
   const int group = heads / kv_heads;
+  const RopeArgs rope{cos_t, sin_t, slots};
   dim3 grid(tokens, kv_heads * ((group + kHeadsPerBlock - 1) / kHeadsPerBlock), n_splits);
-#define ALOFA_DECODE(DT, NW)                                                                                              \
-  attention_decode_kernel<DT, NW><<<grid, 64 * NW, 0, stream>>>(                                                          \
+#define ALOFA_DECODE(DT, NW, ROPE)                                                                                        \
+  attention_decode_kernel<DT, NW, ROPE><<<grid, 64 * NW, 0, stream>>>(                                                    \
       static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                            \
-      static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), block_table, max_blocks, req_of_token,    \
-      positions, rows, heads, kv_heads, bs_shift, window, scale)
-  switch (d / 16) {
-    case 1: ALOFA_DECODE(1, 8); break;
-    case 2: ALOFA_DECODE(2, 8); break;
-    case 3: ALOFA_DECODE(3, 8); break;
-    case 4: ALOFA_DECODE(4, 8); break;
-    case 5: ALOFA_DECODE(5, 8); break;
-    case 6: ALOFA_DECODE(6, 8); break;
-    case 7: ALOFA_DECODE(7, 8); break;
-    case 8: ALOFA_DECODE(8, 8); break;
-    case 9: ALOFA_DECODE(9, 4); break;
-    case 10: ALOFA_DECODE(10, 4); break;
-    case 11: ALOFA_DECODE(11, 4); break;
-    case 12: ALOFA_DECODE(12, 4); break;
-    case 13: ALOFA_DECODE(13, 4); break;
-    case 14: ALOFA_DECODE(14, 4); break;
-    case 15: ALOFA_DECODE(15, 4); break;
-    default: ALOFA_DECODE(16, 4); break;
+      static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), block_table, max_blocks, req_of_token,                \
+      positions, rows, heads, kv_heads, bs_shift, window, scale, rope)
+  if (fused) {
+    switch (d / 64) {
+      case 1: ALOFA_DECODE(4, 8, true); break;
+      case 2: ALOFA_DECODE(8, 8, true); break;
+      case 3: ALOFA_DECODE(12, 4, true); break;
+      default: ALOFA_DECODE(16, 4, true); break;
+    }
+  } else {
+    switch (d / 16) {
+      case 1: ALOFA_DECODE(1, 8, false); break;
+      case 2: ALOFA_DECODE(2, 8, false); break;
+      case 3: ALOFA_DECODE(3, 8, false); break;
+      case 4: ALOFA_DECODE(4, 8, false); break;
+      case 5: ALOFA_DECODE(5, 8, false); break;
+      case 6: ALOFA_DECODE(6, 8, false); break;
+      case 7: ALOFA_DECODE(7, 8, false); break;
+      case 8: ALOFA_DECODE(8, 8, false); break;
+      case 9: ALOFA_DECODE(9, 4, false); break;
+      case 10: ALOFA_DECODE(10, 4, false); break;
+      case 11: ALOFA_DECODE(11, 4, false); break;
+      case 12: ALOFA_DECODE(12, 4, false); break;
+      case 13: ALOFA_DECODE(13, 4, false); break;
+      case 14: ALOFA_DECODE(14, 4, false); break;
+      case 15: ALOFA_DECODE(15, 4, false); break;
+      default: ALOFA_DECODE(16, 4, false); break;
+    }
   }
 #undef ALOFA_DECODE
   if (check_launch("attention_decode")) return 1;

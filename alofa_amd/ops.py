@@ -341,9 +341,14 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
 
 
 def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
-                     max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None) -> None:
+                     max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
+                     rope: Optional[tuple] = None) -> None:
     """bfloat16 attention for tokens of requests that bring few tokens: every
-    token of the batch, or the tokens ``rows`` (int32 indices into the batch)."""
+    token of the batch, or the tokens ``rows`` (int32 indices into the batch).
+    With ``rope`` = (cos, sin, slots) the rows of ``q`` are the fused projection's
+    [queries | keys | values] of ONE new token per request, not yet rotated: the
+    kernel rotates queries and the new key itself, uses the new key and value from
+    registers and writes them to the token's cache slot (``can_fuse_rope_into_decode``)."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     for n, t in (("req_of_token", req_of_token), ("positions", positions)):
         _gpu(n, t, torch.int32, 1), _contig(n, t)
@@ -353,13 +358,31 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     if rows is not None:
         _gpu("rows", rows, torch.int32, 1), _contig("rows", rows)
         n_tok = rows.shape[0]
+    cos = sin = slots = None
+    if rope is not None:
+        cos, sin, slots = rope
+        if not can_fuse_rope_into_decode(d) or q.shape[1] < (heads + 2 * kv_heads) * d:
+            raise AlofaError("unsupported", "the rotary decode kernel needs head sizes in steps of 64 and rows of queries, keys and values",
+                             f"head_dim={d} q={tuple(q.shape)}")
+        _gpu("cos", cos, torch.float32, 2), _gpu("sin", sin, torch.float32, 2), _contig("cos", cos), _contig("sin", sin)
+        if cos.shape != sin.shape or cos.shape[1] != d // 2:
+            raise AlofaError("shape_mismatch", "rotary table must be [positions, d/2]", f"cos={tuple(cos.shape)} d={d}")
+        _gpu("slots", slots, torch.int64, 1), _contig("slots", slots)
+        if slots.shape[0] != T:
+            raise AlofaError("shape_mismatch", "one cache slot per token", f"slots={tuple(slots.shape)} T={T}")
     n_splits = decode_splits(n_tok, heads, kv_heads, d, min(max_context, window or max_context))
     floats = n_tok * heads * n_splits * (d + 2) if n_splits > 1 else 0
     if floats and (scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous()):
         raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")
     _call("alofa_attention_decode", _ptr(out), _L(_rows("out", out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
           _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(rows),
-          _I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits), _stream())
+          _I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits),
+          _ptr(cos), _ptr(sin), _ptr(slots), _stream())
+
+
+def can_fuse_rope_into_decode(d: int) -> bool:
+    """Head sizes for which the decode attention kernel can rotate and write the new token itself."""
+    return d % 64 == 0
 
 
 PREFILL_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 256)

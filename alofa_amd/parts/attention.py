@@ -80,25 +80,30 @@ class GQAAttention(Mixer):
                                 qkv[:, hd:hd + self.kv_heads * self.d].unflatten(1, (self.kv_heads, self.d)))
             table = ctx.identity_rotation(self.d)
         cos, sin = table
-        if kv.owner:
-            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d, kv.slots, kv.k, kv.v)
-        else:
-            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
         attn = ctx.scratch("attn", (T, self.heads * self.d), self.rt.dtype)
         common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
         pow2_pages = kv.k.shape[2] >= ops.MIN_FAST_PAGE and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
         fast_prefill = self.d in ops.PREFILL_HEAD_DIMS
+        # one new token per request: the decode kernel rotates it and writes its cache slot itself
+        fused = (not exact and pow2_pages and kv.owner and ctx.max_q_len == 1 and ctx.long_tiles is None
+                 and ops.can_fuse_rope_into_decode(self.d))
+        if fused:
+            pass
+        elif kv.owner:
+            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d, kv.slots, kv.k, kv.v)
+        else:
+            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
         if exact or not pow2_pages or (ctx.long_tiles is not None and not fast_prefill):
             # the exact path, and page or head sizes the bfloat16 kernels are not built for
             ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
         else:
             if ctx.long_tiles is not None:      # portions of prompts
                 ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, ctx.long_tiles, *common)
-            if ctx.n_short:                     # single tokens and very short portions, all key heads' groups together
+            if ctx.n_short:                     # single tokens and very short portions, all query heads of a key head together
                 floats = ops.decode_scratch_floats(ctx.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
                 partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
                 ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common,
-                                     ctx.max_context, partial, rows=ctx.short_rows)
+                                     ctx.max_context, partial, rows=ctx.short_rows, rope=(cos, sin, kv.slots) if fused else None)
         if self.b_o is not None:
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
             ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)

@@ -244,7 +244,7 @@ def test_pool_too_small_is_a_named_error(tiny_dirs):
     assert e.value.name == "out_of_range"
 
 
-@pytest.mark.parametrize("name", ["A", "C"])
+@pytest.mark.parametrize("name", ["A", "C", "D"])      # D: the decode kernel rotates and writes the new token itself
 def test_decode_graph_replays_equal_eager_steps(tiny_dirs, name):
     """Decode steps replay a captured HIP graph. Every replay is compared with
     the same step run eagerly, with other work (portions of other requests,

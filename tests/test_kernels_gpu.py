@@ -268,6 +268,49 @@ def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
                               max_q_len=4, max_context=bucket)
 
 
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(14, 2, 64, 16), (8, 2, 128, 32), (20, 1, 64, 8), (3, 3, 256, 16)])
+@pytest.mark.parametrize("window", [None, 21])
+@pytest.mark.parametrize("bucket", [700, 8192])
+def test_decode_attention_that_rotates_and_writes_the_new_token(heads, kv_heads, d, bs, window, bucket):
+    """One new token per request, handed over as the fused projection's row [queries | keys | values]
+    before rotation: the kernel rotates queries and the new key, attends over the cache and the new
+    token, and writes the new key and value to the token's slot (which holds NaN before)."""
+    rng = np.random.default_rng(19)
+    lens, n = [1, 37, 700, 64, 333, 16, 17], 7
+    c = paged_case(rng, lens, [1] * n, heads, kv_heads, d, bs, torch.bfloat16)
+    cos, sin = pm.rope_table(max(lens), d, 1e4)
+    o = ops()
+    assert o.can_fuse_rope_into_decode(d)
+    qkv = np.zeros((n, (heads + 2 * kv_heads) * d), np.float32)
+    kc, vc = c["kc"].clone(), c["vc"].clone()
+    slots, refs = [], []
+    table = c["table"].cpu().numpy()
+    for r, L in enumerate(lens):
+        q_raw = bf(rng.standard_normal((1, heads * d)).astype(np.float32))
+        k_raw = bf(rng.standard_normal((1, kv_heads * d)).astype(np.float32))
+        pos = np.array([L - 1])
+        q_rot = bf(pm.rope_apply(q_raw, cos, sin, pos, d).astype(np.float32))
+        k_rot = bf(pm.rope_apply(k_raw, cos, sin, pos, d).astype(np.float32))
+        k = c["k"][r].copy()
+        k[L - 1] = k_rot[0]                          # what the cache must hold for the new token afterwards
+        qkv[r] = np.concatenate([q_raw[0], k_raw[0], c["v"][r][L - 1]])
+        slot = int(table[r, (L - 1) // bs]) * bs + (L - 1) % bs
+        slots.append(slot)
+        kc[slot // bs, :, slot % bs] = float("nan")                          # not written yet
+        vc[slot // bs, :, :, slot % bs] = float("nan")
+        refs.append((pm.attention(q_rot, k, c["v"][r], heads, kv_heads, d, window), k_rot[0], c["v"][r][L - 1]))
+    out = torch.empty(n, heads * d, device=DEV, dtype=torch.bfloat16)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    scratch = torch.empty(max(1, o.decode_scratch_floats(n, heads, kv_heads, d, bucket, window)), device=DEV)
+    o.attention_decode(out, t(qkv, torch.bfloat16), kc, vc, c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, bucket, scratch,
+                       rope=(t(cos[:, :d // 2]), t(sin[:, :d // 2]), t(np.array(slots, np.int64), torch.int64)))
+    close(out, np.concatenate([a for a, _, _ in refs]), BF16, "attention with the new token from registers")
+    kc_h, vc_h = kc.float().cpu().numpy(), vc.float().cpu().numpy()
+    for r, slot in enumerate(slots):
+        close(kc_h[slot // bs, :, slot % bs].reshape(-1), refs[r][1], BF16, "new key in its slot")
+        assert np.array_equal(vc_h[slot // bs, :, :, slot % bs].reshape(-1), refs[r][2]), "new value in its slot"
+
+
 @pytest.mark.parametrize("heads,kv_heads,d", [(5, 1, 80), (2, 2, 96), (3, 1, 64)])
 def test_decode_attention_with_many_splits(heads, kv_heads, d):
     """One token over 5,000 keys, the launch shaped for a far longer context: the keys are shared out
