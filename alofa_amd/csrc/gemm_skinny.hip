@@ -225,8 +225,10 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
   const Workspace& g_ws = workspace();
   if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr) {
     const int steps = (K + 31) / 32;
-    // (a split costs a trip through memory: only while every wave keeps at least two steps of its own)
-    while (k_splits < 8 && col_tiles * k_splits * 2 <= 512 && steps / (k_splits * 2) >= kWaves) k_splits *= 2;
+    // (a split costs a trip through memory: only while every wave keeps at least two steps of its own, four
+    // with one tile of rows, whose steps are light)
+    const int min_steps = (MT == 1) ? 2 * kWaves : kWaves;
+    while (k_splits < 8 && col_tiles * k_splits * 2 <= 512 && steps / (k_splits * 2) >= min_steps) k_splits *= 2;
     if (col_tiles > kGemmCounters || static_cast<int64_t>(col_tiles) * k_splits * MT * NT * 256 > g_ws.tile_floats) k_splits = 1;
   }
   // loads in flight: many for one row tile (latency is all there is), fewer as row tiles take the registers
