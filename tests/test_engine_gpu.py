@@ -183,6 +183,22 @@ def test_random_configurations(tmp_path, seed):
         assert_close(collect(r, portions("y", requests["r0"]))["y"], ref["r0"], dtype, f"[{what}] {dtype} portions")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_model_stored_in_float32(tmp_path, dtype):
+    """Tensors stored in 32-bit stay so: in the bfloat16 engine they are multiplied as float32
+    (the always-valid kernels), activations in bfloat16; the float32 engine is exact as ever."""
+    from alofa_amd.replay import Replayer
+    from alofa_amd.weights import write_random_model
+    write_random_model(TINY["B"], tmp_path, seed=77, store_dtype="float32")
+    ids = random_ids(78, 90, TINY["B"]["vocab_size"])
+    ref = plain_logits(tmp_path, tuple(ids))
+    r = Replayer(tmp_path, dtype, 256)
+    import torch
+    assert all(b.mixer.w_qkv.dtype is torch.float32 for b in r.model.blocks)
+    assert_close(collect(r, bulk_and_tail("a", ids))["a"], ref, dtype, "float32 storage, bulk+tail")
+    assert_close(collect(r, portions("b", ids))["b"], ref, dtype, "float32 storage, portions")
+
+
 @pytest.mark.parametrize("block_size", [16, 32, 64])
 def test_page_size_does_not_matter(replayers, tiny_dirs, block_size):
     ids = ids_of("B")
