@@ -1,23 +1,29 @@
-// Matrix products for many rows (prompt portions), bfloat16 on MFMA:
-// out[m, n] = sum_k A[m, k] * W[n, k].
+// Matrix products whose operands are shared through LDS, bfloat16 on MFMA:
+// out[m, n] = sum_k A[m, k] * W[n, k]. For prompt portions, and for few rows
+// against weights so big that reading the rows again for every few weight rows
+// (as the streaming kernel does) would cost more than the weights themselves.
 //
-// A block of four wavefronts (2 x 2) computes a 128 x 128 tile of the output,
-// every wave a 64 x 64 quarter as 2 x 2 tiles of v_mfma_f32_32x32x16_bf16; for
-// outputs too small to fill the chip with such tiles the block computes 64 x 64
-// (one MFMA tile per wave). Per step of 64 along K the block stages a slab of A
-// and of W in LDS
-// (16-byte loads along K; rows are padded by 8 elements so that the fragment
-// reads fall on distinct banks), while the next slab is already on its way from
-// memory into registers. Accumulation is float; each output element has one
-// accumulator that takes the products in ascending k, whatever M is.
+// A block of four wavefronts (2 x 2) computes a tile of 64 WTM x 64 WTN outputs,
+// every wave WTM x WTN tiles of v_mfma_f32_32x32x16_bf16: 128 x 128 where such
+// tiles fill the chip, 64 x 64 otherwise. Per step of 64 along K the block
+// stages a slab of A and of W in LDS (16-byte loads along K; rows are padded by
+// 8 elements so that the fragment reads fall on distinct banks), while the next
+// slabs are already on their way from memory into registers. Accumulation is
+// float; each output element has one accumulator that takes the products in
+// ascending k, whatever M is.
+//
+// Where even the small tiles are too few for the chip (few rows, few columns, a
+// long K), blockIdx.z shares K out as well: every block leaves its partial tile
+// in the workspace, and the one that arrives last adds them in a fixed order and
+// runs the epilogue (the protocol of the streaming kernel, see there).
 //
 // Operand layout of the instruction, lane l: A holds row l % 32 and B column
 // l % 32, both the reduction indices 8 * (l / 32) .. + 7 of the 16; D holds
 // column l % 32 and, in acc[i], row 8 * (i / 4) + 4 * (l / 32) + i % 4.
 //
 // Epilogues: store (+ bias), add to the float residual stream, and SwiGLU, for
-// which a block computes the gate and the up product of the same 64 columns
-// (its W slab holds 64 rows of each) and writes silu(gate) * up.
+// which a block computes the gate and the up product of the same columns (its
+// W slab holds as many rows of each) and writes silu(gate) * up.
 #include "common.h"
 
 namespace alofa {
@@ -30,16 +36,27 @@ enum MfmaEpilogue : int { kMfStore = 0, kMfResidual = 1, kMfSwiglu = 2 };
 constexpr int TK = 64, PAD = 8;
 constexpr int kRow = TK + PAD;  // LDS row length in elements
 
-// WT: MFMA tiles per wave along each of m and n (2: 128 x 128 block tile, 1: 64 x 64).
+// WTM, WTN: MFMA tiles per wave along m and along n; the block tile is 64 WTM x 64 WTN.
 // PF: slabs on their way from memory while another is being multiplied.
-template <int kEpilogue, typename TO, int WT, int PF>
+// kSplitK: blockIdx.z takes a share of K; the shares meet in the workspace (see below).
+template <int kEpilogue, typename TO, int WTM, int WTN, int PF, bool kSplitK>
 __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, int64_t ldo,
                                                         const bf16_t* __restrict__ A, int64_t lda,
                                                         const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                                         int64_t ldw, const float* __restrict__ bias, int M, int N,
-                                                        int K) {
-  constexpr int TM = 64 * WT, TN = 64 * WT;
-  static_assert(kEpilogue != kMfSwiglu || WT == 2, "the swiglu epilogue needs two column tiles per wave");
+                                                        int K_all, float* __restrict__ ws, int* __restrict__ counters) {
+  constexpr int TM = 64 * WTM, TN = 64 * WTN;
+  // swiglu: the first half of a wave's column tiles are gate columns, the second half the up columns of the same outputs
+  constexpr int kGateTiles = WTN / 2;
+  static_assert(kEpilogue != kMfSwiglu || WTN % 2 == 0, "the swiglu epilogue needs an even number of column tiles per wave");
+  __shared__ int last_block;
+  // this block's share of K: slabs [k_begin, K)
+  int k_begin = 0, K = K_all;
+  if (kSplitK) {
+    const int slabs = (K_all + TK - 1) / TK, per_split = (slabs + static_cast<int>(gridDim.z) - 1) / static_cast<int>(gridDim.z);
+    k_begin = blockIdx.z * per_split * TK;
+    K = min(K_all, k_begin + per_split * TK);
+  }
   __shared__ __attribute__((aligned(16))) bf16_t As[TM * kRow];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[TN * kRow];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -47,90 +64,95 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
   constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * kOutCols;
 
-  // global -> register staging: TM * 8 chunks of 16 bytes per slab, NC per thread
-  constexpr int NC = WT * 2;
-  int c_row[NC];
-#pragma unroll
-  for (int j = 0; j < NC; ++j) c_row[j] = (tid + 256 * j) / 8;
+  // global -> register staging: 8 chunks of 16 bytes per slab row; a thread takes row (tid + 256 j) / 8
+  constexpr int NCA = WTM * 2, NCW = WTN * 2;
   const int c_k = (tid % 8) * 8;
-  const bf16_t* a_src[NC];
-  const bf16_t* w_src[NC];
-  bool a_ok[NC], w_ok[NC];
+  const bf16_t* a_src[NCA];
+  const bf16_t* w_src[NCW];
+  bool a_ok[NCA], w_ok[NCW];
 #pragma unroll
-  for (int j = 0; j < NC; ++j) {
-    const int m = m0 + c_row[j];
+  for (int j = 0; j < NCA; ++j) {
+    const int m = m0 + (tid + 256 * j) / 8;
     a_ok[j] = m < M;
     a_src[j] = A + static_cast<int64_t>(a_ok[j] ? m : 0) * lda + c_k;
-    int n;
+  }
+#pragma unroll
+  for (int j = 0; j < NCW; ++j) {
+    const int row = (tid + 256 * j) / 8;
+    int n = n0 + row;
     const bf16_t* base = W;
-    if (kEpilogue == kMfSwiglu) {  // slab rows 0..63: gate rows n0..n0+63, rows 64..127: up rows of the same columns
-      n = n0 + (c_row[j] % 64);
-      if (c_row[j] >= 64) base = W2;
-    } else {
-      n = n0 + c_row[j];
+    if (kEpilogue == kMfSwiglu && row >= TN / 2) {  // slab rows below TN / 2: gate rows n0 ..; the others: up rows of the same columns
+      n = n0 + row - TN / 2;
+      base = W2;
     }
     w_ok[j] = n < N;
     w_src[j] = base + static_cast<int64_t>(w_ok[j] ? n : 0) * ldw + c_k;
   }
 
-  f32x16 acc[WT][WT];
+  f32x16 acc[WTM][WTN];
 #pragma unroll
-  for (int i = 0; i < WT; ++i)
+  for (int i = 0; i < WTM; ++i)
 #pragma unroll
-    for (int j = 0; j < WT; ++j)
+    for (int j = 0; j < WTN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  uint4 a_reg[PF][NC], w_reg[PF][NC];
-  auto fetch = [&](uint4 (&a)[NC], uint4 (&w)[NC], int k0) {
+  uint4 a_reg[PF][NCA], w_reg[PF][NCW];
+  auto fetch = [&](uint4 (&a)[NCA], uint4 (&w)[NCW], int k0) {
     // Every lane issues every load (from the row's start where the values are not wanted; zeros are put in
     // their place at staging): with loads that are always issued the compiler can count them and wait for
     // the oldest slab only, so that the later ones stay on their way.
     const int koff = (k0 + c_k < K) ? k0 : -c_k;
 #pragma unroll
-    for (int j = 0; j < NC; ++j) {
-      a[j] = *reinterpret_cast<const uint4*>(a_src[j] + koff);
-      w[j] = *reinterpret_cast<const uint4*>(w_src[j] + koff);
-    }
-  };
-  auto stage = [&](const uint4 (&a)[NC], const uint4 (&w)[NC], int k0) {
-    const bool k_ok = k0 + c_k < K;
+    for (int j = 0; j < NCA; ++j) a[j] = *reinterpret_cast<const uint4*>(a_src[j] + koff);
 #pragma unroll
-    for (int j = 0; j < NC; ++j) {
-      const uint32_t ka = 0u - static_cast<uint32_t>(k_ok && a_ok[j]), kw = 0u - static_cast<uint32_t>(k_ok && w_ok[j]);   // all ones or zero
-      *reinterpret_cast<uint4*>(&As[c_row[j] * kRow + c_k]) = make_uint4(a[j].x & ka, a[j].y & ka, a[j].z & ka, a[j].w & ka);
-      *reinterpret_cast<uint4*>(&Ws[c_row[j] * kRow + c_k]) = make_uint4(w[j].x & kw, w[j].y & kw, w[j].z & kw, w[j].w & kw);
+    for (int j = 0; j < NCW; ++j) w[j] = *reinterpret_cast<const uint4*>(w_src[j] + koff);
+  };
+  auto stage = [&](const uint4 (&a)[NCA], const uint4 (&w)[NCW], int k0) {
+    const bool k_ok = k0 + c_k < K;
+    const int first = (tid / 8) * kRow + c_k;    // chunk j lies 32 slab rows further on
+#pragma unroll
+    for (int j = 0; j < NCA; ++j) {
+      const uint32_t ka = 0u - static_cast<uint32_t>(k_ok && a_ok[j]);   // all ones or zero
+      *reinterpret_cast<uint4*>(&As[first + j * 32 * kRow]) = make_uint4(a[j].x & ka, a[j].y & ka, a[j].z & ka, a[j].w & ka);
+    }
+#pragma unroll
+    for (int j = 0; j < NCW; ++j) {
+      const uint32_t kw = 0u - static_cast<uint32_t>(k_ok && w_ok[j]);
+      *reinterpret_cast<uint4*>(&Ws[first + j * 32 * kRow]) = make_uint4(w[j].x & kw, w[j].y & kw, w[j].z & kw, w[j].w & kw);
     }
   };
 
   // rows of the fragments this lane reads
   const int frag_row = lane % 32, frag_k = (lane / 32) * 8;
-  int a_off[WT], w_off[WT];
+  int a_off[WTM], w_off[WTN];
 #pragma unroll
-  for (int i = 0; i < WT; ++i) {
-    a_off[i] = (wm * 32 * WT + i * 32 + frag_row) * kRow + frag_k;
-    // swiglu: tile 0 = gate rows of this wave's 32 columns, tile 1 = the up rows of the same columns
-    w_off[i] = ((kEpilogue == kMfSwiglu) ? (i * 64 + wn * 32 + frag_row) : (wn * 32 * WT + i * 32 + frag_row)) * kRow + frag_k;
+  for (int i = 0; i < WTM; ++i) a_off[i] = (wm * 32 * WTM + i * 32 + frag_row) * kRow + frag_k;
+#pragma unroll
+  for (int j = 0; j < WTN; ++j) {
+    int row = wn * 32 * WTN + j * 32 + frag_row;
+    if (kEpilogue == kMfSwiglu)   // this wave's 32 kGateTiles output columns: their gate rows, then their up rows
+      row = (j < kGateTiles) ? wn * 32 * kGateTiles + j * 32 + frag_row : TN / 2 + wn * 32 * kGateTiles + (j - kGateTiles) * 32 + frag_row;
+    w_off[j] = row * kRow + frag_k;
   }
   auto multiply = [&]() {
 #pragma unroll
     for (int ks = 0; ks < TK; ks += 16) {
-      bf16x8 a[WT], w[WT];
+      bf16x8 a[WTM], w[WTN];
 #pragma unroll
-      for (int i = 0; i < WT; ++i) {
-        a[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&As[a_off[i] + ks]));
-        w[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Ws[w_off[i] + ks]));
-      }
+      for (int i = 0; i < WTM; ++i) a[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&As[a_off[i] + ks]));
 #pragma unroll
-      for (int i = 0; i < WT; ++i)
+      for (int j = 0; j < WTN; ++j) w[j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&Ws[w_off[j] + ks]));
 #pragma unroll
-        for (int j = 0; j < WT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int j = 0; j < WTN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
     }
   };
 
 #pragma unroll
-  for (int p = 0; p < PF; ++p) fetch(a_reg[p], w_reg[p], p * TK);
-  for (int k0 = 0; k0 < K; k0 += PF * TK) {
+  for (int p = 0; p < PF; ++p) fetch(a_reg[p], w_reg[p], k_begin + p * TK);
+  for (int k0 = k_begin; k0 < K; k0 += PF * TK) {
 #pragma unroll
     for (int p = 0; p < PF; ++p) {
       if (k0 + p * TK < K) {    // uniform over the block
@@ -143,16 +165,61 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
     }
   }
 
+  if (kSplitK) {
+    // The shares of K meet in the workspace: every block leaves its tile there (at device scope: written
+    // through to memory, where blocks on every die find it) and is counted once every wave's stores have
+    // been acknowledged; the block counted last adds the tiles in split order, so the sum is the same on
+    // every run, goes on to the epilogue and puts the counter back to zero.
+    const int splits = gridDim.z, tile_id = blockIdx.y * gridDim.x + blockIdx.x;
+    constexpr int kTileFloats = WTM * WTN * 16 * 256;
+    float* mine = ws + (static_cast<int64_t>(tile_id) * splits + blockIdx.z) * kTileFloats;
+#pragma unroll
+    for (int i = 0; i < WTM; ++i)
+#pragma unroll
+      for (int j = 0; j < WTN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          __hip_atomic_store(mine + ((i * WTN + j) * 16 + e) * 256 + tid, acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      const int arrived = atomicAdd(&counters[tile_id], 1);
+      last_block = arrived == splits - 1;
+      if (last_block) atomicExch(&counters[tile_id], 0);
+    }
+    __syncthreads();
+    if (!last_block) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const float* parts = ws + static_cast<int64_t>(tile_id) * splits * kTileFloats;
+#pragma unroll
+    for (int i = 0; i < WTM; ++i)
+#pragma unroll
+      for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int sp = 0; sp < splits; ++sp) {
+          float part[16];
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            part[e] = __hip_atomic_load(parts + static_cast<int64_t>(sp) * kTileFloats + ((i * WTN + j) * 16 + e) * 256 + tid,
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] += part[e];
+        }
+      }
+  }
+
   // epilogue
   const int col = lane % 32, row_base = (lane / 32) * 4;
+  constexpr int kOutTiles = (kEpilogue == kMfSwiglu) ? kGateTiles : WTN;
 #pragma unroll
-  for (int i = 0; i < WT; ++i) {
+  for (int i = 0; i < WTM; ++i) {
 #pragma unroll
-    for (int j = 0; j < ((kEpilogue == kMfSwiglu) ? 1 : WT); ++j) {
-      const int n = (kEpilogue == kMfSwiglu) ? n0 + wn * 32 + col : n0 + wn * 32 * WT + j * 32 + col;
+    for (int j = 0; j < kOutTiles; ++j) {
+      const int n = n0 + wn * 32 * kOutTiles + j * 32 + col;
       if (n >= N) continue;
       const float b = (bias && kEpilogue == kMfStore) ? bias[n] : 0.f;
-      const int m_first = m0 + wm * 32 * WT + i * 32 + row_base;      // element e: row m_first + 8 * (e / 4) + e % 4
+      const int m_first = m0 + wm * 32 * WTM + i * 32 + row_base;      // element e: row m_first + 8 * (e / 4) + e % 4
       TO* column = out + n;
       float old[16];
       if (kEpilogue == kMfResidual) {      // all sixteen old values set out before any is needed
@@ -172,35 +239,70 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
         } else if (kEpilogue == kMfResidual) {
           store_f32(dst, old[e] + acc[i][j][e]);
         } else {
-          const float g = acc[i][0][e];
-          store_f32(dst, g / (1.f + __expf(-g)) * acc[i][WT - 1][e]);
+          const float g = acc[i][j][e];
+          store_f32(dst, g / (1.f + __expf(-g)) * acc[i][(j + kGateTiles) % WTN][e]);
         }
       }
     }
   }
 }
 
+template <int kEpilogue, typename TO, int WTM, int WTN, int PF, bool kSplitK>
+static void launch_tile(dim3 grid, void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
+                        const float* bias, int M, int N, int K, hipStream_t stream) {
+  const Workspace& g_ws = workspace();
+  gemm_mfma_kernel<kEpilogue, TO, WTM, WTN, PF, kSplitK><<<grid, 256, 0, stream>>>(
+      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
+      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, kSplitK ? g_ws.tiles : nullptr, kSplitK ? g_ws.counters : nullptr);
+}
+
+// How many shares of K make `tiles` output tiles (of tile_floats each) fill the chip: doubled while the blocks
+// stay within two per compute unit, every share keeps at least four slabs and the partial tiles fit the workspace.
+static int k_shares(int64_t tiles, int64_t tile_floats, int K) {
+  const Workspace& g_ws = workspace();
+  if (g_ws.tiles == nullptr || tiles > kGemmCounters) return 1;
+  const int slabs = (K + TK - 1) / TK;
+  int shares = 1;
+  while (shares < 16 && tiles * shares * 2 <= 512 && slabs / (shares * 2) >= 4 && tiles * shares * 2 * tile_floats <= g_ws.tile_floats)
+    shares *= 2;
+  return shares;
+}
+
 template <int kEpilogue, typename TO>
 static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                        const float* bias, int M, int N, int K, hipStream_t stream) {
-  // Big tiles (one slab ahead) when they fill the chip: about two blocks per compute unit, which hide one
-  // another's waits. Small tiles (two slabs ahead) otherwise: few big tiles, each alone on its compute
-  // unit, were slower here even with four slabs ahead.
-  const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
-  if (kEpilogue == kMfSwiglu || big_blocks >= 512) {
-    constexpr int cols = (kEpilogue == kMfSwiglu) ? 64 : 128;
-    dim3 grid((N + cols - 1) / cols, (M + 127) / 128);
-    gemm_mfma_kernel<kEpilogue, TO, 2, 1><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
-                                                                     static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2),
-                                                                     ldw, bias, M, N, K);
+  if constexpr (kEpilogue == kMfSwiglu) {
+    // Tiles of 128 rows unless they are fewer than the compute units or half empty. (A tile of 128 x 128
+    // outputs, 256 rows of W, leaves room for one block per compute unit only: slower.)
+    if (M > 64 && static_cast<int64_t>((N + 63) / 64) * ((M + 127) / 128) >= 256) {
+      dim3 grid((N + 63) / 64, (M + 127) / 128);
+      launch_tile<kEpilogue, TO, 2, 2, 1, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+    } else {
+      dim3 grid((N + 63) / 64, (M + 63) / 64);
+      launch_tile<kEpilogue, TO, 1, 2, 2, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+    }
+    return check_launch("gemm_mfma");
   } else {
-    constexpr int kE = (kEpilogue == kMfSwiglu) ? kMfStore : kEpilogue;   // (never taken for swiglu)
-    dim3 grid((N + 63) / 64, (M + 63) / 64);
-    gemm_mfma_kernel<kE, TO, 1, 2><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda,
-                                                              static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw,
-                                                              bias, M, N, K);
+    // Big tiles (one slab ahead) when they fill the chip: about two blocks per compute unit, which hide one
+    // another's waits. Small tiles (two slabs ahead) otherwise: few big tiles, each alone on its compute
+    // unit, were slower here even with four slabs ahead. Where even the small tiles are too few, K is
+    // shared out among blocks as well.
+    const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
+    if (big_blocks >= 512) {
+      dim3 grid((N + 127) / 128, (M + 127) / 128);
+      launch_tile<kEpilogue, TO, 2, 2, 1, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+    } else {
+      dim3 grid((N + 63) / 64, (M + 63) / 64);
+      const int shares = k_shares(static_cast<int64_t>(grid.x) * grid.y, 64 * 64, K);
+      if (shares > 1) {
+        grid.z = shares;
+        launch_tile<kEpilogue, TO, 1, 1, 2, true>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      } else {
+        launch_tile<kEpilogue, TO, 1, 1, 2, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      }
+    }
+    return check_launch("gemm_mfma");
   }
-  return check_launch("gemm_mfma");
 }
 
 }  // namespace alofa

@@ -130,6 +130,38 @@ SKINNY_MAX_ROWS = 64
 SWIGLU = 2
 
 
+def few_rows_kernel(M: int, w_rows: int, K: int) -> str:
+    """Which bfloat16 product takes ``M`` rows against ``w_rows`` rows of weights
+    (gate and up together for the fused feed-forward entry): ``"stream"``, every
+    wave reading its own operands straight from memory (M <= 64 only), or
+    ``"tiled"``, blocks that share both operands through LDS.
+
+    The streaming kernel reads the rows of ``a`` once per 16 or 32 weight rows, so
+    its time grows with M; the tiled kernel's hardly does, but it needs more work
+    per block to get going. Measured on one MI355X at the projection sizes of
+    0.5B, 7B and 32B models, the tiled kernel wins from these weight sizes on
+    (w_rows * K, in elements): 64 M at 5..8 rows, 24 M at 9..16 rows, 10 M above."""
+    if M > SKINNY_MAX_ROWS:
+        return "tiled"
+    elements = w_rows * K
+    if M <= 4:
+        return "stream"
+    if M <= 8:
+        return "tiled" if elements >= 64 << 20 else "stream"
+    if M <= 16:
+        return "tiled" if elements >= 24 << 20 else "stream"
+    return "tiled" if elements >= 10 << 20 else "stream"
+
+
+def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int) -> str:
+    kernel = kernel or few_rows_kernel(M, w_rows, K)
+    if kernel == "stream" and M <= SKINNY_MAX_ROWS:
+        return "alofa_gemm_skinny"
+    if kernel == "tiled":
+        return "alofa_gemm_mfma"
+    raise AlofaError("invalid_argument", "no such product kernel for these rows", f"kernel={kernel} M={M}")
+
+
 _workspace_ready = False
 
 
@@ -154,9 +186,10 @@ def _mfma_operands(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         add_to_out: bool = False, exact: bool = False) -> None:
+         add_to_out: bool = False, exact: bool = False, kernel: Optional[str] = None) -> None:
     """out = a @ w.T (+ bias), or out += a @ w.T when ``add_to_out`` (out is then
-    the float32 residual stream). w is [out_features, in_features]."""
+    the float32 residual stream). w is [out_features, in_features]. ``kernel``
+    names the bfloat16 kernel ("stream" or "tiled") instead of ``few_rows_kernel``."""
     _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w", w, None, 2)
     M, K = a.shape
     N = w.shape[0]
@@ -170,8 +203,7 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
         raise AlofaError("invalid_argument", "the residual stream is float32", f"out={out.dtype}")
     if not exact and _mfma_operands(a, w):
         _ensure_workspace(a.device)
-        # few rows: the weight-streaming kernel; many rows: the tiled one
-        _call("alofa_gemm_skinny" if M <= SKINNY_MAX_ROWS else "alofa_gemm_mfma", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
+        _call(_product_entry(kernel, M, N, K), _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
               _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(None if add_to_out else bias), _I(M), _I(N), _I(K),
               _I(ADD_TO_RESIDUAL if add_to_out else STORE), _stream())
         return
@@ -180,8 +212,9 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
           _I(ADD_TO_RESIDUAL if add_to_out else STORE), _I(int(exact)), _stream())
 
 
-def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, exact: bool = False) -> None:
-    """out = silu(a @ w_gate.T) * (a @ w_up.T)."""
+def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, exact: bool = False,
+                kernel: Optional[str] = None) -> None:
+    """out = silu(a @ w_gate.T) * (a @ w_up.T). ``kernel`` as for ``gemm``."""
     _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w_gate", w_gate, None, 2), _gpu("w_up", w_up, None, 2)
     M, K = a.shape
     N = w_gate.shape[0]
@@ -190,7 +223,8 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: 
     if w_gate.dtype is not w_up.dtype or _rows("w_gate", w_gate) != _rows("w_up", w_up):
         raise AlofaError("invalid_argument", "gate and up matrices must share dtype and layout")
     if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up):
-        _call("alofa_gemm_skinny" if M <= SKINNY_MAX_ROWS else "alofa_gemm_mfma", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
+        _ensure_workspace(a.device)
+        _call(_product_entry(kernel, M, 2 * N, K), _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
               _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), _stream())
         return
     _call("alofa_gemm_swiglu_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),

@@ -8,6 +8,7 @@ import torch
 
 from plain import model as pm
 from plain import sampler as ps
+from alofa_amd.errors import AlofaError
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -86,21 +87,30 @@ def test_gemm_exact(M, N, K):
     assert torch.equal(one[0], out[M - 1])
 
 
-@pytest.mark.parametrize("M,N,K", SHAPES)
-def test_gemm_bf16(M, N, K):
+# shapes whose few tiles make the tiled kernel share K out among blocks as well
+DEEP_SHAPES = [(40, 130, 1000), (9, 64, 4864), (130, 200, 2056), (64, 896, 672)]
+
+
+@pytest.mark.parametrize("kernel", ["stream", "tiled"])
+@pytest.mark.parametrize("M,N,K", SHAPES + DEEP_SHAPES)
+def test_gemm_bf16(M, N, K, kernel):
+    if kernel == "stream" and M > ops().SKINNY_MAX_ROWS:
+        pytest.skip("the streaming kernel takes at most 64 rows")
     rng = np.random.default_rng(3)
     a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
     b = rng.standard_normal(N).astype(np.float32)
     out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
-    ops().gemm(out, t(a, torch.bfloat16), t(w, torch.bfloat16), t(b))
+    ops().gemm(out, t(a, torch.bfloat16), t(w, torch.bfloat16), t(b), kernel=kernel)
     close(out, pm.linear(a, w, b), BF16, "bf16 out")
     outf = torch.empty(M, N, device=DEV)
-    ops().gemm(outf, t(a, torch.bfloat16), t(w, torch.bfloat16))
+    ops().gemm(outf, t(a, torch.bfloat16), t(w, torch.bfloat16), kernel=kernel)
     close(outf, pm.linear(a, w), 1e-4, "f32 out")
     res = rng.standard_normal((M, N)).astype(np.float32)
     acc = t(res)
-    ops().gemm(acc, t(a, torch.bfloat16), t(w, torch.bfloat16), add_to_out=True)
+    ops().gemm(acc, t(a, torch.bfloat16), t(w, torch.bfloat16), add_to_out=True, kernel=kernel)
     close(acc, pm.add(res, pm.linear(a, w)), 1e-4, "residual")
+    if kernel == "tiled":
+        return
     # a weight stored in float32 stays float32 and is multiplied as such
     outw = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
     w32 = rng.standard_normal((N, K)).astype(np.float32) * 0.1
@@ -115,17 +125,18 @@ def test_gemm_split_over_blocks_is_repeatable():
     of different shapes alternate, so that what the workspace held before is never the answer."""
     rng = np.random.default_rng(40)
     cases = []
-    for M, N, K in [(3, 1082, 672), (40, 864, 672), (5, 672, 4864), (2, 144, 2048)]:
+    for M, N, K, kernel in [(3, 1082, 672, "stream"), (40, 864, 672, "stream"), (5, 672, 4864, "stream"), (2, 144, 2048, "stream"),
+                            (40, 864, 672, "tiled"), (150, 672, 4864, "tiled"), (20, 144, 2048, "tiled")]:
         a = t(bf(rng.standard_normal((M, K)).astype(np.float32)), torch.bfloat16)
         w = t(bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1), torch.bfloat16)
         out = torch.empty(M, N, device=DEV)
-        ops().gemm(out, a, w)
-        cases.append((a, w, out, out.clone()))
-        close(out, pm.linear(a.float().cpu().numpy(), w.float().cpu().numpy()), 1e-4, f"{M}x{N}x{K}")
+        ops().gemm(out, a, w, kernel=kernel)
+        cases.append((a, w, out, out.clone(), kernel))
+        close(out, pm.linear(a.float().cpu().numpy(), w.float().cpu().numpy()), 1e-4, f"{M}x{N}x{K} {kernel}")
     differing = torch.zeros((), dtype=torch.int64, device=DEV)
-    for _ in range(1500):
-        for a, w, out, first in cases:
-            ops().gemm(out, a, w)
+    for _ in range(1000):
+        for a, w, out, first, kernel in cases:
+            ops().gemm(out, a, w, kernel=kernel)
             differing += (out != first).sum()
     assert int(differing) == 0
 
@@ -139,8 +150,11 @@ def test_gemm_takes_a_strided_view():
     close(out, pm.linear(big[:, 100:200], w), EXACT)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 176, 64), (37, 200, 240), (130, 97, 80), (257, 176, 200)])
-def test_gemm_swiglu(M, N, K):
+@pytest.mark.parametrize("kernel", ["stream", "tiled"])
+@pytest.mark.parametrize("M,N,K", [(1, 176, 64), (37, 200, 240), (64, 130, 264), (130, 97, 80), (257, 176, 200), (300, 20000, 72)])
+def test_gemm_swiglu(M, N, K, kernel):
+    if kernel == "stream" and M > ops().SKINNY_MAX_ROWS:
+        pytest.skip("the streaming kernel takes at most 64 rows")
     rng = np.random.default_rng(5)
     a = rng.standard_normal((M, K)).astype(np.float32)
     wg, wu = rng.standard_normal((N, K)).astype(np.float32), rng.standard_normal((N, K)).astype(np.float32)
@@ -149,7 +163,7 @@ def test_gemm_swiglu(M, N, K):
     close(out, pm.swiglu(pm.linear(a, wg), pm.linear(a, wu)), EXACT, "exact")
     ab, gb, ub = bf(a), bf(wg * 0.2), bf(wu * 0.2)
     outb = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
-    ops().gemm_swiglu(outb, t(ab, torch.bfloat16), t(gb, torch.bfloat16), t(ub, torch.bfloat16))
+    ops().gemm_swiglu(outb, t(ab, torch.bfloat16), t(gb, torch.bfloat16), t(ub, torch.bfloat16), kernel=kernel)
     close(outb, pm.swiglu(pm.linear(ab, gb), pm.linear(ab, ub)), BF16, "bf16")
     g, u = rng.standard_normal((M, N)).astype(np.float32) * 8, rng.standard_normal((M, N)).astype(np.float32)
     g[0, 0] = -1e4                                                     # far negative gate: 0, not NaN
@@ -426,3 +440,15 @@ def test_kernels_refuse_what_they_cannot_take():
         o.rmsnorm(torch.empty(2, 8, device=DEV, dtype=torch.bfloat16), torch.empty(2, 8, device=DEV), torch.empty(8, device=DEV), 1e-6, True)
     with pytest.raises(AlofaError):
         o.argmax(torch.empty(2, dtype=torch.int32, device=DEV), torch.empty(3, 8, device=DEV))
+
+
+def test_product_kernel_choice():
+    """The choice between the two bfloat16 products: few rows and small weights stream, many
+    rows or big weights are tiled; a kernel that cannot take the rows is an error, not a guess."""
+    o = ops()
+    assert o.few_rows_kernel(1, 151936, 896) == "stream" and o.few_rows_kernel(8, 151936, 896) == "tiled"
+    assert o.few_rows_kernel(64, 2 * 4864, 896) == "stream" and o.few_rows_kernel(32, 3584, 3584) == "tiled"
+    assert o.few_rows_kernel(65, 8, 8) == "tiled"
+    a, w = torch.zeros(70, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(16, 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(AlofaError):
+        o.gemm(torch.empty(70, 16, device=DEV), a, w, kernel="stream")
