@@ -13,7 +13,7 @@
 // ascending k, whatever M is.
 //
 // Where even the small tiles are too few for the chip (few rows, few columns, a
-// long K), blockIdx.z shares K out as well: every block leaves its partial tile
+// long K), K is shared out among blocks as well: every block leaves its partial tile
 // in the workspace, and the one that arrives last adds them in a fixed order and
 // runs the epilogue (the protocol of the streaming kernel, see there).
 //
@@ -36,25 +36,51 @@ enum MfmaEpilogue : int { kMfStore = 0, kMfResidual = 1, kMfSwiglu = 2 };
 constexpr int TK = 64, PAD = 8;
 constexpr int kRow = TK + PAD;  // LDS row length in elements
 
+// Which tile a block computes. The chip is eight dies, each with an L2 of its own, and blocks go to the
+// dies in turn (block i to die i % 8). Dealt out row by row, every die computes tiles from all over the
+// output and pulls all of A and all of W through its L2: fine while both fit there, and measured a few
+// percent faster then than the path below; with operands beyond the L2s (projections of 7B-sized models
+// and up) it costs up to a fifth of the time. For those (by_die) the tiles are numbered along a path that
+// stays within squares of 8 x 8 tiles (8 tile rows at a time, column by column), every die takes one
+// contiguous stretch of the path, and the blocks resident on a die together share a handful of A and W
+// panels. With K shared out, the shares are the slowest index (blocks of different shares have nothing
+// in common).
+struct TilePlace {
+  int bm, bn, share;
+};
+__device__ __forceinline__ TilePlace place_tile(int block, int tiles_m, int tiles_n, int shares, bool by_die) {
+  constexpr int kDies = 8, kGroup = 8;
+  const int tiles = tiles_m * tiles_n, total = tiles * shares;
+  if (!by_die) return {block % tiles / tiles_n, block % tiles_n, block / tiles};
+  const int die = block % kDies, local = block / kDies;
+  const int step = die * (total / kDies) + min(die, total % kDies) + local;   // dies before this one hold that many blocks
+  const int t = step % tiles;
+  const int per_group = kGroup * tiles_n, first_m = (t / per_group) * kGroup, within = t % per_group;
+  const int rows = min(tiles_m - first_m, kGroup);
+  return {first_m + within % rows, within / rows, step / tiles};
+}
+
 // WTM, WTN: MFMA tiles per wave along m and along n; the block tile is 64 WTM x 64 WTN.
 // PF: slabs on their way from memory while another is being multiplied.
-// kSplitK: blockIdx.z takes a share of K; the shares meet in the workspace (see below).
+// kSplitK: a block takes a share of K; the shares meet in the workspace (see below).
 template <int kEpilogue, typename TO, int WTM, int WTN, int PF, bool kSplitK>
 __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, int64_t ldo,
                                                         const bf16_t* __restrict__ A, int64_t lda,
                                                         const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
                                                         int64_t ldw, const float* __restrict__ bias, int M, int N,
-                                                        int K_all, float* __restrict__ ws, int* __restrict__ counters) {
+                                                        int K_all, int tiles_m, int tiles_n, int shares,
+                                                        float* __restrict__ ws, int* __restrict__ counters, int by_die) {
   constexpr int TM = 64 * WTM, TN = 64 * WTN;
   // swiglu: the first half of a wave's column tiles are gate columns, the second half the up columns of the same outputs
   constexpr int kGateTiles = WTN / 2;
   static_assert(kEpilogue != kMfSwiglu || WTN % 2 == 0, "the swiglu epilogue needs an even number of column tiles per wave");
   __shared__ int last_block;
+  const TilePlace place = place_tile(blockIdx.x, tiles_m, tiles_n, shares, by_die != 0);
   // this block's share of K: slabs [k_begin, K)
   int k_begin = 0, K = K_all;
   if (kSplitK) {
-    const int slabs = (K_all + TK - 1) / TK, per_split = (slabs + static_cast<int>(gridDim.z) - 1) / static_cast<int>(gridDim.z);
-    k_begin = blockIdx.z * per_split * TK;
+    const int slabs = (K_all + TK - 1) / TK, per_split = (slabs + shares - 1) / shares;
+    k_begin = place.share * per_split * TK;
     K = min(K_all, k_begin + per_split * TK);
   }
   __shared__ __attribute__((aligned(16))) bf16_t As[TM * kRow];
@@ -62,7 +88,7 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int wm = wave / 2, wn = wave % 2;
   constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
-  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * kOutCols;
+  const int m0 = place.bm * TM, n0 = place.bn * kOutCols;
 
   // global -> register staging: 8 chunks of 16 bytes per slab row; a thread takes row (tid + 256 j) / 8
   constexpr int NCA = WTM * 2, NCW = WTN * 2;
@@ -170,9 +196,9 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
     // through to memory, where blocks on every die find it) and is counted once every wave's stores have
     // been acknowledged; the block counted last adds the tiles in split order, so the sum is the same on
     // every run, goes on to the epilogue and puts the counter back to zero.
-    const int splits = gridDim.z, tile_id = blockIdx.y * gridDim.x + blockIdx.x;
+    const int splits = shares, tile_id = place.bm * tiles_n + place.bn;
     constexpr int kTileFloats = WTM * WTN * 16 * 256;
-    float* mine = ws + (static_cast<int64_t>(tile_id) * splits + blockIdx.z) * kTileFloats;
+    float* mine = ws + (static_cast<int64_t>(tile_id) * splits + place.share) * kTileFloats;
 #pragma unroll
     for (int i = 0; i < WTM; ++i)
 #pragma unroll
@@ -248,12 +274,16 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 }
 
 template <int kEpilogue, typename TO, int WTM, int WTN, int PF, bool kSplitK>
-static void launch_tile(dim3 grid, void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
+static void launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                         const float* bias, int M, int N, int K, hipStream_t stream) {
   const Workspace& g_ws = workspace();
-  gemm_mfma_kernel<kEpilogue, TO, WTM, WTN, PF, kSplitK><<<grid, 256, 0, stream>>>(
+  // operands beyond what the eight L2s hold together (4 MB each)
+  const int w_rows = (kEpilogue == kMfSwiglu) ? 2 * N : N;
+  const int by_die = (static_cast<int64_t>(M) + w_rows) * K * 2 > (32 << 20);
+  gemm_mfma_kernel<kEpilogue, TO, WTM, WTN, PF, kSplitK><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
-      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, kSplitK ? g_ws.tiles : nullptr, kSplitK ? g_ws.counters : nullptr);
+      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, tiles_m, tiles_n, shares, kSplitK ? g_ws.tiles : nullptr,
+      kSplitK ? g_ws.counters : nullptr, by_die);
 }
 
 // How many shares of K make `tiles` output tiles (of tile_floats each) fill the chip: doubled while the blocks
@@ -275,11 +305,9 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     // Tiles of 128 rows unless they are fewer than the compute units or half empty. (A tile of 128 x 128
     // outputs, 256 rows of W, leaves room for one block per compute unit only: slower.)
     if (M > 64 && static_cast<int64_t>((N + 63) / 64) * ((M + 127) / 128) >= 256) {
-      dim3 grid((N + 63) / 64, (M + 127) / 128);
-      launch_tile<kEpilogue, TO, 2, 2, 1, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 63) / 64, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
     } else {
-      dim3 grid((N + 63) / 64, (M + 63) / 64);
-      launch_tile<kEpilogue, TO, 1, 2, 2, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 63) / 64, (M + 63) / 64, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
     }
     return check_launch("gemm_mfma");
   } else {
@@ -289,16 +317,14 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     // shared out among blocks as well.
     const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
     if (big_blocks >= 512) {
-      dim3 grid((N + 127) / 128, (M + 127) / 128);
-      launch_tile<kEpilogue, TO, 2, 2, 1, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 127) / 128, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
     } else {
-      dim3 grid((N + 63) / 64, (M + 63) / 64);
-      const int shares = k_shares(static_cast<int64_t>(grid.x) * grid.y, 64 * 64, K);
+      const int tiles_n = (N + 63) / 64, tiles_m = (M + 63) / 64;
+      const int shares = k_shares(static_cast<int64_t>(tiles_n) * tiles_m, 64 * 64, K);
       if (shares > 1) {
-        grid.z = shares;
-        launch_tile<kEpilogue, TO, 1, 1, 2, true>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+        launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
       } else {
-        launch_tile<kEpilogue, TO, 1, 1, 2, false>(grid, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+        launch_tile<kEpilogue, TO, 1, 1, 2, false>(tiles_n, tiles_m, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
       }
     }
     return check_launch("gemm_mfma");

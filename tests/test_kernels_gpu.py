@@ -452,3 +452,22 @@ def test_product_kernel_choice():
     a, w = torch.zeros(70, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(16, 64, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(AlofaError):
         o.gemm(torch.empty(70, 16, device=DEV), a, w, kernel="stream")
+
+
+def test_gemm_with_operands_beyond_the_l2():
+    """Operands of more than 32 MB make the tiled kernel deal its tiles out die by die (another
+    numbering of the blocks): every tile must still be computed exactly once, with K shared out
+    among blocks and with the SwiGLU epilogue too."""
+    rng = np.random.default_rng(41)
+    for M, N, K in [(130, 9000, 2048), (40, 1100, 16384)]:
+        a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.05)
+        res = rng.standard_normal((M, N)).astype(np.float32)
+        acc = t(res)
+        ops().gemm(acc, t(a, torch.bfloat16), t(w, torch.bfloat16), add_to_out=True, kernel="tiled")
+        close(acc, pm.add(res, pm.linear(a, w)), 1e-4, f"residual {M}x{N}x{K}")
+    M, N, K = 70, 4200, 2048
+    a = bf(rng.standard_normal((M, K)).astype(np.float32))
+    g, u = bf(rng.standard_normal((N, K)).astype(np.float32) * 0.03), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.03)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm_swiglu(out, t(a, torch.bfloat16), t(g, torch.bfloat16), t(u, torch.bfloat16), kernel="tiled")
+    close(out, pm.swiglu(pm.linear(a, g), pm.linear(a, u)), BF16, "swiglu")
