@@ -176,18 +176,35 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
     }
   };
 
+  // The slabs set out in the order in which they are needed, and the compiler may not change it: the
+  // loads of a wave complete in order, and the wait for slab p must leave the later ones on their way.
 #pragma unroll
-  for (int p = 0; p < PF; ++p) fetch(a_reg[p], w_reg[p], k_begin + p * TK);
-  for (int k0 = k_begin; k0 < K; k0 += PF * TK) {
+  for (int p = 0; p < PF; ++p) {
+    fetch(a_reg[p], w_reg[p], k_begin + p * TK);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // Whole rounds of PF slabs first, without a branch inside: a slab that could be skipped would make the
+  // compiler wait for every load at the next one (on the path past it the loads just issued are the
+  // youngest). The last, partial round follows the loop and sets no further loads out.
+  int k0 = k_begin;
+  for (; k0 + (PF - 1) * TK < K; k0 += PF * TK) {
 #pragma unroll
     for (int p = 0; p < PF; ++p) {
-      if (k0 + p * TK < K) {    // uniform over the block
-        __syncthreads();        // the previous slab has been read by every wave
-        stage(a_reg[p], w_reg[p], k0 + p * TK);
-        __syncthreads();
-        fetch(a_reg[p], w_reg[p], k0 + (p + PF) * TK);
-        multiply();
-      }
+      __builtin_amdgcn_sched_barrier(0);   // (nor may slab p's staging, and with it the wait for its loads, move up into the step before)
+      __syncthreads();        // the previous slab has been read by every wave
+      stage(a_reg[p], w_reg[p], k0 + p * TK);
+      __syncthreads();
+      fetch(a_reg[p], w_reg[p], k0 + (p + PF) * TK);
+      multiply();
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < PF - 1; ++p) {
+    if (k0 + p * TK < K) {    // uniform over the block
+      __syncthreads();
+      stage(a_reg[p], w_reg[p], k0 + p * TK);
+      __syncthreads();
+      multiply();
     }
   }
 
