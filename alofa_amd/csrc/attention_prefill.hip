@@ -91,69 +91,86 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
   const int first_key = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
   const int t_begin = first_key / BKV, t_end = last_pos / BKV;     // inclusive
 
-  // staging: 16-byte chunks, 64 * d / 8 of K (eight channels of a key) and as many of V^T (eight keys of a channel)
+  // staging: 16-byte chunks, 64 * d / 8 of K (eight channels of a key) and as many of V^T (eight keys of a
+  // channel; one page: pages hold at least eight tokens). Every lane issues every load, from a visible key
+  // in place of one that is not (what such a load brings is cleared at staging): loads that are always
+  // issued can stay on their way while the tile before is worked on, a load under a branch is waited for at
+  // once. The page numbers of a tile are looked up one tile ahead of its keys and values for the same reason.
   constexpr int kChunks = BKV * d / 8;
   constexpr int kPerThread = (kChunks + 255) / 256;
+  const int page_mask = (1 << bs_shift) - 1;
+  const int v_first = first_key & ~7, v_last = last_pos & ~7;    // first and last visible group of eight keys
   uint4 k_reg[kPerThread], v_reg[kPerThread];
+  int k_page[kPerThread], v_page[kPerThread];
+  auto chunk_of = [&](int j) { const int c = tid + 256 * j; return c < kChunks ? c : kChunks - 1; };
+  auto k_key = [&](int t, int j) { return t * BKV + chunk_of(j) / (d / 8); };
+  auto v_key0 = [&](int t, int j) { return t * BKV + (chunk_of(j) % 8) * 8; };
+  auto clamp = [](int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); };
+  auto lookup = [&](int t) {
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) {
+      k_page[j] = table[clamp(k_key(t, j), first_key, last_pos) >> bs_shift];
+      v_page[j] = table[clamp(v_key0(t, j), v_first, v_last) >> bs_shift];
+    }
+  };
   auto fetch = [&](int t) {
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
-      const int c = tid + 256 * j;
-      k_reg[j] = v_reg[j] = make_uint4(0, 0, 0, 0);
-      if (c < kChunks) {
-        const int key = t * BKV + c / (d / 8), ch = (c % (d / 8)) * 8;
-        if (key <= last_pos && key >= first_key) {
-          // pages hold a power of two of tokens: block = key >> shift, slot = key & mask
-          const int64_t blk = table[key >> bs_shift];
-          const int64_t base = ((((blk * kv_heads + hk) << bs_shift) + (key & ((1 << bs_shift) - 1))) * d) + ch;
-          k_reg[j] = *reinterpret_cast<const uint4*>(k_cache + base);
-        }
-        // keys key0 .. key0 + 7 of channel c / 8 (one page: pages hold at least eight tokens)
-        const int key0 = t * BKV + (c % 8) * 8, channel = c / 8;
-        if (key0 <= last_pos && key0 + 7 >= first_key) {
-          const int64_t blk = table[key0 >> bs_shift];
-          const int64_t base = (((blk * kv_heads + hk) * d + channel) << bs_shift) + (key0 & ((1 << bs_shift) - 1));
-          uint4 v = *reinterpret_cast<const uint4*>(v_cache + base);
-          // what lies beyond the visible keys is not data: it is cleared, so that a weight of zero times it is zero
-          const int lo_e = first_key - key0, hi_e = last_pos - key0 + 1;   // elements lo_e .. hi_e - 1 are visible
-          if (lo_e > 0 || hi_e < 8) {
-            uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-              if (e < lo_e || e >= hi_e) w[e / 2] &= (e % 2) ? 0x0000ffffu : 0xffff0000u;
-            v = make_uint4(w[0], w[1], w[2], w[3]);
-          }
-          v_reg[j] = v;
-        }
-      }
+      const int c = chunk_of(j);
+      const int key = clamp(k_key(t, j), first_key, last_pos), ch = (c % (d / 8)) * 8;
+      k_reg[j] = *reinterpret_cast<const uint4*>(
+          k_cache + ((((static_cast<int64_t>(k_page[j]) * kv_heads + hk) << bs_shift) + (key & page_mask)) * d) + ch);
+      const int key0 = clamp(v_key0(t, j), v_first, v_last), channel = c / 8;
+      v_reg[j] = *reinterpret_cast<const uint4*>(
+          v_cache + (((static_cast<int64_t>(v_page[j]) * kv_heads + hk) * d + channel) << bs_shift) + (key0 & page_mask));
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](int t) {
+    // all 64 keys of the tile visible to the block (all but its first and last tiles): nothing to clear
+    const bool whole = t * BKV >= first_key && t * BKV + BKV - 1 <= last_pos;   // uniform over the team
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
       const int c = tid + 256 * j;
       if (c < kChunks) {
-        const int key = c / (d / 8), ch = (c % (d / 8)) * 8;
-        *reinterpret_cast<uint4*>(&Ks[key * KROW + ch]) = k_reg[j];
+        uint4 kv = k_reg[j], vv = v_reg[j];
+        if (!whole) {
+          // what lies beyond the visible keys is not data: it is cleared, so that a weight of zero times it is zero
+          const int key = k_key(t, j);
+          const uint32_t kk = 0u - static_cast<uint32_t>(key >= first_key && key <= last_pos);   // all ones or zero
+          kv = make_uint4(kv.x & kk, kv.y & kk, kv.z & kk, kv.w & kk);
+          const int key0 = v_key0(t, j);
+          const int lo_e = first_key - key0, hi_e = last_pos - key0 + 1;   // elements lo_e .. hi_e - 1 are visible
+          uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const uint32_t keep = 0u - static_cast<uint32_t>(e >= lo_e && e < hi_e);
+            w[e / 2] &= (e % 2) ? (keep << 16) | 0x0000ffffu : keep | 0xffff0000u;
+          }
+          vv = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+        *reinterpret_cast<uint4*>(&Ks[(c / (d / 8)) * KROW + (c % (d / 8)) * 8]) = kv;
         // row c / 8 of V^T, keys 8 (c % 8) .. + 7. Groups of four keys are permuted within a row by the row's
         // number / 8, so that lanes reading rows r and r + 8 hit different banks: the two groups of this chunk
         // stay in their 16 bytes and change places when that number is odd.
         const int sw = ((c / 8) >> 3) & 7;
-        const uint4 v = (sw & 1) ? make_uint4(v_reg[j].z, v_reg[j].w, v_reg[j].x, v_reg[j].y) : v_reg[j];
-        *reinterpret_cast<uint4*>(&Vt[(c / 8) * VROW + ((((c % 8) * 2) ^ (sw & 6)) << 2)]) = v;
+        if (sw & 1) vv = make_uint4(vv.z, vv.w, vv.x, vv.y);
+        *reinterpret_cast<uint4*>(&Vt[(c / 8) * VROW + ((((c % 8) * 2) ^ (sw & 6)) << 2)]) = vv;
       }
     }
   };
 
-  if (t_begin + team <= t_end) fetch(t_begin + team);
+  lookup(t_begin + team);
+  fetch(t_begin + team);
+  lookup(t_begin + team + TEAMS);
   for (int t0 = t_begin; t0 <= t_end; t0 += TEAMS) {     // uniform over the block
     const int t = t0 + team;
     const bool mine = t <= t_end;
     __syncthreads();      // the previous tile has been read by every wave
-    if (mine) stage();
+    if (mine) stage(t);
     __syncthreads();
     if (!mine) continue;
-    if (t + TEAMS <= t_end) fetch(t + TEAMS);
+    fetch(t + TEAMS);
+    lookup(t + 2 * TEAMS);
 
     // S^T for the four 16-key quarters of the tile
     f32x4 s[4];

@@ -74,7 +74,8 @@ class StepContext:
         # up to 64 rows. short_rows is None when every row is short.
         self.n_short = sum(s.n for s in spans if s.n <= SHORT)
         self.short_rows: Optional[torch.Tensor] = None
-        self.long_tiles: Optional[torch.Tensor] = None
+        self.long_runs: Optional[list] = None         # (request index, first row, rows <= 64, first position) per tile of rows
+        self._long_tiles: dict = {}
         self.entry_slots = self.entry_tokens = None   # request slot and token count per entry, as arrays
         self.positions: torch.Tensor = None
         self.req_of_token: torch.Tensor = None
@@ -83,6 +84,15 @@ class StepContext:
 
     def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
         return self.fn.scratch(name, shape, dtype)
+
+    def prefill_tiles(self, heads: int, window: Optional[int] = None) -> torch.Tensor:
+        """The runs of rows of this step's prompt portions as blocks for the prefill
+        attention kernel, for a mixer with ``heads`` query heads (how the runs share
+        blocks depends on how many blocks there are): built once per step and kind."""
+        key = (heads, window)
+        if key not in self._long_tiles:
+            self._long_tiles[key] = torch.tensor(ops.pair_tiles(self.long_runs, window, heads), dtype=torch.int32, device=self.fn.device)
+        return self._long_tiles[key]
 
     def kv(self, entry: int) -> KVView:
         owner_entry = self.fn.cache_entry[entry]
@@ -206,9 +216,8 @@ class StepFunction:
         ctx._slots = [slots_d[g] for g in range(n_groups)]
         rows = torch.tensor(want_rows, dtype=torch.int32, device=dev) if want_rows else None
         if ctx.n_short < T:
-            tiles = [(i, s.row0 + q0, min(TILE_ROWS, s.n - q0), s.pos0 + q0)
-                     for i, s in enumerate(spans) if s.n > SHORT for q0 in range(0, s.n, TILE_ROWS)]
-            ctx.long_tiles = torch.tensor(ops.pair_tiles(tiles), dtype=torch.int32, device=dev)
+            ctx.long_runs = [(i, s.row0 + q0, min(TILE_ROWS, s.n - q0), s.pos0 + q0)
+                             for i, s in enumerate(spans) if s.n > SHORT for q0 in range(0, s.n, TILE_ROWS)]
             if ctx.n_short:
                 ctx.short_rows = torch.tensor([r for s in spans if s.n <= SHORT for r in range(s.row0, s.row0 + s.n)],
                                               dtype=torch.int32, device=dev)

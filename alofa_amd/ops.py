@@ -422,11 +422,27 @@ def can_fuse_rope_into_decode(d: int) -> bool:
 PREFILL_HEAD_DIMS = (16, 32, 48, 64, 96, 128, 256)
 
 
-def pair_tiles(runs: list, window: Optional[int] = None) -> list:
+_compute_units: Optional[int] = None
+
+
+def compute_units() -> int:
+    global _compute_units
+    if _compute_units is None:
+        _compute_units = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+    return _compute_units
+
+
+def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = None) -> list:
     """``runs``: (request index, first row, rows <= 64, position of the first
-    row) per run of rows. Returns per block two runs (the second may be empty):
-    the run that walks the most key tiles shares a block with the one that
-    walks the fewest, and so on, so that blocks carry about the same work."""
+    row) per run of rows. Returns per block two runs (the second may be empty).
+    When there are more blocks (runs x ``heads``) than compute units, the run
+    that walks the most key tiles shares a block with the one that walks the
+    fewest, and so on, so that blocks carry about the same work; with fewer,
+    every run has a block of its own (a portion deep in a long context would
+    otherwise leave most of the chip idle)."""
+    if heads is not None and len(runs) * heads <= compute_units():
+        return [[list(r), [0, 0, 0, 0]] for r in runs]
+
     def key_tiles(r):
         first = max(0, r[3] - window + 1) if window else 0
         return (r[3] + r[2] - 1) // 64 - first // 64 + 1
@@ -436,7 +452,6 @@ def pair_tiles(runs: list, window: Optional[int] = None) -> list:
         out.append([list(order[i]), list(order[j]) if j > i else [0, 0, 0, 0]])
         i, j = i + 1, j - 1
     return out
-
 
 
 def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale) -> None:

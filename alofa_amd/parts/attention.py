@@ -85,7 +85,7 @@ class GQAAttention(Mixer):
         pow2_pages = kv.k.shape[2] >= ops.MIN_FAST_PAGE and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
         fast_prefill = self.d in ops.PREFILL_HEAD_DIMS
         # one new token per request: the decode kernel rotates it and writes its cache slot itself
-        fused = (not exact and pow2_pages and kv.owner and ctx.max_q_len == 1 and ctx.long_tiles is None
+        fused = (not exact and pow2_pages and kv.owner and ctx.max_q_len == 1 and ctx.long_runs is None
                  and ops.can_fuse_rope_into_decode(self.d))
         if fused:
             pass
@@ -93,12 +93,12 @@ class GQAAttention(Mixer):
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d, kv.slots, kv.k, kv.v)
         else:
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
-        if exact or not pow2_pages or (ctx.long_tiles is not None and not fast_prefill):
+        if exact or not pow2_pages or (ctx.long_runs is not None and not fast_prefill):
             # the exact path, and page or head sizes the bfloat16 kernels are not built for
             ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
         else:
-            if ctx.long_tiles is not None:      # portions of prompts
-                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, ctx.long_tiles, *common)
+            if ctx.long_runs is not None:       # portions of prompts
+                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, ctx.prefill_tiles(self.heads, self.window), *common)
             if ctx.n_short:                     # single tokens and very short portions, all query heads of a key head together
                 floats = ops.decode_scratch_floats(ctx.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
                 partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None

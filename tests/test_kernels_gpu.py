@@ -360,11 +360,16 @@ def test_prefill_attention(heads, kv_heads, d, bs, window):
         row += n
     out = torch.zeros(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
     scale = float(np.float32(1) / np.sqrt(np.float32(d)))
-    paired = ops().pair_tiles(tiles, window)
-    assert sorted(tuple(r) for b in paired for r in b if r[2]) == sorted(tiles) and len(paired) == (len(tiles) + 1) // 2
-    ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(paired, np.int32), torch.int32), heads, kv_heads, d, window, scale)
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(len(lens))])
-    close(out, ref, BF16, "prefill attention")
+    # two runs per block (many blocks) and a block per run (fewer blocks than compute units)
+    paired, single = ops().pair_tiles(tiles, window), ops().pair_tiles(tiles, window, heads)
+    assert sorted(tuple(r) for b in paired for r in b if r[2]) == sorted(tiles) and len(paired) == (len(tiles) + 1) // 2
+    assert [tuple(b[0]) for b in single] == tiles and all(b[1][2] == 0 for b in single)
+    assert len(ops().pair_tiles(tiles * 40, window, heads)) == len(tiles) * 20
+    for name, blocks in (("paired", paired), ("single", single)):
+        out.zero_()
+        ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(blocks, np.int32), torch.int32), heads, kv_heads, d, window, scale)
+        close(out, ref, BF16, f"prefill attention, {name}")
 
 
 def test_prefill_attention_far_key():
