@@ -185,17 +185,25 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
         s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kv), qf[ds], s[kt], 0, 0, 0);
       }
     }
-    // scale, mask, running maximum. Scores are kept in units of log2(e) so that the
-    // weights are single exp2 instructions; tiles that every row of the block sees
-    // whole (all but the last one or two) skip the masking.
+    // scale, mask, running maximum. Scores are taken in units of log2(e) so that the weights are single
+    // exp2 instructions. Tiles that every row of the block sees whole (all but the last one or two) skip
+    // the masking: their maximum is taken over the raw scores and the scale goes into the exponent's
+    // multiply-add.
     float p[16];
     float tile_max = -FLT_MAX;
     const bool whole = t * BKV + BKV - 1 <= pos0 && (window <= 0 || t * BKV > last_pos - window);
+    float corr, sum = 0.f;
     if (whole) {
 #pragma unroll
+      for (int i = 0; i < 16; ++i) tile_max = fmaxf(tile_max, s[i / 4][i % 4]);
+      tile_max = rows_max(tile_max);     // over the four lanes that share the query row
+      const float m_new = fmaxf(m, tile_max * scale2);
+      corr = __builtin_amdgcn_exp2f(m - m_new);    // 1 while nothing was seen yet (both -FLT_MAX)
+      m = m_new;
+#pragma unroll
       for (int i = 0; i < 16; ++i) {
-        p[i] = s[i / 4][i % 4] * scale2;
-        tile_max = fmaxf(tile_max, p[i]);
+        p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i / 4][i % 4], scale2, -m_new));
+        sum += p[i];
       }
     } else {
 #pragma unroll
@@ -205,18 +213,17 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
         p[i] = seen ? s[i / 4][i % 4] * scale2 : -FLT_MAX;
         tile_max = fmaxf(tile_max, p[i]);
       }
-    }
-    tile_max = rows_max(tile_max);     // over the four lanes that share the query row
-    const float m_new = fmaxf(m, tile_max);
-    const float corr = __builtin_amdgcn_exp2f(m - m_new);    // 1 while nothing was seen yet (both -FLT_MAX)
-    m = m_new;
-    float sum = 0.f;
-    // a masked score is -FLT_MAX: its weight is 0 unless the row has seen nothing yet
-    // (m_new is then -FLT_MAX too), which the second test catches
+      tile_max = rows_max(tile_max);
+      const float m_new = fmaxf(m, tile_max);
+      corr = __builtin_amdgcn_exp2f(m - m_new);
+      m = m_new;
+      // a masked score is -FLT_MAX: its weight is 0 unless the row has seen nothing yet
+      // (m_new is then -FLT_MAX too), which the test catches
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      p[i] = (p[i] > -FLT_MAX) ? __builtin_amdgcn_exp2f(p[i] - m_new) : 0.f;
-      sum += p[i];
+      for (int i = 0; i < 16; ++i) {
+        p[i] = (p[i] > -FLT_MAX) ? __builtin_amdgcn_exp2f(p[i] - m_new) : 0.f;
+        sum += p[i];
+      }
     }
     l = l * corr + sum;   // this lane's share of the row's sum; the four lanes of a row meet at the end
     bf16x8 pf[2];
