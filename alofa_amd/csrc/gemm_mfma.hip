@@ -333,7 +333,10 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     // unit, were slower here even with four slabs ahead. Where even the small tiles are too few, K is
     // shared out among blocks as well.
     const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
-    if (big_blocks >= 512) {
+    if (M <= 64 && (N + 127) / 128 >= 256) {
+      // one tile of rows against a long matrix (the vocabulary): tiles of 64 rows, so that no empty rows are staged
+      launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 127) / 128, 1, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+    } else if (big_blocks >= 512) {
       launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 127) / 128, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
     } else {
       const int tiles_n = (N + 63) / 64, tiles_m = (M + 63) / 64;

@@ -130,7 +130,7 @@ SKINNY_MAX_ROWS = 64
 SWIGLU = 2
 
 
-def few_rows_kernel(M: int, w_rows: int, K: int) -> str:
+def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
     """Which bfloat16 product takes ``M`` rows against ``w_rows`` rows of weights
     (gate and up together for the fused feed-forward entry): ``"stream"``, every
     wave reading its own operands straight from memory (M <= 64 only), or
@@ -140,8 +140,12 @@ def few_rows_kernel(M: int, w_rows: int, K: int) -> str:
     its time grows with M; the tiled kernel's hardly does, but it needs more work
     per block to get going. Measured on one MI355X at the projection sizes of
     0.5B, 7B and 32B models, the tiled kernel wins from these weight sizes on
-    (w_rows * K, in elements): 64 M at 5..8 rows, 24 M at 9..16 rows, 10 M above."""
+    (w_rows * K, in elements): 64 M at 5..8 rows, 24 M at 9..16 rows, 10 M above;
+    and against a matrix as long as a vocabulary (256 column tiles of 128 or more)
+    from the first row on."""
     if M > SKINNY_MAX_ROWS:
+        return "tiled"
+    if not swiglu and (w_rows + 127) // 128 >= 256:
         return "tiled"
     elements = w_rows * K
     if M <= 4:
@@ -153,8 +157,8 @@ def few_rows_kernel(M: int, w_rows: int, K: int) -> str:
     return "tiled" if elements >= 10 << 20 else "stream"
 
 
-def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int) -> str:
-    kernel = kernel or few_rows_kernel(M, w_rows, K)
+def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
+    kernel = kernel or few_rows_kernel(M, w_rows, K, swiglu)
     if kernel == "stream" and M <= SKINNY_MAX_ROWS:
         return "alofa_gemm_skinny"
     if kernel == "tiled":
@@ -224,7 +228,7 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: 
         raise AlofaError("invalid_argument", "gate and up matrices must share dtype and layout")
     if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up):
         _ensure_workspace(a.device)
-        _call(_product_entry(kernel, M, 2 * N, K), _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
+        _call(_product_entry(kernel, M, 2 * N, K, True), _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
               _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), _stream())
         return
     _call("alofa_gemm_swiglu_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),

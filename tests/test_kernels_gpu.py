@@ -88,7 +88,7 @@ def test_gemm_exact(M, N, K):
 
 
 # shapes whose few tiles make the tiled kernel share K out among blocks as well
-DEEP_SHAPES = [(40, 130, 1000), (9, 64, 4864), (130, 200, 2056), (64, 896, 672)]
+DEEP_SHAPES = [(40, 130, 1000), (9, 64, 4864), (130, 200, 2056), (64, 896, 672), (3, 33000, 72), (50, 40011, 40)]   # the last two: a long matrix, 64-row tiles
 
 
 @pytest.mark.parametrize("kernel", ["stream", "tiled"])
@@ -451,7 +451,8 @@ def test_product_kernel_choice():
     """The choice between the two bfloat16 products: few rows and small weights stream, many
     rows or big weights are tiled; a kernel that cannot take the rows is an error, not a guess."""
     o = ops()
-    assert o.few_rows_kernel(1, 151936, 896) == "stream" and o.few_rows_kernel(8, 151936, 896) == "tiled"
+    assert o.few_rows_kernel(1, 151936, 896) == "tiled" and o.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "stream"
+    assert o.few_rows_kernel(4, 4608, 3584) == "stream" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
     assert o.few_rows_kernel(64, 2 * 4864, 896) == "stream" and o.few_rows_kernel(32, 3584, 3584) == "tiled"
     assert o.few_rows_kernel(65, 8, 8) == "tiled"
     a, w = torch.zeros(70, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(16, 64, device=DEV, dtype=torch.bfloat16)
