@@ -21,7 +21,7 @@ class Engine:
     by default enough for ``max_batch`` requests of ``max_tokens``."""
 
     def __init__(self, model_dir, dtype: str = "bfloat16", max_tokens: int = 256, max_batch: int = 8,
-                 kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 256, max_chunk: int = 64,
+                 kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 2048, max_chunk: int = 512,
                  watermark_permille: int = 900, max_wait_ticks: int = 8, seed: int = 1234, device: str = "cuda:0",
                  trace_path=None):
         from .csrc.build import load

@@ -36,8 +36,10 @@ def blocks_for(seq: int, block_size: int) -> int:
 
 @dataclass(frozen=True)
 class SchedConfig:
-    token_budget: int = 256
-    max_chunk: int = 64
+    # names and meanings as src/alofa/engine/scheduler.mojo:104-105; the defaults there (256 and 64) are a
+    # CPU's, these are sized for steps that keep an MI355X busy
+    token_budget: int = 2048
+    max_chunk: int = 512
     block_size: int = 16
     capacity_blocks: int = 1024
     watermark_permille: int = 900
