@@ -2,7 +2,8 @@
 the generality of the assembly: a toy mixer with state of its own, defined
 here, is registered, built from a weight file and stepped without a change to
 the engine's files; one model mixes mixers, names a layer twice in its run
-order and lets an entry read another entry's cache."""
+order and lets an entry read another entry's cache. A second toy model has a
+feed-forward with routing and a position encoding that is no rotation."""
 import dataclasses
 import json
 
@@ -254,4 +255,174 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype):
     got = collect(r, steps)                          # state slots are used again by later requests, and zeroed
     for k in requests:
         assert_close(got[k], refs[k], dtype, f"toy mixed {k}")
+    r.cache.check()
+
+
+# ------------------------------------- a toy feed-forward with routing, a toy position encoding
+
+TOY_EXPERTS = 3
+
+
+def register_toy_routed():
+    """Two more parts defined outside the engine: a feed-forward that sends every token to one
+    of several experts (router logits in float32 or wider, first maximum wins), and a position
+    encoding that is no rotation (a position-dependent wave added to queries and keys), so that
+    the attention part has to call the encoding instead of using a rotation table."""
+    from alofa_amd.config import LayerSpec, ModelConfig, ModelSpec, PartSpec, RunEntry, register_architecture
+    from alofa_amd.parts import FeedForward, PositionEncoding, register_part
+    from alofa_amd.weights import TensorRule
+
+    class RoutedExperts(FeedForward):
+        @classmethod
+        def tensors(cls, spec):
+            p = spec.params
+            pre, h, i = p["prefix"], p["hidden"], p["intermediate"]
+            rules = {pre + "router.weight": TensorRule((p["experts"], h))}
+            for e in range(p["experts"]):
+                rules[f"{pre}experts.{e}.in.weight"] = TensorRule((i, h))
+                rules[f"{pre}experts.{e}.out.weight"] = TensorRule((h, i))
+            return rules
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            p = spec.params
+            wide = torch.float64 if rt.exact else torch.float32
+            self.wide = wide
+            self.router = weights[p["prefix"] + "router.weight"].to(rt.device, wide)
+            self.w_in = [weights[f"{p['prefix']}experts.{e}.in.weight"].to(rt.device, wide) for e in range(p["experts"])]
+            self.w_out = [weights[f"{p['prefix']}experts.{e}.out.weight"].to(rt.device, wide) for e in range(p["experts"])]
+
+        def forward(self, ctx, x, residual):
+            xw = x.to(self.wide)
+            choice = torch.argmax(xw @ self.router.T, dim=1)
+            for e in range(len(self.w_in)):
+                rows = torch.nonzero(choice == e).flatten()
+                if rows.numel():
+                    y = torch.relu(xw[rows] @ self.w_in[e].T) @ self.w_out[e].T
+                    residual.index_add_(0, rows, y.to(residual.dtype))
+
+    class AddedWave(PositionEncoding):
+        """q[t, :, c] += amp * sin(pos[t] * base^(-c/d)), k[t, :, c] += amp * cos(the same angle)."""
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            d = spec.params["head_dim"]
+            self.amp = float(spec.params["amp"])
+            self.freq = torch.tensor([spec.params["base"] ** (-c / d) for c in range(d)], dtype=torch.float64, device=rt.device)
+
+        def apply(self, ctx, q, k):
+            ang = ctx.positions.to(torch.float64)[:, None] * self.freq[None, :]
+            q += (self.amp * torch.sin(ang))[:, None, :].to(q.dtype)
+            k += (self.amp * torch.cos(ang))[:, None, :].to(k.dtype)
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyRoutedConfig(ModelConfig):
+        hidden: int
+        vocab: int
+        heads: int
+        head_dim: int
+        inter: int
+        architecture = "ToyRoutedForCausalLM"
+
+        @classmethod
+        def from_dict(cls, raw, where="<dict>"):
+            return cls(raw["hidden"], raw["vocab"], raw["heads"], raw["head_dim"], raw["inter"])
+
+        def to_dict(self):
+            return dict(dataclasses.asdict(self), architectures=[self.architecture])
+
+        def spec(self):
+            h = self.hidden
+
+            def norms(p):
+                return (PartSpec("rmsnorm", {"name": p + "n0.weight", "width": h, "eps": 1e-5}),
+                        PartSpec("rmsnorm", {"name": p + "n1.weight", "width": h, "eps": 1e-5}))
+
+            def att(p, position):
+                return PartSpec("gqa_attention", {"prefix": p + "att.", "hidden": h, "heads": self.heads, "kv_heads": 1, "head_dim": self.head_dim,
+                                                  "qkv_bias": True, "out_bias": False, "window": None, "position": position})
+            layers = (LayerSpec("a.", PartSpec("prenorm"), att("a.", PartSpec("toy_added_wave", {"head_dim": self.head_dim, "amp": 0.5, "base": 50.0})),
+                                PartSpec("toy_routed", {"prefix": "a.moe.", "hidden": h, "intermediate": self.inter, "experts": TOY_EXPERTS}), norms("a.")),
+                      LayerSpec("b.", PartSpec("prenorm"), att("b.", PartSpec("rotary", {"theta": 10000.0, "head_dim": self.head_dim})),
+                                PartSpec("swiglu", {"prefix": "b.ff.", "hidden": h, "intermediate": self.inter}), norms("b.")))
+            return ModelSpec(h, self.vocab, 256, PartSpec("token_embedding", {"name": "emb.weight", "vocab": self.vocab, "width": h}),
+                             layers, (RunEntry(0), RunEntry(1)), PartSpec("rmsnorm", {"name": "nf.weight", "width": h, "eps": 1e-5}),
+                             PartSpec("lm_head", {"name": "head.weight", "tied_to": None, "vocab": self.vocab, "width": h}))
+
+    register_part("feed_forward", "toy_routed", RoutedExperts)
+    register_part("position", "toy_added_wave", AddedWave)
+    register_architecture("ToyRoutedForCausalLM", ToyRoutedConfig)
+
+
+def toy_routed_plain(w, ids, heads, d):
+    """The same model as loops over the plain parts; returns the logits and the experts chosen."""
+    f64 = np.float64
+    hid = pm.embed(w["emb.weight"], ids)
+    T = len(ids)
+    pos = np.arange(T)
+    # layer a: attention whose queries and keys get the added wave, then the routed experts
+    n = pm.rmsnorm(hid, w["a.n0.weight"], 1e-5)
+    ang = pos[:, None].astype(f64) * np.array([50.0 ** (-c / d) for c in range(d)])[None, :]
+    q = pm.linear(n, w["a.att.q_proj.weight"], w["a.att.q_proj.bias"]).reshape(T, heads, d) + (0.5 * np.sin(ang))[:, None, :].astype(np.float32)
+    k = pm.linear(n, w["a.att.k_proj.weight"], w["a.att.k_proj.bias"]).reshape(T, 1, d) + (0.5 * np.cos(ang))[:, None, :].astype(np.float32)
+    v = pm.linear(n, w["a.att.v_proj.weight"], w["a.att.v_proj.bias"])
+    hid = pm.add(hid, pm.linear(pm.attention(q.reshape(T, heads * d), k.reshape(T, d), v, heads, 1, d), w["a.att.o_proj.weight"]))
+    n = pm.rmsnorm(hid, w["a.n1.weight"], 1e-5).astype(f64)
+    logits = n @ w["a.moe.router.weight"].astype(f64).T
+    choice = logits.argmax(axis=1)
+    top2 = np.sort(logits, axis=1)[:, -2:]
+    assert (top2[:, 1] - top2[:, 0]).min() > 1.0, "the test's routing must not hang on rounding"
+    y = np.zeros((T, hid.shape[1]), f64)
+    for e in range(TOY_EXPERTS):
+        rows = choice == e
+        y[rows] = np.maximum(n[rows] @ w[f"a.moe.experts.{e}.in.weight"].astype(f64).T, 0) @ w[f"a.moe.experts.{e}.out.weight"].astype(f64).T
+    hid = pm.add(hid, y.astype(np.float32))
+    # layer b: rotary attention and a dense feed-forward
+    cos, sin = pm.rope_table(T, d, 10000.0)
+    n = pm.rmsnorm(hid, w["b.n0.weight"], 1e-5)
+    q = pm.rope_apply(pm.linear(n, w["b.att.q_proj.weight"], w["b.att.q_proj.bias"]), cos, sin, pos, d)
+    k = pm.rope_apply(pm.linear(n, w["b.att.k_proj.weight"], w["b.att.k_proj.bias"]), cos, sin, pos, d)
+    v = pm.linear(n, w["b.att.v_proj.weight"], w["b.att.v_proj.bias"])
+    hid = pm.add(hid, pm.linear(pm.attention(q, k, v, heads, 1, d), w["b.att.o_proj.weight"]))
+    n = pm.rmsnorm(hid, w["b.n1.weight"], 1e-5)
+    hid = pm.add(hid, pm.linear(pm.swiglu(pm.linear(n, w["b.ff.gate_proj.weight"]), pm.linear(n, w["b.ff.up_proj.weight"])), w["b.ff.down_proj.weight"]))
+    return pm.linear(pm.rmsnorm(hid, w["nf.weight"], 1e-5), w["head.weight"]), choice
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, dtype):
+    """A feed-forward with routing and a position encoding that is no rotation, both defined here,
+    in one model beside the engine's own rotary attention and dense feed-forward. The embedding
+    carries a tag per token (one of three channels set high, by token id) and the router reads
+    those channels, so that the choice of expert is far from a tie and every expert is used."""
+    from safetensors.torch import load_file as load_t, save_file as save_t
+    from helpers import collect, mixed, portions, whole
+    from alofa_amd.replay import Replayer
+    from alofa_amd.weights import write_random_model
+    register_toy_routed()
+    raw = {"architectures": ["ToyRoutedForCausalLM"], "hidden": 40, "vocab": 83, "heads": 2, "head_dim": 16, "inter": 24}
+    write_random_model(raw, tmp_path, seed=11, std=0.06)
+    st = load_t(tmp_path / "model.safetensors")
+    e = st["emb.weight"].float()
+    e[:, :TOY_EXPERTS] = 0
+    e[torch.arange(83), torch.arange(83) % TOY_EXPERTS] = 6.0
+    st["emb.weight"] = e.to(st["emb.weight"].dtype)
+    r_w = torch.zeros_like(st["a.moe.router.weight"].float())
+    r_w[torch.arange(TOY_EXPERTS), torch.arange(TOY_EXPERTS)] = 1.0
+    st["a.moe.router.weight"] = r_w.to(st["a.moe.router.weight"].dtype)
+    save_t(st, tmp_path / "model.safetensors")
+    w = pm.read_weights(tmp_path)
+    r = Replayer(tmp_path, dtype, 512)
+    requests = {f"q{i}": random_ids(60 + i, n, 83) for i, n in enumerate([90, 45, 70, 64, 50])}
+    refs, used = {}, set()
+    for k, ids in requests.items():
+        refs[k], choice = toy_routed_plain(w, ids, 2, 16)
+        used |= set(choice.tolist())
+    assert used == set(range(TOY_EXPERTS))
+    assert_close(collect(r, whole("w", requests["q0"]))["w"], refs["q0"], dtype, "toy routed whole")
+    assert_close(collect(r, portions("p", requests["q0"]))["p"], refs["q0"], dtype, "toy routed portions")
+    steps, peak = mixed(requests, seed=3)
+    got = collect(r, steps)
+    for k in requests:
+        assert_close(got[k], refs[k], dtype, f"toy routed mixed {k}")
     r.cache.check()
