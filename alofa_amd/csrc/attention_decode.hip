@@ -93,6 +93,11 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int c16 = lane % 16, g = lane / 16;
   const int n_parts = gridDim.z, n_splits = n_parts * NW, split = blockIdx.z * NW + wave;
+  // The chain of dependent loads is what a short context's attention takes its time from: position and request ->
+  // pages -> keys. With one token per request the request is the token's own number (req_of_token may be null
+  // then), and the first 64 pages of its table set out at once, before the position says which pages are needed.
+  const int32_t* table = block_table + static_cast<int64_t>(req_of_token ? req_of_token[t] : t) * max_blocks;
+  int my_page = table[lane < max_blocks ? lane : max_blocks - 1];
   const int p = positions[t];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   // the visible keys lo..p lie in the 16-key tiles first..last; a wave takes a contiguous run of tiles
@@ -100,7 +105,6 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   const int per_split = (last - first + 1 + n_splits - 1) / n_splits;
   const int tile_begin = first + split * per_split;
   const int tile_end = (tile_begin + per_split < last + 1) ? tile_begin + per_split : last + 1;
-  const int32_t* table = block_table + static_cast<int64_t>(req_of_token[t]) * max_blocks;
   const int bs_mask = (1 << bs_shift) - 1;
 
   // this lane's head and its fragments of Q (heads beyond the group: zeros)
@@ -166,8 +170,10 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   int page_base = (tile_begin << 4) >> bs_shift;
   const int last_page = p >> bs_shift;
   // (pages that a window has passed read -1: they are never used, and 0 keeps every address inside the cache)
-  int my_page = (tile_begin < tile_end && page_base + lane <= last_page) ? table[page_base + lane] : 0;
-  my_page = my_page < 0 ? 0 : my_page;
+  if (page_base != 0) {     // uniform over the wave: a share that starts past the pages already on their way
+    my_page = (tile_begin < tile_end && page_base + lane <= last_page) ? table[page_base + lane] : 0;
+  }
+  my_page = (my_page < 0 || page_base + lane > last_page) ? 0 : my_page;
 
   // Operands of the step that starts at tile `tile` (two tiles): keys [tile][ds], values [tile][nt]. Every
   // lane issues every load, from the nearest visible key where its own is not visible (such scores are
@@ -386,7 +392,8 @@ extern "C" int64_t alofa_attention_decode_scratch(int tokens, int heads, int d, 
 }
 
 // cos_t, sin_t, slots: null for queries that are rotated and a cache that is written already; else (see RopeArgs)
-// q holds rows [queries | keys | values] of one new token per request.
+// q holds rows [queries | keys | values] of one new token per request. req_of_token may be null when every
+// request brings one token: token i then belongs to row i of block_table.
 extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
                                       void* k_cache, void* v_cache, const int32_t* block_table,
                                       int max_blocks, const int32_t* req_of_token, const int32_t* positions,

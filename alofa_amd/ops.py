@@ -383,15 +383,23 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
                      rope: Optional[tuple] = None) -> None:
     """bfloat16 attention for tokens of requests that bring few tokens: every
     token of the batch, or the tokens ``rows`` (int32 indices into the batch).
+    ``req_of_token`` None: every request brings one token and token i is request
+    i (the kernel then starts on the block table without waiting for an index).
     With ``rope`` = (cos, sin, slots) the rows of ``q`` are the fused projection's
     [queries | keys | values] of ONE new token per request, not yet rotated: the
     kernel rotates queries and the new key itself, uses the new key and value from
     registers and writes them to the token's cache slot (``can_fuse_rope_into_decode``)."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     for n, t in (("req_of_token", req_of_token), ("positions", positions)):
+        if t is None and n == "req_of_token":
+            continue
         _gpu(n, t, torch.int32, 1), _contig(n, t)
         if t.shape[0] != T:
             raise AlofaError("shape_mismatch", "one request index and one position per token")
+    if req_of_token is None and (rows is not None or block_table.shape[0] < T):
+        # no request indices: token i is the one token of request i
+        raise AlofaError("invalid_argument", "without request indices every request brings one token, in table order",
+                         f"tokens={T} table_rows={block_table.shape[0]} rows={'given' if rows is not None else 'none'}")
     n_tok = T
     if rows is not None:
         _gpu("rows", rows, torch.int32, 1), _contig("rows", rows)

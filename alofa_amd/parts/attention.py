@@ -102,7 +102,9 @@ class GQAAttention(Mixer):
             if ctx.n_short:                     # single tokens and very short portions, all query heads of a key head together
                 floats = ops.decode_scratch_floats(ctx.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
                 partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
-                ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common,
+                # (one token per request and nothing else in the step: token i is request i)
+                one_each = ctx.max_q_len == 1 and ctx.short_rows is None and ctx.long_runs is None
+                ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, None if one_each else ctx.req_of_token, ctx.positions, *common,
                                      ctx.max_context, partial, rows=ctx.short_rows, rope=(cos, sin, kv.slots) if fused else None)
         if self.b_o is not None:
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)

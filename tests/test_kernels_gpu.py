@@ -323,6 +323,13 @@ def test_decode_attention_that_rotates_and_writes_the_new_token(heads, kv_heads,
     for r, slot in enumerate(slots):
         close(kc_h[slot // bs, :, slot % bs].reshape(-1), refs[r][1], BF16, "new key in its slot")
         assert np.array_equal(vc_h[slot // bs, :, :, slot % bs].reshape(-1), refs[r][2]), "new value in its slot"
+    # one token per request, in table order: the request indices may be left out, and nothing changes
+    again = torch.empty_like(out)
+    o.attention_decode(again, t(qkv, torch.bfloat16), kc, vc, c["table"], None, c["pos"], heads, kv_heads, d, window, scale, bucket, scratch,
+                       rope=(t(cos[:, :d // 2]), t(sin[:, :d // 2]), t(np.array(slots, np.int64), torch.int64)))
+    assert torch.equal(again, out)
+    with pytest.raises(AlofaError):
+        o.attention_decode(again, t(qkv, torch.bfloat16), kc, vc, c["table"][:n - 1], None, c["pos"], heads, kv_heads, d, window, scale, bucket, scratch)
 
 
 @pytest.mark.parametrize("heads,kv_heads,d", [(5, 1, 80), (2, 2, 96), (3, 1, 64)])
