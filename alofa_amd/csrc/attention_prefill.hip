@@ -297,6 +297,11 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
 
 using namespace alofa;
 
+// Teams per block: as many as the registers (128 per lane with four teams, and no spills) and the LDS of a
+// compute unit hold at this head size.
+template <int DT>
+constexpr int kTeams = (DT <= 2 || DT == 4) ? 4 : DT <= 8 ? 2 : 1;
+
 extern "C" int alofa_attention_prefill_supports(int d) {
   return d == 16 || d == 32 || d == 48 || d == 64 || d == 96 || d == 128 || d == 256;
 }
@@ -315,9 +320,8 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
   ALOFA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
                 "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
   dim3 grid(n_tiles, heads);
-  // teams per block: as many as the registers and LDS of a compute unit hold at this head size
 #define ALOFA_PREFILL(DT)                                                                                                 \
-  attention_prefill_kernel<DT, (DT <= 4 ? 4 : DT <= 8 ? 2 : 1)><<<grid, 256 * (DT <= 4 ? 4 : DT <= 8 ? 2 : 1), 0, stream>>>( \
+  attention_prefill_kernel<DT, kTeams<DT>><<<grid, 256 * kTeams<DT>, 0, stream>>>(                                           \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
       static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
   switch (d / 16) {
