@@ -383,8 +383,9 @@ __global__ void __launch_bounds__(64) attention_merge_kernel(bf16_t* __restrict_
 
 using namespace alofa;
 
-// Waves per block: each takes a share of the keys; their states meet in LDS (which bounds their number).
-extern "C" int alofa_attention_decode_waves(int d) { return d <= 128 ? 8 : 4; }
+// Waves per block: each takes a share of the keys; their states meet in LDS (which bounds their number). From head
+// size 128 on four: a block of eight waves leaves 256 registers to a lane, which these head sizes do not fit without spills.
+extern "C" int alofa_attention_decode_waves(int d) { return d < 128 ? 8 : 4; }
 
 // Floats of scratch that n_splits > 1 needs.
 extern "C" int64_t alofa_attention_decode_scratch(int tokens, int heads, int d, int n_splits) {
@@ -425,7 +426,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   if (fused) {
     switch (d / 64) {
       case 1: ALOFA_DECODE(4, 8, true); break;
-      case 2: ALOFA_DECODE(8, 8, true); break;
+      case 2: ALOFA_DECODE(8, 4, true); break;
       case 3: ALOFA_DECODE(12, 4, true); break;
       default: ALOFA_DECODE(16, 4, true); break;
     }
@@ -438,7 +439,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
       case 5: ALOFA_DECODE(5, 8, false); break;
       case 6: ALOFA_DECODE(6, 8, false); break;
       case 7: ALOFA_DECODE(7, 8, false); break;
-      case 8: ALOFA_DECODE(8, 8, false); break;
+      case 8: ALOFA_DECODE(8, 4, false); break;
       case 9: ALOFA_DECODE(9, 4, false); break;
       case 10: ALOFA_DECODE(10, 4, false); break;
       case 11: ALOFA_DECODE(11, 4, false); break;

@@ -304,7 +304,7 @@ MIN_FAST_PAGE = 8         # the bfloat16 attention kernels load eight keys of a 
 
 def decode_waves(d: int) -> int:
     """Waves of a decode attention block; each takes a share of the keys (the kernel's own rule)."""
-    return 8 if d <= 128 else 4
+    return 8 if d < 128 else 4
 
 
 def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
