@@ -117,6 +117,59 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, co
   }
 }
 
+// The same for bfloat16 and head sizes in steps of 16, eight pairs (or eight value channels) per thread with
+// 16-byte accesses; the arithmetic and the rounding are those of the kernel above, element for element.
+__global__ void __launch_bounds__(256) rope_kv_write_vec_kernel(
+    bf16_t* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int32_t* __restrict__ positions, const int64_t* __restrict__ slots, bf16_t* __restrict__ k_cache,
+    bf16_t* __restrict__ v_cache, int tokens, int heads, int kv_heads, int d, int block_size, int write_cache) {
+#pragma clang fp contract(off)
+  const int half = d / 2;
+  const int rot_units = (heads + kv_heads) * (half / 8), v_units = write_cache ? kv_heads * (d / 8) : 0;
+  const int units = rot_units + v_units;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= static_cast<int64_t>(tokens) * units) return;
+  const int t = static_cast<int>(idx / units), u = static_cast<int>(idx % units);
+  bf16_t* row = qkv + static_cast<int64_t>(t) * row_stride;
+  const int64_t slot = slots ? slots[t] : 0;
+  const int64_t blk = slot / block_size, off = slot % block_size;
+  if (u < rot_units) {
+    const int head = u / (half / 8), j = (u % (half / 8)) * 8;
+    const int pos = positions[t];
+    const float* cs = cos_t + static_cast<int64_t>(pos) * half + j;
+    const float* sn = sin_t + static_cast<int64_t>(pos) * half + j;
+    bf16_t* x = row + static_cast<int64_t>(head) * d + j;
+    const uint4 av = *reinterpret_cast<const uint4*>(x), bv = *reinterpret_cast<const uint4*>(x + half);
+    const float4 c0 = *reinterpret_cast<const float4*>(cs), c1 = *reinterpret_cast<const float4*>(cs + 4);
+    const float4 s0 = *reinterpret_cast<const float4*>(sn), s1 = *reinterpret_cast<const float4*>(sn + 4);
+    const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+    const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w}, sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // two elements per 32-bit word, the lower one first
+      const float a0 = __uint_as_float(aw[e] << 16), a1 = __uint_as_float(aw[e] & 0xffff0000u);
+      const float b0 = __uint_as_float(bw[e] << 16), b1 = __uint_as_float(bw[e] & 0xffff0000u);
+      lo[e] = pack_bf16x2(a0 * c[2 * e] - b0 * sv[2 * e], a1 * c[2 * e + 1] - b1 * sv[2 * e + 1]);
+      hi[e] = pack_bf16x2(b0 * c[2 * e] + a0 * sv[2 * e], b1 * c[2 * e + 1] + a1 * sv[2 * e + 1]);
+    }
+    bf16_t* dst = x;
+    if (head >= heads) {
+      if (!write_cache) return;
+      dst = k_cache + ((blk * kv_heads + (head - heads)) * block_size + off) * d + j;
+    }
+    *reinterpret_cast<uint4*>(dst) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    *reinterpret_cast<uint4*>(dst + half) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+  } else {
+    const int v = u - rot_units, hk = v / (d / 8), ch = (v % (d / 8)) * 8;
+    const uint4 vv = *reinterpret_cast<const uint4*>(row + static_cast<int64_t>(heads + kv_heads + hk) * d + ch);
+    const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+    bf16_t* dst = v_cache + ((blk * kv_heads + hk) * d + ch) * block_size + off;      // values lie transposed: [channel][slot]
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dst[static_cast<int64_t>(e) * block_size] = static_cast<bf16_t>((e % 2) ? (w[e / 2] >> 16) : (w[e / 2] & 0xffffu));
+  }
+}
+
 // ---- SwiGLU (unfused) ------------------------------------------------------
 // out = gate / (1 + exp(-gate)) * up, element-wise.
 template <typename T, typename Acc>
@@ -171,7 +224,15 @@ extern "C" int alofa_rope_kv_write(void* qkv, int dtype, int64_t row_stride, con
     rope_kv_write_kernel<float><<<tokens, threads, 0, stream>>>(static_cast<float*>(qkv), row_stride, cos_t, sin_t, positions, slots,
                                                                  static_cast<float*>(k_cache), static_cast<float*>(v_cache), heads,
                                                                  kv_heads, d, block_size, write_cache);
-  else if (dtype == kBF16)
+  else if (dtype == kBF16 && d % 16 == 0 && row_stride % 8 == 0 && reinterpret_cast<uintptr_t>(qkv) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(cos_t) % 16 == 0 && reinterpret_cast<uintptr_t>(sin_t) % 16 == 0 &&
+           (!write_cache || reinterpret_cast<uintptr_t>(k_cache) % 16 == 0)) {
+    const int64_t units = static_cast<int64_t>(heads + kv_heads) * (d / 16) + (write_cache ? static_cast<int64_t>(kv_heads) * (d / 8) : 0);
+    const int64_t blocks = (static_cast<int64_t>(tokens) * units + 255) / 256;
+    rope_kv_write_vec_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+        static_cast<bf16_t*>(qkv), row_stride, cos_t, sin_t, positions, slots, static_cast<bf16_t*>(k_cache),
+        static_cast<bf16_t*>(v_cache), tokens, heads, kv_heads, d, block_size, write_cache);
+  } else if (dtype == kBF16)
     rope_kv_write_kernel<bf16_t><<<tokens, threads, 0, stream>>>(static_cast<bf16_t*>(qkv), row_stride, cos_t, sin_t, positions, slots,
                                                                   static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), heads,
                                                                   kv_heads, d, block_size, write_cache);
