@@ -117,23 +117,22 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int64_t row_stride, co
   }
 }
 
-// The same for bfloat16 and head sizes in steps of 16, eight pairs (or eight value channels) per thread with
-// 16-byte accesses; the arithmetic and the rounding are those of the kernel above, element for element.
+// The same for bfloat16 and head sizes in steps of 16. Rotation: eight pairs per thread with 16-byte accesses;
+// the arithmetic and the rounding are those of the kernel above, element for element. Values: a thread takes one
+// channel of eight consecutive tokens; where these lie in eight consecutive, aligned slots of one page (portions
+// of prompts do) they leave as one 16-byte store into the transposed cache instead of eight scattered ones.
 __global__ void __launch_bounds__(256) rope_kv_write_vec_kernel(
     bf16_t* __restrict__ qkv, int64_t row_stride, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int32_t* __restrict__ positions, const int64_t* __restrict__ slots, bf16_t* __restrict__ k_cache,
     bf16_t* __restrict__ v_cache, int tokens, int heads, int kv_heads, int d, int block_size, int write_cache) {
 #pragma clang fp contract(off)
   const int half = d / 2;
-  const int rot_units = (heads + kv_heads) * (half / 8), v_units = write_cache ? kv_heads * (d / 8) : 0;
-  const int units = rot_units + v_units;
+  const int rot_units = (heads + kv_heads) * (half / 8);
+  const int64_t rot_threads = static_cast<int64_t>(tokens) * rot_units;
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (idx >= static_cast<int64_t>(tokens) * units) return;
-  const int t = static_cast<int>(idx / units), u = static_cast<int>(idx % units);
-  bf16_t* row = qkv + static_cast<int64_t>(t) * row_stride;
-  const int64_t slot = slots ? slots[t] : 0;
-  const int64_t blk = slot / block_size, off = slot % block_size;
-  if (u < rot_units) {
+  if (idx < rot_threads) {
+    const int t = static_cast<int>(idx / rot_units), u = static_cast<int>(idx % rot_units);
+    bf16_t* row = qkv + static_cast<int64_t>(t) * row_stride;
     const int head = u / (half / 8), j = (u % (half / 8)) * 8;
     const int pos = positions[t];
     const float* cs = cos_t + static_cast<int64_t>(pos) * half + j;
@@ -156,17 +155,39 @@ __global__ void __launch_bounds__(256) rope_kv_write_vec_kernel(
     bf16_t* dst = x;
     if (head >= heads) {
       if (!write_cache) return;
-      dst = k_cache + ((blk * kv_heads + (head - heads)) * block_size + off) * d + j;
+      const int64_t slot = slots[t];
+      dst = k_cache + ((slot / block_size * kv_heads + (head - heads)) * block_size + slot % block_size) * d + j;
     }
     *reinterpret_cast<uint4*>(dst) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
     *reinterpret_cast<uint4*>(dst + half) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-  } else {
-    const int v = u - rot_units, hk = v / (d / 8), ch = (v % (d / 8)) * 8;
-    const uint4 vv = *reinterpret_cast<const uint4*>(row + static_cast<int64_t>(heads + kv_heads + hk) * d + ch);
-    const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
-    bf16_t* dst = v_cache + ((blk * kv_heads + hk) * d + ch) * block_size + off;      // values lie transposed: [channel][slot]
+    return;
+  }
+  if (!write_cache) return;
+  // values: thread = (group of eight tokens, key head, channel); consecutive lanes take consecutive channels
+  const int64_t v_idx = idx - rot_threads;
+  const int per_group = kv_heads * d;
+  const int64_t group = v_idx / per_group;
+  if (group * 8 >= tokens) return;
+  const int hk = static_cast<int>(v_idx % per_group) / d, ch = static_cast<int>(v_idx % per_group) % d;
+  const int t0 = static_cast<int>(group) * 8, n = (tokens - t0 < 8) ? tokens - t0 : 8;
+  int64_t slot[8];
+  uint32_t val[8];
+  bool run = n == 8 && block_size % 8 == 0;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) dst[static_cast<int64_t>(e) * block_size] = static_cast<bf16_t>((e % 2) ? (w[e / 2] >> 16) : (w[e / 2] & 0xffffu));
+  for (int e = 0; e < 8; ++e) {
+    const int t = t0 + (e < n ? e : 0);
+    slot[e] = slots[t];
+    val[e] = qkv[static_cast<int64_t>(t) * row_stride + static_cast<int64_t>(heads + kv_heads + hk) * d + ch];
+    run = run && slot[e] == slot[0] + e;
+  }
+  run = run && slot[0] % 8 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+  if (run) {      // eight slots of one page side by side (pages hold a multiple of eight tokens)
+    bf16_t* dst = v_cache + ((slot[0] / block_size * kv_heads + hk) * d + ch) * block_size + slot[0] % block_size;
+    *reinterpret_cast<uint4*>(dst) = make_uint4(val[0] | (val[1] << 16), val[2] | (val[3] << 16), val[4] | (val[5] << 16), val[6] | (val[7] << 16));
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      if (e < n) v_cache[((slot[e] / block_size * kv_heads + hk) * d + ch) * block_size + slot[e] % block_size] = static_cast<bf16_t>(val[e]);
   }
 }
 
@@ -227,8 +248,9 @@ extern "C" int alofa_rope_kv_write(void* qkv, int dtype, int64_t row_stride, con
   else if (dtype == kBF16 && d % 16 == 0 && row_stride % 8 == 0 && reinterpret_cast<uintptr_t>(qkv) % 16 == 0 &&
            reinterpret_cast<uintptr_t>(cos_t) % 16 == 0 && reinterpret_cast<uintptr_t>(sin_t) % 16 == 0 &&
            (!write_cache || reinterpret_cast<uintptr_t>(k_cache) % 16 == 0)) {
-    const int64_t units = static_cast<int64_t>(heads + kv_heads) * (d / 16) + (write_cache ? static_cast<int64_t>(kv_heads) * (d / 8) : 0);
-    const int64_t blocks = (static_cast<int64_t>(tokens) * units + 255) / 256;
+    const int64_t threads_needed = static_cast<int64_t>(tokens) * (heads + kv_heads) * (d / 16) +
+                                   (write_cache ? static_cast<int64_t>((tokens + 7) / 8) * kv_heads * d : 0);
+    const int64_t blocks = (threads_needed + 255) / 256;
     rope_kv_write_vec_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
         static_cast<bf16_t*>(qkv), row_stride, cos_t, sin_t, positions, slots, static_cast<bf16_t*>(k_cache),
         static_cast<bf16_t*>(v_cache), tokens, heads, kv_heads, d, block_size, write_cache);
