@@ -291,9 +291,14 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 }
 
 template <int kEpilogue, typename TO, int WTM, int WTN, int PF, bool kSplitK>
-static void launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
-                        const float* bias, int M, int N, int K, hipStream_t stream) {
+static int launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
+                       const float* bias, int M, int N, int K, hipStream_t stream) {
   const Workspace& g_ws = workspace();
+  if (kSplitK) {   // the partial tiles and the counters of all tiles must lie within the workspace: checked here, whatever chose the shares
+    const int64_t tiles = static_cast<int64_t>(tiles_n) * tiles_m;
+    ALOFA_REQUIRE(g_ws.tiles != nullptr && tiles <= g_ws.n_counters && tiles * shares * (WTM * WTN * 16 * 256) <= g_ws.tile_floats,
+                  "gemm_mfma: %lld tiles in %d shares of K do not fit the workspace", static_cast<long long>(tiles), shares);
+  }
   // operands beyond what the eight L2s hold together (4 MB each)
   const int w_rows = (kEpilogue == kMfSwiglu) ? 2 * N : N;
   const int by_die = (static_cast<int64_t>(M) + w_rows) * K * 2 > (32 << 20);
@@ -301,6 +306,7 @@ static void launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
       static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, tiles_m, tiles_n, shares, kSplitK ? g_ws.tiles : nullptr,
       kSplitK ? g_ws.counters : nullptr, by_die);
+  return 0;
 }
 
 // How many shares of K make `tiles` output tiles (of tile_floats each) fill the chip: doubled while the blocks
@@ -322,9 +328,9 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     // Tiles of 128 rows unless they are fewer than the compute units or half empty. (A tile of 128 x 128
     // outputs, 256 rows of W, leaves room for one block per compute unit only: slower.)
     if (M > 64 && static_cast<int64_t>((N + 63) / 64) * ((M + 127) / 128) >= 256) {
-      launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 63) / 64, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      if (launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 63) / 64, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     } else {
-      launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 63) / 64, (M + 63) / 64, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 63) / 64, (M + 63) / 64, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     }
     return check_launch("gemm_mfma");
   } else {
@@ -335,16 +341,16 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
     if (M <= 64 && (N + 127) / 128 >= 256) {
       // one tile of rows against a long matrix (the vocabulary): tiles of 64 rows, so that no empty rows are staged
-      launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 127) / 128, 1, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 127) / 128, 1, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     } else if (big_blocks >= 512) {
-      launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 127) / 128, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+      if (launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 127) / 128, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     } else {
       const int tiles_n = (N + 63) / 64, tiles_m = (M + 63) / 64;
       const int shares = k_shares(static_cast<int64_t>(tiles_n) * tiles_m, 64 * 64, K);
       if (shares > 1) {
-        launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+        if (launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
       } else {
-        launch_tile<kEpilogue, TO, 1, 1, 2, false>(tiles_n, tiles_m, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+        if (launch_tile<kEpilogue, TO, 1, 1, 2, false>(tiles_n, tiles_m, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
       }
     }
     return check_launch("gemm_mfma");
