@@ -118,6 +118,7 @@ def main():
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=PROMPT, help="prompt length of the timed decode steps' requests (context = prompt + steps so far)")
     ap.add_argument("--layers", type=int, default=QWEN25_05B["num_hidden_layers"], help="fewer layers than the configuration has, where memory or time needs it")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
@@ -138,7 +139,10 @@ def main():
             print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
                                           "frac": round(prefill_flops(cfg, 2048) / pt / PEAK_FLOPS[args.dtype], 4)}}))
             return 0
-        ms, ctx_lens = measure_decode(d, cfg, args.dtype, args.batch, args.steps, args.warmup)
+        if not 1 <= args.prompt <= CONTEXT - args.steps - args.warmup - 1:
+            print(f"--prompt must leave room for the decode steps within the context of {CONTEXT}")
+            return 2
+        ms, ctx_lens = measure_decode(d, cfg, args.dtype, args.batch, args.steps, args.warmup, prompt=args.prompt)
         value = args.batch / ms
         dbytes = 2 if args.dtype == "bfloat16" else 4
         achieved = decode_bytes(cfg, ctx_lens, dbytes) / ms / 1e9
@@ -149,7 +153,7 @@ def main():
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0, 0.02), uniform random token ids)",
             "config": {"model": "Qwen2.5-0.5B sizes, random weights", "layers": args.layers, "layers_full": QWEN25_05B["num_hidden_layers"],
                        "hidden": 896, "heads": 14, "kv_heads": 2, "head_dim": 64, "intermediate": 4864, "vocab": 151936,
-                       "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT, "decode_context": int(sum(ctx_lens) / len(ctx_lens)),
+                       "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": args.prompt, "decode_context": int(sum(ctx_lens) / len(ctx_lens)),
                        "kv_block": BLOCK, "tied_embeddings": True, "parallelism": "single GPU"},
             "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(achieved / PEAK_HBM_GBS, 4)},
