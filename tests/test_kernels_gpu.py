@@ -91,11 +91,13 @@ def test_gemm_exact(M, N, K):
 DEEP_SHAPES = [(40, 130, 1000), (9, 64, 4864), (130, 200, 2056), (64, 896, 672), (3, 33000, 72), (50, 40011, 40)]   # the last two: a long matrix, 64-row tiles
 
 
-@pytest.mark.parametrize("kernel", ["stream", "tiled"])
-@pytest.mark.parametrize("M,N,K", SHAPES + DEEP_SHAPES)
+def with_kernels(shapes):
+    """Every shape with each bfloat16 product that takes it (the streaming kernel: at most 64 rows)."""
+    return [(*shape, kernel) for shape in shapes for kernel in ("stream", "tiled") if kernel == "tiled" or shape[0] <= 64]
+
+
+@pytest.mark.parametrize("M,N,K,kernel", with_kernels(SHAPES + DEEP_SHAPES))
 def test_gemm_bf16(M, N, K, kernel):
-    if kernel == "stream" and M > ops().SKINNY_MAX_ROWS:
-        pytest.skip("the streaming kernel takes at most 64 rows")
     rng = np.random.default_rng(3)
     a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
     b = rng.standard_normal(N).astype(np.float32)
@@ -150,11 +152,8 @@ def test_gemm_takes_a_strided_view():
     close(out, pm.linear(big[:, 100:200], w), EXACT)
 
 
-@pytest.mark.parametrize("kernel", ["stream", "tiled"])
-@pytest.mark.parametrize("M,N,K", [(1, 176, 64), (37, 200, 240), (64, 130, 264), (130, 97, 80), (257, 176, 200), (300, 20000, 72)])
+@pytest.mark.parametrize("M,N,K,kernel", with_kernels([(1, 176, 64), (37, 200, 240), (64, 130, 264), (130, 97, 80), (257, 176, 200), (300, 20000, 72)]))
 def test_gemm_swiglu(M, N, K, kernel):
-    if kernel == "stream" and M > ops().SKINNY_MAX_ROWS:
-        pytest.skip("the streaming kernel takes at most 64 rows")
     rng = np.random.default_rng(5)
     a = rng.standard_normal((M, K)).astype(np.float32)
     wg, wu = rng.standard_normal((N, K)).astype(np.float32), rng.standard_normal((N, K)).astype(np.float32)
