@@ -18,12 +18,14 @@ class Engine:
     """``max_tokens`` is the context window of one request (prompt + generated),
     as the reference's ALOFA_MAX_TOKENS (src/alofa/srv/config.mojo:94-97).
     ``kv_blocks`` pages of ``block_size`` tokens make the pool of each cache group;
-    by default enough for ``max_batch`` requests of ``max_tokens``."""
+    by default enough for ``max_batch`` requests of ``max_tokens``. With
+    ``share_prefixes`` a new request starts on the whole pages a resident request has
+    written for the same first tokens (src/alofa/runtime/kv/space.mojo:166-243, block by block)."""
 
     def __init__(self, model_dir, dtype: str = "bfloat16", max_tokens: int = 256, max_batch: int = 8,
                  kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 2048, max_chunk: int = 512,
                  watermark_permille: int = 900, max_wait_ticks: int = 8, seed: int = 1234, device: str = "cuda:0",
-                 trace_path=None):
+                 trace_path=None, share_prefixes: bool = False):
         from .csrc.build import load
         load()
         self.config, self.model = load_model(Path(model_dir), dtype, device)
@@ -38,7 +40,7 @@ class Engine:
         self.step_fn = StepFunction(self.model, self.cache, n_positions=max_tokens)
         self.sched_cfg = SchedConfig(token_budget, max_chunk, block_size, kv_blocks, watermark_permille, max_wait_ticks,
                                      n_slots=max(32, max_batch))
-        self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path)
+        self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path, share_prefixes=share_prefixes)
         self.seed = seed
         self._next_id = 1
 

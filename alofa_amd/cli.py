@@ -19,6 +19,8 @@ and the engine's own:
   ALOFA_BLOCK_SIZE ALOFA_KV_BLOCKS ALOFA_TOKEN_BUDGET ALOFA_MAX_CHUNK
   ALOFA_WATERMARK_PERMILLE ALOFA_MAX_WAIT_TICKS   cache and scheduler
   ALOFA_TRACE              file that receives the scheduler trace
+  ALOFA_SHARE_PREFIX       1: a new request starts on the pages a running one wrote
+                           for the same first tokens                 (0)
   ALOFA_RANDOM_CONFIG      config.json to make random weights from (with ALOFA_SEED)
                            into ALOFA_WEIGHTS when that folder has no model yet
 
@@ -112,7 +114,8 @@ def main(argv=None) -> int:
                     max_chunk=env_int("ALOFA_MAX_CHUNK", 512, 1, 1 << 20),
                     watermark_permille=env_int("ALOFA_WATERMARK_PERMILLE", 900, 1, 1000),
                     max_wait_ticks=env_int("ALOFA_MAX_WAIT_TICKS", 8, 0, 1 << 20), seed=seed,
-                    trace_path=env_str("ALOFA_TRACE", "") or None)
+                    trace_path=env_str("ALOFA_TRACE", "") or None,
+                    share_prefixes=bool(env_int("ALOFA_SHARE_PREFIX", 0, 0, 1)))
     outs = engine.generate(prompts, max_new=max_new,
                            temperature=env_float("ALOFA_TEMPERATURE", 0.0, 0.0, 1e6),
                            top_k=env_int("ALOFA_TOP_K", 0, 0, 1 << 30), top_p=env_float("ALOFA_TOP_P", 1.0, 1e-9, 1.0),

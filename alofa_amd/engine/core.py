@@ -45,11 +45,16 @@ class Request:
     rng: Optional[SplitMix64] = None
     reported: bool = False
     preemptions: int = 0
+    shared: int = 0                  # prompt tokens taken over from another request's pages
 
 
 class EngineCore:
-    def __init__(self, step_fn: StepFunction, sched_cfg: SchedConfig, trace_path=None):
+    def __init__(self, step_fn: StepFunction, sched_cfg: SchedConfig, trace_path=None, share_prefixes: bool = False):
         self.fn = step_fn
+        # a new request starts on the whole pages of a resident request with the same first tokens
+        # (by reference count) instead of computing them again; off unless asked for
+        self.share_prefixes = bool(share_prefixes)
+        self.shared_tokens = 0
         self.cache = step_fn.cache
         pool_blocks = min((g.pool.n_blocks for g in self.cache.groups), default=sched_cfg.capacity_blocks)
         if sched_cfg.capacity_blocks > pool_blocks:
@@ -62,6 +67,10 @@ class EngineCore:
         self._cancels: list = []
         self._to_report: list = []
         self._freed_blocks = 0
+        # blocks the scheduler charges a request with when it finishes (prompt + max_new), kept from
+        # submission until the scheduler has let go of the id: a finished request may be released
+        # before the tick that reports its completion
+        self._charge: dict = {}
         self.sampler = Sampler()
         self.ticks = 0
         self.last_rows = 0
@@ -72,7 +81,7 @@ class EngineCore:
 
     # ------------------------------------------------------------ requests
     def submit(self, req: int, prompt: list, max_new: int, params: Optional[SampleParams] = None, seed: int = 1234) -> None:
-        if req in self.requests:
+        if req in self.requests or req in self._charge:
             raise AlofaError("invalid_argument", "duplicate request id", f"request={req}")
         if len(prompt) == 0 or max_new <= 0:
             raise AlofaError("invalid_argument", "a request needs a prompt and a positive max_new", f"request={req}")
@@ -83,6 +92,7 @@ class EngineCore:
             raise AlofaError("out_of_range", "token id outside the vocabulary", f"request={req} vocab={vocab}")
         self.requests[req] = Request(req, [int(t) for t in prompt], int(max_new), params or SampleParams(temperature=0.0), int(seed),
                                      rng=SplitMix64(seed))
+        self._charge[req] = blocks_for(len(prompt) + int(max_new), self.sched.cfg.block_size)
         self._arrivals.append(req)
 
     def can_admit(self, prompt_len: int, max_new: int) -> bool:
@@ -109,6 +119,20 @@ class EngineCore:
         return (bool(self._arrivals) or bool(self._cancels) or bool(self._to_report) or self._freed_blocks > 0
                 or any(r.state != DONE for r in self.requests.values()))
 
+    def _scheduler_let_go(self, cancelled: list, finished: list) -> None:
+        """What follows from the scheduler's phases 1 and 2: a cancelled request loses its pages here
+        too (the scheduler subtracted its blocks itself), and the blocks the scheduler moved to its
+        "cached" count for a finished one are owed back on the next tick, since this engine keeps
+        no prefix cache. The request itself may already have been released."""
+        for c in cancelled:
+            self._charge.pop(c, None)
+            r = self.requests.get(c)
+            if r is not None and r.state != DONE:
+                self._drop(r)
+                r.state = DONE
+        for f in finished:
+            self._freed_blocks += self._charge.pop(f, 0)
+
     # ---------------------------------------------------------------- tick
     def _drop(self, r: Request) -> None:
         if self.cache.has(r.id):
@@ -124,39 +148,36 @@ class EngineCore:
         try:
             act = self.sched.step(inp)
         except AlofaError:
-            for a in arrivals:  # a refused admission retires the whole tick's arrivals
-                self.requests[a].state = DONE
+            # a refused admission: the scheduler applied last tick's news (phases 0 to 2 stand) and
+            # took none of this tick's arrivals; they are retired so that nothing asks for them again
+            self._scheduler_let_go(inp.cancelled, inp.finished)
+            for a in arrivals:
+                self._charge.pop(a, None)
+                if a in self.requests:
+                    self.requests[a].state = DONE
             raise
         if self._trace:
             self._trace.write(trace_line(inp, act) + "\n")
             self._trace.flush()
         self.last_action = act
-        for c in inp.cancelled:
-            r = self.requests.get(c)
-            if r is not None and r.state != DONE:
-                self._drop(r)
-                r.state = DONE
+        self._scheduler_let_go(inp.cancelled, act.finished)
         for p in act.preempted:
             r = self.requests[p]
             self._drop(r)
             r.out, r.fed, r.state, r.rng = [], 0, QUEUED, SplitMix64(r.seed)
             r.preemptions += 1
-        bs = self.sched.cfg.block_size
-        for f in act.finished:
-            # the scheduler moved this sequence's blocks to its "cached" count; this
-            # engine keeps no prefix cache, so they are reported back next tick
-            r = self.requests.get(f)
-            if r is not None:
-                self._freed_blocks += blocks_for(len(r.prompt) + r.max_new, bs)
         entries, owes = [], []
         for req, start, end in act.prefill:
             r = self.requests[req]
+            skip = 0
             if start == 0 and not self.cache.has(req):
                 self.cache.admit(req)
+                if self.share_prefixes:
+                    skip = r.shared = self._take_shared_prefix(r, end)
             elif r.fed != start:
                 raise AlofaError("invalid_argument", "prefill slice does not continue the request", f"request={req} fed={r.fed} start={start}")
             last = end == len(r.prompt)
-            entries.append(StepEntry(req, r.prompt[start:end], [end - start - 1] if last else []))
+            entries.append(StepEntry(req, r.prompt[start + skip:end], [end - start - skip - 1] if last else []))
             owes.append(req if last else None)
             r.fed, r.state = end, RESIDENT
         for req in act.decode:
@@ -168,6 +189,30 @@ class EngineCore:
             entries.append(StepEntry(req, [r.out[-1]], [0]))
             owes.append(req)
         return entries, owes
+
+    def _take_shared_prefix(self, r: Request, end: int) -> int:
+        """Let the freshly admitted ``r`` hold the whole pages that a resident request has already
+        written for the same first tokens; returns how many tokens of the slice ``[0, end)`` are
+        history from now on. The slice's last token is always computed
+        (src/alofa/engine/executor.mojo:459-479)."""
+        bs = self.cache.block_size
+        best, donor = 0, None
+        for o in self.requests.values():
+            if o is r or o.state != RESIDENT or not self.cache.has(o.id):
+                continue
+            known = (o.prompt + o.out)[:self.cache.length(o.id)]
+            n = 0
+            for a, b in zip(known, r.prompt[:end - 1]):
+                if a != b:
+                    break
+                n += 1
+            if n // bs > best // bs:
+                best, donor = n, o
+        if donor is None:
+            return 0
+        got = self.cache.share_prefix(donor.id, r.id, best)
+        self.shared_tokens += got
+        return got
 
     def choose(self, logits: torch.Tensor, owes: list) -> list:
         """One token per row of ``logits``, for the requests in ``owes`` (in order)."""

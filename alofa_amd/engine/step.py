@@ -110,6 +110,31 @@ class StepContext:
     def identity_rotation(self, head_dim: int):
         return self.fn.identity_rotation(head_dim)
 
+    def digest(self) -> int:
+        """One number for the layout of this step as the kernels will see it (read back from the
+        device): which request slot brings which rows at which positions, and per cache group the
+        pages behind every request and the slot every row is written to. Equal steps on equal
+        caches give equal digests; it is the scheduler digest's arithmetic
+        (src/alofa/engine/executor.mojo:980-999 for the step's, scheduler.mojo:463-479 for the folding)."""
+        h = 0
+
+        def fold(values):
+            nonlocal h
+            for x in values:
+                h = (h * 1000003 + int(x) + 1) % 2147483647       # + 1: "no page" is -1
+
+        bs = self.fn.cache.block_size
+        for s in self.spans:
+            fold((s.slot, s.row0, s.n, s.pos0))
+        fold(self.positions.cpu().tolist())
+        fold(self.req_of_token.cpu().tolist())
+        for table, slots in zip(self._tables, self._slots):
+            t = table.cpu()
+            for i, s in enumerate(self.spans):
+                fold(t[i, :(s.pos0 + s.n + bs - 1) // bs].tolist())
+            fold(slots.cpu().tolist())
+        return h
+
 
 class StepFunction:
     def __init__(self, model, cache: CacheManager, n_positions: int):

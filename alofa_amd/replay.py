@@ -10,7 +10,21 @@ Steps come on standard input, one JSON object a line:
 
 For a step in which something is wanted, ``DIR/<step>.f32`` receives the logits
 at the wanted places ([wanted, vocab] little-endian float32, in the order of the
-entries and of ``want``). After every step a line ``done <step>`` is printed."""
+entries and of ``want``). After every step a line ``done <step>`` is printed.
+
+A request's first entry may start on pages another live request has filled:
+
+    {"id": "b", "share": {"from": "a", "tokens": 32}, "tokens": [...from position 0...], "want": [40]}
+
+``tokens`` then holds b's tokens from its first one, of which up to 32 must equal
+a's. The whole pages among them that a has written are held by both requests from
+then on (by reference count) and their arithmetic is skipped: they are b's
+history. At least b's last token of the entry is always computed
+(src/alofa/engine/executor.mojo:459-479), b writes its own tokens to fresh pages
+only (src/alofa/runtime/kv/__init__.mojo:24-30), and a may end before b. Places
+in ``want`` count from the entry's first token and must lie beyond what was
+shared. A model whose layers see only a window of keys, or that carries state,
+shares nothing and computes everything."""
 from __future__ import annotations
 
 import argparse
@@ -38,6 +52,8 @@ class Replayer:
         # the position table is as long as a request can get here, not the checkpoint's
         # max_position_embeddings, which the reference does not read (qwen.mojo:849)
         self.fn = StepFunction(self.model, self.cache, n_positions=max(int(max_tokens), 64))
+        self.tokens: dict = {}       # request -> the tokens it has been given so far
+        self.shared: dict = {}       # request -> tokens it took over from another request's pages
 
     def step(self, rec: dict):
         """Run one step record; returns float32 logits [wanted, vocab] as a NumPy
@@ -45,18 +61,48 @@ class Replayer:
         from .engine.step import StepEntry
         entries = []
         for e in rec.get("entries", []):
-            if not self.cache.has(e["id"]):
+            tokens, want = [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]
+            if "share" in e:
+                skipped = self._share(e["id"], e["share"], tokens)
+                if any(w < skipped for w in want):
+                    self.cache.free(e["id"])
+                    del self.tokens[e["id"]]
+                    raise AlofaError("out_of_range", "a wanted place lies in the shared prefix, which is not computed",
+                                     f"request={e['id']} shared={skipped} want={min(want)}")
+                tokens, want = tokens[skipped:], [w - skipped for w in want]
+            elif not self.cache.has(e["id"]):
                 self.cache.admit(e["id"])
-            entries.append(StepEntry(e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])]))
+                self.tokens[e["id"]] = []
+            entries.append(StepEntry(e["id"], tokens, want))
         out = None
         if entries:
             logits = self.fn.run(entries)
+            for e in entries:
+                self.tokens[e.request].extend(e.tokens)
             if logits is not None:
                 out = logits.detach().cpu().numpy().astype("<f4")
         for r in rec.get("end", []):
             if self.cache.has(r):
                 self.cache.free(r)
+                del self.tokens[r]
         return out
+
+    def _share(self, req, share: dict, tokens: list) -> int:
+        """Start ``req`` on the pages of ``share["from"]``; returns how many of ``tokens`` are
+        its history from now on."""
+        src, n = share["from"], int(share["tokens"])
+        if self.cache.has(req):
+            raise AlofaError("invalid_argument", "only a request's first entry can share a prefix", f"request={req}")
+        if not self.cache.has(src):
+            raise AlofaError("invalid_argument", "the request to share with is not live", f"request={req} from={src}")
+        if n < 0 or n > len(tokens) or tokens[:n] != self.tokens[src][:n]:
+            raise AlofaError("invalid_argument", "the tokens to share are not the other request's first tokens", f"request={req} from={src} tokens={n}")
+        self.cache.admit(req)
+        # the entry's last token is always computed: its logits are what the request speaks from
+        skipped = self.cache.share_prefix(src, req, min(n, len(tokens) - 1))
+        self.tokens[req] = tokens[:skipped]
+        self.shared[req] = skipped
+        return skipped
 
 
 def main(argv=None) -> int:

@@ -199,11 +199,28 @@ def test_model_stored_in_float32(tmp_path, dtype):
     assert_close(collect(r, portions("b", ids))["b"], ref, dtype, "float32 storage, portions")
 
 
-@pytest.mark.parametrize("block_size", [16, 32, 64])
-def test_page_size_does_not_matter(replayers, tiny_dirs, block_size):
-    ids = ids_of("B")
-    ref = plain_logits(tiny_dirs["B"], tuple(ids))
-    assert_close(collect(replayers("B", "float32", 512, block_size), portions("p", ids))["p"], ref, "float32", f"page {block_size}")
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("block_size", [8, 24, 32, 64])
+def test_page_size_does_not_matter(tiny_dirs, dtype, block_size):
+    """Every cutting with other pages than 16 tokens: powers of two that the bfloat16 attention kernels
+    take, and 24, for which the bfloat16 engine falls back to the always-valid attention kernel."""
+    from alofa_amd.replay import Replayer
+    for name in ("B", "C"):
+        ids = ids_of(name)
+        ref = plain_logits(tiny_dirs[name], tuple(ids))
+        r = Replayer(tiny_dirs[name], dtype, 512, block_size)
+        assert r.cache.block_size == block_size
+        assert_close(collect(r, whole("w", ids))["w"], ref, dtype, f"{name} page {block_size} whole")
+        assert_close(collect(r, bulk_and_tail("t", ids))["t"], ref, dtype, f"{name} page {block_size} bulk+tail")
+        assert_close(collect(r, portions("p", ids))["p"], ref, dtype, f"{name} page {block_size} portions")
+        vocab = TINY[name]["vocab_size"]
+        requests = {f"r{i}": random_ids(200 + i, n, vocab) for i, n in enumerate([LENGTHS[name], 41, 77, 64, 35])}
+        steps, peak = mixed(requests, seed=block_size)
+        r = Replayer(tiny_dirs[name], dtype, peak, block_size)
+        got = collect(r, steps)
+        r.cache.check()
+        for k, v in requests.items():
+            assert_close(got[k], plain_logits(tiny_dirs[name], tuple(v)), dtype, f"{name} page {block_size} mixed {k}")
 
 
 def test_causality_and_other_tables(replayers, tiny_dirs):
@@ -220,6 +237,117 @@ def test_causality_and_other_tables(replayers, tiny_dirs):
     both = collect(r, [{"step": 0, "entries": [{"id": "x", "tokens": ids[:30], "want": [29]},
                                                 {"id": "y", "tokens": changed[:50], "want": [49]}], "end": ["x", "y"]}])
     assert np.array_equal(both["x"][0], a[29]) and np.array_equal(both["y"][0], b[49])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_another_requests_block_table_changes_the_logits(tiny_dirs, dtype):
+    """The control of tests/unit/test_batch_executor.mojo:585-601 there: a request that is handed
+    another request's block table reads that request's keys, and its logits change. Also the
+    step's digest: the same steps lay out the same way, swapped tables do not."""
+    import torch
+    from alofa_amd.engine.step import StepEntry
+    from alofa_amd.replay import Replayer
+    x, y = ids_of("A", seed=51, n=40), ids_of("A", seed=52, n=40)
+
+    def decode(swap):
+        r = Replayer(tiny_dirs["A"], dtype, 512)      # a fresh pool: the same pages in the same order
+        r.step({"step": 0, "entries": [{"id": "x", "tokens": x[:39], "want": []}, {"id": "y", "tokens": y[:39], "want": []}], "end": []})
+        ctx, ids, rows = r.fn.begin([StepEntry("x", x[39:], [0]), StepEntry("y", y[39:], [0])])
+        if swap:
+            ctx._tables = [t[torch.tensor([1, 0], device=t.device)].contiguous() for t in ctx._tables]
+        digest = ctx.digest()
+        logits = r.model.logits(ctx, r.model.forward(ctx, ids), rows).cpu().numpy().copy()
+        r.fn.finish(ctx)
+        r.step({"step": 1, "entries": [], "end": ["x", "y"]})
+        return logits, digest
+    straight, d0 = decode(False)
+    again, d1 = decode(False)
+    swapped, d2 = decode(True)
+    assert np.array_equal(straight, again) and d0 == d1 and d2 != d0
+    assert np.abs(swapped - straight).max() > 1e-3, "the logits do not depend on whose pages are read"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("n_shared", [16, 32, 48])
+def test_request_starts_on_another_requests_pages(replayers, tiny_dirs, name, dtype, n_shared):
+    """Request b begins with the first tokens of the live request a and takes a's whole pages for
+    them instead of computing them (src/alofa/runtime/kv/space.mojo:166-243, block by block): b
+    goes on in portions and token by token, a ends first, and b's logits equal the plain model's
+    at every computed position. What b writes lands in pages of its own
+    (src/alofa/runtime/kv/__init__.mojo:24-30)."""
+    vocab = TINY[name]["vocab_size"]
+    a_ids = ids_of(name, seed=31, n=70)
+    b_ids = a_ids[:n_shared + 5] + random_ids(32, 60, vocab)          # five more equal tokens: only whole pages are shared
+    b_ids[n_shared + 5] = (a_ids[n_shared + 5] + 1) % vocab
+    ref_a, ref_b = plain_logits(tiny_dirs[name], tuple(a_ids)), plain_logits(tiny_dirs[name], tuple(b_ids))
+    r = replayers(name, dtype)
+    pool = r.cache.groups[0].pool
+    got_a = [r.step({"step": 0, "entries": [{"id": "a", "tokens": a_ids[:60], "want": list(range(60))}], "end": []})]
+    free_before = pool.n_free
+    first = n_shared + 9
+    out = r.step({"step": 1, "entries": [{"id": "a", "tokens": a_ids[60:63], "want": [0, 1, 2]},
+                                          {"id": "b", "share": {"from": "a", "tokens": n_shared + 5}, "tokens": b_ids[:first],
+                                           "want": list(range(n_shared, first))}], "end": []})
+    assert r.shared["b"] == n_shared and r.cache.length("b") == first
+    ta, tb = r.cache.table("a", 0), r.cache.table("b", 0)
+    k = n_shared // 16
+    assert tb[:k] == ta[:k] and all(pool.refcnt_of(p) == 2 for p in tb[:k])
+    assert not set(tb[k:]) & set(ta) and all(pool.refcnt_of(p) == 1 for p in tb[k:])     # its own writes go to fresh pages
+    assert free_before - pool.n_free == len(tb) - k
+    got_a.append(out[:3])
+    got_b = [out[3:]]
+    r.cache.check()
+    # a goes on and ends; b continues in portions of changing size, then token by token
+    got_a.append(r.step({"step": 2, "entries": [{"id": "a", "tokens": a_ids[63:], "want": list(range(7))}], "end": ["a"]}))
+    assert all(pool.refcnt_of(p) == 1 for p in tb[:k]), "the pages stay with b when a ends"
+    pos, step = first, 3
+    for n in (7, 2, 11, 3):
+        got_b.append(r.step({"step": step, "entries": [{"id": "b", "tokens": b_ids[pos:pos + n], "want": list(range(n))}], "end": []}))
+        pos, step = pos + n, step + 1
+    # another request takes the pages a gave back while b still reads the shared ones
+    other = random_ids(33, 40, vocab)
+    got_o = r.step({"step": step, "entries": [{"id": "o", "tokens": other, "want": [39]}], "end": ["o"]})
+    while pos < len(b_ids):
+        got_b.append(r.step({"step": step + pos, "entries": [{"id": "b", "tokens": [b_ids[pos]], "want": [0]}],
+                             "end": ["b"] if pos == len(b_ids) - 1 else []}))
+        pos += 1
+    r.cache.check()
+    assert pool.n_free == pool.n_blocks
+    assert_close(np.concatenate(got_a), ref_a, dtype, f"{name} donor")
+    assert_close(np.concatenate(got_b), ref_b[n_shared:], dtype, f"{name} sharer, {n_shared} tokens shared")
+    assert_close(got_o, plain_logits(tiny_dirs[name], tuple(other))[-1:], dtype, f"{name} bystander")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sharing_rules(replayers, tiny_dirs, dtype):
+    """A prompt that is shared whole still computes its last token; a model with a window shares
+    nothing and computes everything; misuse is refused by name."""
+    from alofa_amd.errors import AlofaError
+    ids = ids_of("A", seed=41, n=48)
+    ref = plain_logits(tiny_dirs["A"], tuple(ids))
+    r = replayers("A", dtype)
+    r.step({"step": 0, "entries": [{"id": "a", "tokens": ids, "want": []}], "end": []})
+    out = r.step({"step": 1, "entries": [{"id": "b", "share": {"from": "a", "tokens": 32}, "tokens": ids[:32], "want": [31]}], "end": []})
+    assert r.shared["b"] == 16 and r.cache.length("b") == 32          # the page that holds the last token is b's own
+    assert_close(out, ref[31:32], dtype, "whole prompt shared")
+    for bad in ({"id": "b", "share": {"from": "a", "tokens": 16}, "tokens": ids[:20], "want": []},       # not b's first entry
+                {"id": "c", "share": {"from": "zz", "tokens": 16}, "tokens": ids[:20], "want": []},      # no such request
+                {"id": "c", "share": {"from": "a", "tokens": 16}, "tokens": ids[1:21], "want": []},      # other tokens
+                {"id": "c", "share": {"from": "a", "tokens": 16}, "tokens": ids[:20], "want": [3]}):     # a place that is not computed
+        with pytest.raises(AlofaError):
+            r.step({"step": 2, "entries": [bad], "end": []})
+        assert not r.cache.has("c")
+    r.step({"step": 4, "entries": [], "end": ["a", "b"]})
+    r.cache.check()
+    # windows: nothing is shared, everything is computed, the logits are right all the same
+    cids = ids_of("C", seed=42, n=80)
+    cref = plain_logits(tiny_dirs["C"], tuple(cids))
+    rc = replayers("C", dtype)
+    rc.step({"step": 0, "entries": [{"id": "a", "tokens": cids[:64], "want": []}], "end": []})
+    out = rc.step({"step": 1, "entries": [{"id": "b", "share": {"from": "a", "tokens": 48}, "tokens": cids, "want": list(range(48, 80))}], "end": ["a", "b"]})
+    assert rc.shared["b"] == 0
+    assert_close(out, cref[48:], dtype, "window model recomputes")
 
 
 def test_trace_run_program(tiny_dirs, tmp_path):

@@ -98,6 +98,144 @@ def test_pages_run_out_preemption_recomputes(tiny_dirs):
     assert all(g.pool.n_free == g.pool.n_blocks for g in eng.cache.groups)
 
 
+def held_nothing(eng):
+    s = eng.core.sched
+    assert s.blocks_used == 0 and s.cached_blocks == 0 and s.n_live() == 0
+    eng.cache.check()
+    assert not eng.cache.requests and all(g.pool.n_free == g.pool.n_blocks for g in eng.cache.groups)
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_release_as_soon_as_done(tiny_dirs, name):
+    """A caller that drives tick() and releases each request the moment it is done, before the
+    tick that reports its completion: 40 requests through a pool that holds two at a time."""
+    from alofa_amd import Engine
+    vocab = TINY[name]["vocab_size"]
+    eng = Engine(tiny_dirs[name], dtype="float32", max_tokens=64, kv_blocks=8, watermark_permille=1000, max_chunk=16, token_budget=32)
+    core = eng.core
+    prompts = {i: random_ids(300 + i, 5 + i % 23, vocab) for i in range(40)}
+    want = {i: plain_greedy(tiny_dirs[name], prompts[i], 6) for i in range(40)}
+    waiting, live, ticks = list(range(40)), [], 0
+    while waiting or live:
+        while waiting and core.can_admit(len(prompts[waiting[0]]), 6):
+            live.append(waiting.pop(0))
+            core.submit(live[-1], prompts[live[-1]], 6)
+        core.tick()
+        ticks += 1
+        assert ticks < 2000, f"stuck: blocks_used={core.sched.blocks_used} cached={core.sched.cached_blocks}"
+        assert core.sched.blocks_used == core.sched.blocks_held() + core.sched.cached_blocks
+        for r in [r for r in live if core.is_done(r)]:
+            assert core.output(r) == want[r], f"request {r}"
+            core.release(r)
+            live.remove(r)
+    assert eng.cache.groups[0].pool.high_water <= 8
+    core.run(10)
+    held_nothing(eng)
+
+
+def test_cancel_half_prefilled_and_queued(tiny_dirs):
+    from alofa_amd import Engine
+    eng = Engine(tiny_dirs["A"], dtype="float32", max_tokens=96, max_chunk=8, token_budget=8)
+    core = eng.core
+    a, b, c = random_ids(61, 30, 256), random_ids(62, 9, 256), random_ids(63, 7, 256)
+    core.submit(1, a, 5), core.submit(2, b, 5)
+    core.tick()
+    assert core.requests[1].fed == 8 and core.requests[2].fed == 0 and eng.cache.has(1)
+    core.cancel(1)                                    # half prefilled: its pages go back
+    core.tick()
+    assert core.is_done(1) and not eng.cache.has(1) and core.output(1) == []
+    core.submit(3, c, 4)
+    core.cancel(2)                                    # still queued
+    core.submit(4, a, 3), core.cancel(4)              # arrival and cancel of one id in one tick
+    core.tick()
+    assert core.is_done(2) and core.is_done(4) and core.sched.find(4) < 0
+    core.run(100)
+    assert core.output(3) == plain_greedy(tiny_dirs["A"], c, 4) and core.output(2) == [] and core.output(4) == []
+    for r in (1, 2, 3, 4):
+        core.release(r)
+    held_nothing(eng)
+
+
+def test_decode_time_preemption_recomputes(tiny_dirs):
+    """The scheduler's phase 6: a decode needs a page, none is left, the newest running request is
+    dropped and computed again from its first token. (Reached by a pool that shrinks under running
+    requests; with a standing configuration admission keeps every decode within the pool.)"""
+    from alofa_amd import Engine
+    from alofa_amd.engine.scheduler import SchedConfig
+    prompts = [random_ids(70 + i, 13, 256) for i in range(3)]
+    want = [plain_greedy(tiny_dirs["A"], p, 25) for p in prompts]
+    eng = Engine(tiny_dirs["A"], dtype="float32", max_tokens=64, kv_blocks=9, watermark_permille=1000, max_chunk=32, token_budget=64)
+    core = eng.core
+    for i, p in enumerate(prompts):
+        core.submit(i + 1, p, 25)                     # 3 x 3 blocks
+    core.tick(), core.tick()
+    assert core.sched.blocks_used == 3 and all(len(r.out) == 2 for r in core.requests.values())
+    core.sched.cfg = SchedConfig(64, 32, 16, 5, 1000, 8, 32)     # five blocks: the second page of all three does not fit
+    seen = []
+    for _ in range(400):
+        if not core.has_work():
+            break
+        core.tick()
+        seen += list(core.last_action.preempted)
+        assert core.sched.blocks_used <= 5
+    # request 3 (the last slot) is the one that finds no page: the newest running request other than itself goes
+    assert seen and seen[0] == 2 and core.requests[2].preemptions >= 1 and core.requests[1].preemptions == 0
+    assert [core.output(i + 1) for i in range(3)] == want
+    for i in range(3):
+        core.release(i + 1)
+    held_nothing(eng)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_forty_requests_in_one_batch(tiny_dirs, dtype):
+    from alofa_amd import Engine
+    prompts = [random_ids(400 + i, 3 + i % 17, 256) for i in range(40)]
+    eng = Engine(tiny_dirs["A"], dtype=dtype, max_tokens=64, max_batch=40)
+    core = eng.core
+    for i, p in enumerate(prompts):
+        core.submit(i + 1, p, 8)
+    widest = 0
+    while core.has_work():
+        core.tick()
+        widest = max(widest, len(core.last_action.decode))
+    assert widest == 40
+    outs = [core.output(i + 1) for i in range(40)]
+    for i in range(40):
+        core.release(i + 1)
+    want = [plain_greedy(tiny_dirs["A"], p, 8) for p in prompts]
+    if dtype == "float32":
+        assert outs == want
+    else:
+        assert agreement(outs, want) >= 0.9
+    assert eng.step_fn.graph_replays > 0 or dtype == "float32"
+    held_nothing(eng)
+
+
+def test_engine_shares_prefixes_when_asked(tiny_dirs):
+    """share_prefixes: requests with a common beginning hold its whole pages together and the
+    later ones skip its arithmetic; tokens are the same as without."""
+    from alofa_amd import Engine
+    common = random_ids(81, 40, 256)
+    prompts = [common + random_ids(82 + i, 5 + i, 256) for i in range(4)] + [common[:32]]
+    want = [plain_greedy(tiny_dirs["A"], p, 10) for p in prompts]
+    eng = Engine(tiny_dirs["A"], dtype="float32", max_tokens=96, share_prefixes=True)
+    core = eng.core
+    core.submit(1, prompts[0], 10)
+    core.tick()
+    rows = eng.step_fn.rows_run
+    for i in range(1, 5):
+        core.submit(i + 1, prompts[i], 10)
+    core.tick()
+    assert [core.requests[i + 1].shared for i in range(5)] == [0, 32, 32, 32, 16]
+    assert eng.step_fn.rows_run - rows == 1 + sum(len(p) - 32 for p in prompts[1:4]) + 16
+    eng.cache.check()
+    core.run(100)
+    assert [core.output(i + 1) for i in range(5)] == want
+    for i in range(5):
+        core.release(i + 1)
+    held_nothing(eng)
+
+
 def test_tight_pool_serves_requests_one_after_another(tiny_dirs):
     from alofa_amd import Engine
     from alofa_amd.errors import AlofaError
