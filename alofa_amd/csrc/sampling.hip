@@ -5,8 +5,11 @@
 // then across threads in thread order, and the first index whose running sum
 // exceeds u * total is taken (the last index if none does).
 #include "common.h"
+#include "no_alloc.h"
 
 #include <float.h>
+
+#include <mutex>
 
 namespace alofa {
 
@@ -145,6 +148,60 @@ extern "C" int alofa_argmax(int32_t* out, const float* logits, int64_t stride, i
     return check_launch("argmax");
   }
   float* part_v = static_cast<float*>(scratch);
+  int32_t* part_i = reinterpret_cast<int32_t*>(part_v + static_cast<int64_t>(rows) * kArgmaxChunks);
+  argmax_chunk_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(part_v, part_i, logits, stride, vocab);
+  if (check_launch("argmax_chunk")) return 1;
+  argmax_final_kernel<<<rows, kWave, 0, stream>>>(out, part_v, part_i, vocab);
+  return check_launch("argmax_final");
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// The partial maxima of alofa_argmax_no_alloc live in this array instead of a buffer the caller
+// brings. In host code the array's name is only a stand-in: the memory is reached through the
+// address that hipGetSymbolAddress gives, looked up once per device (every GPU holds a copy of its
+// own) with that device current.
+namespace alofa {
+
+constexpr int64_t kNoAllocScratchBytes = static_cast<int64_t>(ALOFA_ARGMAX_NO_ALLOC_MAX_ROWS) * kArgmaxChunks * (sizeof(float) + sizeof(int32_t));
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_of_device[kMaxDevices];   // null until the first call on that device
+static std::mutex g_scratch_mutex;
+
+// the current device's copy of `scratch`, or null with the error set
+static void* scratch_of_current_device() {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= kMaxDevices) {
+    set_error("argmax_no_alloc: no usable current device: %s [device=%d]", hipGetErrorString(e), device);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (g_scratch_of_device[device] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("argmax_no_alloc: the scratch array has no address on device %d: %s", device, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_of_device[device] = ptr;
+  }
+  return g_scratch_of_device[device];
+}
+
+}  // namespace alofa
+
+extern "C" int alofa_argmax_no_alloc(int32_t* out, const float* logits, int64_t stride, int rows, int vocab, hipStream_t stream) {
+  ALOFA_REQUIRE(out != nullptr && logits != nullptr, "argmax_no_alloc: out and logits must be given");
+  ALOFA_REQUIRE(rows > 0 && vocab > 0 && stride >= vocab, "argmax_no_alloc: rows=%d vocab=%d stride=%lld", rows, vocab, static_cast<long long>(stride));
+  ALOFA_REQUIRE(rows <= ALOFA_ARGMAX_NO_ALLOC_MAX_ROWS, "argmax_no_alloc: at most %d rows fit the built-in scratch [rows=%d]",
+                ALOFA_ARGMAX_NO_ALLOC_MAX_ROWS, rows);
+  void* ptr = scratch_of_current_device();
+  if (ptr == nullptr) return 1;
+  // every (row, chunk) cell that the second kernel reads is written by the first, so nothing
+  // of an earlier call's contents has to be cleared
+  float* part_v = static_cast<float*>(ptr);
   int32_t* part_i = reinterpret_cast<int32_t*>(part_v + static_cast<int64_t>(rows) * kArgmaxChunks);
   argmax_chunk_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(part_v, part_i, logits, stride, vocab);
   if (check_launch("argmax_chunk")) return 1;
