@@ -72,6 +72,52 @@ def test_residual_and_activation_vectors(l0):
     assert not close(pm.swiglu(l0["up_out"], l0["gate_out"]), l0["swiglu_out"])
 
 
+def _bf16_matrix(bits):
+    """The reference's matrices are bfloat16 values widened to float32; the fixture keeps their high halves."""
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def test_attention_block_wiring_vectors(l0):
+    """The whole first half of layer 0 of the real model, from the normed input to the second norm's
+    output: q, k and v projections with their biases, rotation of q and k but not of v, attention,
+    the output projection without bias, the residual sum and the post-attention norm, against the
+    tensors the reference captured (tests/fixtures/qwen2.5-0.5b/layer0/tensors.tsv:1-26 there)."""
+    pre = "model.layers.0.self_attn."
+    w = {pre + "q_proj.weight": _bf16_matrix(l0["q_w_bf16"]), pre + "q_proj.bias": l0["q_b"],
+         pre + "k_proj.weight": l0["k_w"], pre + "k_proj.bias": l0["k_b"],
+         pre + "v_proj.weight": _bf16_matrix(l0["v_w_bf16"]), pre + "v_proj.bias": l0["v_b"],
+         pre + "o_proj.weight": _bf16_matrix(l0["o_w_bf16"])}
+    cfg = {"H": 14, "Hkv": 2, "d": 64, "windows": [None]}
+    pos = np.arange(16)
+    o = pm.attention_block(w, cfg, 0, l0["norm_out"], l0["cos"], l0["sin"], pos)
+    assert close(o, l0["o_out"])
+    hidden1 = pm.add(l0["embed_out"], o)
+    assert close(hidden1, l0["hidden1"])
+    assert close(pm.rmsnorm(hidden1, l0["norm2_w"], 1e-6), l0["norm2_out"])
+    # the projections one by one, as the reference's op list has them (layer0/ops.tsv:2-4, :7)
+    assert close(pm.linear(l0["norm_out"], w[pre + "q_proj.weight"], l0["q_b"]), l0["q_out"])
+    assert close(pm.linear(l0["norm_out"], w[pre + "v_proj.weight"], l0["v_b"]), l0["v_out"])
+    assert close(pm.linear(l0["attn_out"], w[pre + "o_proj.weight"]), l0["o_out"])
+
+    # plausible mistakes must fail: a rotated v, a dropped bias, an output bias that is not there, a post-norm wiring
+    def block_with(rotate_v=False, drop_bias=None):
+        ww = dict(w)
+        if drop_bias:
+            ww[pre + drop_bias + "_proj.bias"] = np.zeros_like(w[pre + drop_bias + "_proj.bias"])
+        q = pm.rope_apply(pm.linear(l0["norm_out"], ww[pre + "q_proj.weight"], ww[pre + "q_proj.bias"]), l0["cos"], l0["sin"], pos, 64)
+        k = pm.rope_apply(pm.linear(l0["norm_out"], ww[pre + "k_proj.weight"], ww[pre + "k_proj.bias"]), l0["cos"], l0["sin"], pos, 64)
+        v = pm.linear(l0["norm_out"], ww[pre + "v_proj.weight"], ww[pre + "v_proj.bias"])
+        if rotate_v:
+            v = pm.rope_apply(v, l0["cos"], l0["sin"], pos, 64)
+        return pm.linear(pm.attention(q, k, v, 14, 2, 64), ww[pre + "o_proj.weight"])
+    assert close(block_with(), l0["o_out"])
+    assert not close(block_with(rotate_v=True), l0["o_out"])
+    for name in ("q", "k", "v"):
+        assert not close(block_with(drop_bias=name), l0["o_out"]), name
+    assert not close(pm.attention_block(w, cfg, 0, l0["embed_out"], l0["cos"], l0["sin"], pos), l0["o_out"])   # no input norm
+    assert not close(pm.rmsnorm(pm.add(l0["embed_out"], o), l0["norm_w"], 1e-6), l0["norm2_out"])               # the other norm's weight
+
+
 # ------------------------------------- special cases and invariants
 
 def test_rmsnorm_special_cases():
@@ -172,6 +218,71 @@ def test_whole_model_shift_of_positions(tiny_dirs):
     assert np.array_equal(a[:7], c[:7]) and not np.array_equal(a[7:], c[7:])
 
 
+def _edited(w, **changes):
+    out = dict(w)
+    out.update(changes)
+    return out
+
+
+def test_second_half_of_the_block_and_the_end_of_the_model(tiny_dirs):
+    """What no vector of the reference reaches (its fixture stops at the SwiGLU output and its
+    last-row logits need weights that are not in the repository: parity unpinned there): the down
+    projection with the second residual sum, the final norm before the head, and the head without
+    bias. Each is fixed by an invariant that a plausible other wiring breaks."""
+    cfg = pm.read_config(tiny_dirs["B"])
+    w = pm.read_weights(tiny_dirs["B"])
+    ids = [int(t) for t in np.random.default_rng(6).integers(0, cfg["V"], 9)]
+    T, h, L = len(ids), cfg["h"], cfg["L"]
+    cos, sin = pm.rope_table(T, cfg["d"], cfg["theta"])
+    pos = np.arange(T)
+    hidden = pm.embed(w["model.embed_tokens.weight"], ids)
+    down = "model.layers.0.mlp.down_proj.weight"
+    post = "model.layers.0.post_attention_layernorm.weight"
+
+    # down_proj = 0: the block returns what the attention half left (hidden + attention), bit for bit
+    n1 = pm.rmsnorm(hidden, w["model.layers.0.input_layernorm.weight"], cfg["eps"])
+    hidden1 = pm.add(hidden, pm.attention_block(w, cfg, 0, n1, cos, sin, pos))
+    zeroed = pm.decoder_block(_edited(w, **{down: np.zeros_like(w[down])}), cfg, 0, hidden, cos, sin, pos)
+    assert np.array_equal(zeroed, hidden1)
+    # the feed-forward reads the normed stream, scaled by the post-attention norm's weight and by
+    # nothing else: its contribution is decoder_block - hidden1, and doubling down_proj doubles
+    # exactly that (a post-norm wiring, or a norm applied to the sum, would not)
+    full = pm.decoder_block(w, cfg, 0, hidden, cos, sin, pos)
+    twice = pm.decoder_block(_edited(w, **{down: 2.0 * w[down]}), cfg, 0, hidden, cos, sin, pos)
+    ff = pm.feed_forward(w, cfg, 0, pm.rmsnorm(hidden1, w[post], cfg["eps"]))
+    assert np.abs(full - pm.add(hidden1, ff)).max() == 0
+    assert np.abs((twice.astype(np.float64) - hidden1) - 2.0 * (full.astype(np.float64) - hidden1)).max() < 1e-6
+    # a zero post-attention norm weight silences the feed-forward whatever its matrices are
+    silent = pm.decoder_block(_edited(w, **{post: np.zeros_like(w[post])}), cfg, 0, hidden, cos, sin, pos)
+    assert np.array_equal(silent, hidden1)
+    # ... but the feed-forward does not read the unnormed stream: scaling the stream's input changes its share
+    assert not np.allclose(pm.feed_forward(w, cfg, 0, hidden1), ff, atol=1e-4)
+
+    # the end of the model. model.norm.weight = 0: every logit is exactly zero (the final norm
+    # stands before the head, and the head has no bias)
+    logits = pm.forward_logits(w, cfg, ids)
+    nothing = pm.forward_logits(_edited(w, **{"model.norm.weight": np.zeros_like(w["model.norm.weight"])}), cfg, ids)
+    assert nothing.shape == logits.shape and not nothing.any()
+    # head = identity (vocabulary cut to the width): the logits are the final norm of the last
+    # block's output, with the norm's weight applied once
+    final = hidden
+    for i in range(L):
+        final = pm.decoder_block(w, cfg, i, final, cos, sin, pos)
+    eye = np.eye(h, dtype=np.float32)
+    through = pm.forward_logits(_edited(w, **{"lm_head.weight": eye}), dict(cfg, V=h), ids)
+    assert np.array_equal(through, pm.rmsnorm(final, w["model.norm.weight"], cfg["eps"]))
+    assert not np.allclose(through, final, atol=1e-3)                   # a head on the unnormed stream
+    x = final.astype(np.float64)
+    want = x / np.sqrt((x * x).mean(axis=1, keepdims=True) + cfg["eps"]) * w["model.norm.weight"].astype(np.float64)
+    assert np.allclose(through, want, rtol=1e-5, atol=1e-6)
+    assert np.array_equal(logits, pm.linear(pm.rmsnorm(final, w["model.norm.weight"], cfg["eps"]), pm.output_matrix(w, cfg)))
+    # tying: config A has no lm_head.weight and multiplies by the embedding
+    cfg_a, w_a = pm.read_config(tiny_dirs["A"]), pm.read_weights(tiny_dirs["A"])
+    assert "lm_head.weight" not in w_a and pm.output_matrix(w_a, cfg_a) is w_a["model.embed_tokens.weight"]
+    with pytest.raises(KeyError):
+        pm.output_matrix(w_a, dict(cfg_a, tied=False))
+
+
 def test_window_config_reaches_the_layers(tiny_dirs):
     cfg = pm.read_config(tiny_dirs["C"])
     assert cfg["windows"] == [None, 40, 40, 40] and cfg["d"] == 48
@@ -223,3 +334,36 @@ def test_sampler_special_cases():
     assert v2 == [1.0, -4.0]
     v3, _ = ps.distribution(np.array([2.0, -2.0], dtype=np.float32), frequency_penalty=0.5, presence_penalty=0.25, history=[1, 1])
     assert v3 == [2.0, -3.25]
+
+
+def test_min_p_and_min_tokens_to_keep_special_cases():
+    """min_p drops what is rarer than min_p times the likeliest entry; the ``min_tokens_to_keep``
+    likeliest entries survive every filter (src/alofa/runtime/sampler.mojo:432-472)."""
+    # two values: probabilities p and 1 - p with a known ratio e^-3 ~ 0.0498
+    logits = np.array([0.0, 3.0, 0.0, 3.0], dtype=np.float32)
+    values, p = ps.distribution(logits, min_p=0.04)            # 0.0498 >= 0.04: everything stays
+    assert all(v > ps.FLOOR for v in values) and abs(sum(p) - 1) < 1e-12
+    values, p = ps.distribution(logits, min_p=0.06)            # 0.0498 < 0.06: the small ones go
+    assert [v > ps.FLOOR for v in values] == [False, True, False, True] and p == [0.0, 0.5, 0.0, 0.5]
+    # the cut compares with min_p * the largest probability, not with min_p itself: 0.4, 0.3, 0.3
+    third = np.log(np.array([0.4, 0.3, 0.3])).astype(np.float32)
+    values, p = ps.distribution(third, min_p=0.7)              # 0.3 >= 0.7 * 0.4 = 0.28
+    assert all(v > ps.FLOOR for v in values)
+    values, p = ps.distribution(third, min_p=0.8)              # 0.3 < 0.32
+    assert [v > ps.FLOOR for v in values] == [True, False, False] and p == [1.0, 0.0, 0.0]
+    # min_tokens_to_keep: the likeliest two survive, ties by the lower index
+    values, p = ps.distribution(third, min_p=0.8, min_tokens_to_keep=2)
+    assert [v > ps.FLOOR for v in values] == [True, True, False] and abs(p[0] - 4 / 7) < 1e-7 and abs(p[1] - 3 / 7) < 1e-7
+    # ... against top_p as well, which alone would stop after the first entry
+    values, p = ps.distribution(third, top_p=0.1)
+    assert [v > ps.FLOOR for v in values] == [True, False, False]
+    values, p = ps.distribution(third, top_p=0.1, min_tokens_to_keep=3)
+    assert all(v > ps.FLOOR for v in values) and np.allclose(p, [0.4, 0.3, 0.3], rtol=1e-6)
+    # top_p takes entries until the running sum reaches it: 0.4 < 0.5 <= 0.7
+    values, p = ps.distribution(third, top_p=0.5)
+    assert [v > ps.FLOOR for v in values] == [True, True, False]
+    # min_p applies to the distribution after temperature
+    cold = ps.distribution(third, temperature=0.5, min_p=0.6)[0]     # 0.16 : 0.09 -> ratio 0.5625 < 0.6
+    assert [v > ps.FLOOR for v in cold] == [True, False, False]
+    warm = ps.distribution(third, temperature=2.0, min_p=0.6)[0]     # ratio 0.866
+    assert all(v > ps.FLOOR for v in warm)
