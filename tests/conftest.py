@@ -14,6 +14,17 @@ if str(ROOT / "tests") not in sys.path:
 FIXTURES = Path(__file__).resolve().parent / "fixtures"
 
 
+def pytest_sessionfinish(session, exitstatus):
+    """With ALOFA_TEST_RATIOS=<file>: how close every bfloat16 comparison came to its bound."""
+    import os
+    path = os.environ.get("ALOFA_TEST_RATIOS")
+    if path:
+        from helpers import RATIOS
+        with open(path, "w") as f:
+            for what, peak, rms in RATIOS:
+                f.write(f"{peak:.3f}\t{rms:.3f}\t{what}\n")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X and the built HIP library")
 

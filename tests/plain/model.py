@@ -172,37 +172,47 @@ def add(a: np.ndarray, b: np.ndarray) -> np.ndarray:
 
 
 # --------------------------------------------------------------- whole model
+# ``store`` (not in the reference, whose activations are all float32): a function applied to every
+# activation that an engine with narrower activations keeps in memory between two operators (the
+# normed stream, q, k and v, rotated q and k, the attention output, the activated feed-forward
+# product); the residual stream and all sums stay as they are. With it the plain model shows how
+# far rounding the activations alone moves the logits, which is what a tolerance for such an
+# engine has to be measured against.
 
-def attention_block(w, cfg, i, x, cos, sin, positions):
+def _keep(x):
+    return x
+
+
+def attention_block(w, cfg, i, x, cos, sin, positions, store=_keep):
     """q, k, v with bias; rotate q and k, not v; attend; output projection
     without bias (src/alofa/model/arch/qwen.mojo:1429-1480)."""
     p = f"model.layers.{i}.self_attn."
-    q = linear(x, w[p + "q_proj.weight"], w[p + "q_proj.bias"])
-    k = linear(x, w[p + "k_proj.weight"], w[p + "k_proj.bias"])
-    v = linear(x, w[p + "v_proj.weight"], w[p + "v_proj.bias"])
-    q = rope_apply(q, cos, sin, positions, cfg["d"])
-    k = rope_apply(k, cos, sin, positions, cfg["d"])
-    a = attention(q, k, v, cfg["H"], cfg["Hkv"], cfg["d"], cfg["windows"][i])
+    q = store(linear(x, w[p + "q_proj.weight"], w[p + "q_proj.bias"]))
+    k = store(linear(x, w[p + "k_proj.weight"], w[p + "k_proj.bias"]))
+    v = store(linear(x, w[p + "v_proj.weight"], w[p + "v_proj.bias"]))
+    q = store(rope_apply(q, cos, sin, positions, cfg["d"]))
+    k = store(rope_apply(k, cos, sin, positions, cfg["d"]))
+    a = store(attention(q, k, v, cfg["H"], cfg["Hkv"], cfg["d"], cfg["windows"][i]))
     return linear(a, w[p + "o_proj.weight"])
 
 
-def feed_forward(w, cfg, i, x):
+def feed_forward(w, cfg, i, x, store=_keep):
     """down(silu(gate(x)) * up(x)), no biases
     (src/alofa/engine/executor.mojo:806-837)."""
     p = f"model.layers.{i}.mlp."
     g = linear(x, w[p + "gate_proj.weight"])
     u = linear(x, w[p + "up_proj.weight"])
-    return linear(swiglu(g, u), w[p + "down_proj.weight"])
+    return linear(store(swiglu(g, u)), w[p + "down_proj.weight"])
 
 
-def decoder_block(w, cfg, i, hidden, cos, sin, positions):
+def decoder_block(w, cfg, i, hidden, cos, sin, positions, store=_keep):
     """Pre-norm block with two residual sums
     (src/alofa/model/arch/qwen.mojo:1418-1510)."""
     p = f"model.layers.{i}."
-    n1 = rmsnorm(hidden, w[p + "input_layernorm.weight"], cfg["eps"])
-    hidden = add(hidden, attention_block(w, cfg, i, n1, cos, sin, positions))
-    n2 = rmsnorm(hidden, w[p + "post_attention_layernorm.weight"], cfg["eps"])
-    return add(hidden, feed_forward(w, cfg, i, n2))
+    n1 = store(rmsnorm(hidden, w[p + "input_layernorm.weight"], cfg["eps"]))
+    hidden = add(hidden, attention_block(w, cfg, i, n1, cos, sin, positions, store))
+    n2 = store(rmsnorm(hidden, w[p + "post_attention_layernorm.weight"], cfg["eps"]))
+    return add(hidden, feed_forward(w, cfg, i, n2, store))
 
 
 def output_matrix(w, cfg):
@@ -215,7 +225,14 @@ def output_matrix(w, cfg):
     raise KeyError("no output matrix: lm_head.weight is absent and the embedding is not tied")
 
 
-def forward_logits(w, cfg, ids, first_position: int = 0) -> np.ndarray:
+def to_bfloat16(x: np.ndarray) -> np.ndarray:
+    """x rounded to the nearest bfloat16 (ties to even), as float32: a ``store`` for the plain model."""
+    bits = np.ascontiguousarray(x, dtype=F32).view(np.uint32).astype(np.uint64)
+    rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) << 16
+    return rounded.astype(np.uint32).view(F32).reshape(np.shape(x))
+
+
+def forward_logits(w, cfg, ids, first_position: int = 0, store=_keep) -> np.ndarray:
     """Logits [len(ids), V] at every position of one sequence whose first token
     stands at ``first_position`` (0 in the reference; another value only shifts
     the rotary angles) (src/alofa/model/arch/qwen.mojo:1362-1525)."""
@@ -224,8 +241,8 @@ def forward_logits(w, cfg, ids, first_position: int = 0) -> np.ndarray:
     cos, sin = rope_table(first_position + T, cfg["d"], cfg["theta"])
     hidden = embed(w["model.embed_tokens.weight"], ids)
     for i in range(cfg["L"]):
-        hidden = decoder_block(w, cfg, i, hidden, cos, sin, positions)
-    y = rmsnorm(hidden, w["model.norm.weight"], cfg["eps"])
+        hidden = decoder_block(w, cfg, i, hidden, cos, sin, positions, store)
+    y = store(rmsnorm(hidden, w["model.norm.weight"], cfg["eps"]))
     return linear(y, output_matrix(w, cfg))
 
 
