@@ -1,12 +1,14 @@
 """The cache manager: keys and values in pages with a block table per request,
 and slots for per-request state of fixed size.
 
-Run entries whose mixers have the same need of history form a *group* with
-pages of its own: one group for mixers that keep every key, one per window
-length for mixers that see only the last ``window`` keys. Within a group one
-block id names a slot of K and V in every entry of the group, so a request has
-one table per group (src/alofa/engine/executor.mojo:117-127 for the one-table
-rule; groups are this engine's own).
+Mixers with the same need of history form a *group* with pages of its own: one
+group for mixers that keep every key, one per window length for mixers that
+see only the last ``window`` keys. Within a group one block id names a page of
+every tensor of every mixer of the group, so a request has one table per group
+(src/alofa/engine/executor.mojo:117-127 for the one-table rule; groups are
+this engine's own). What a page holds is the mixer's business: it names its
+tensors and their page shapes (``CacheNeed.tensors``), the manager allocates
+them.
 
 A table maps the logical block (position // block_size) to a physical one, or
 -1 where no page is held: before the first token, or — in a window group —
@@ -43,13 +45,21 @@ class Group:
     pool: BlockPool
 
 
+def _keyed(needs) -> dict:
+    """Needs by the key their owner is reached with: a dict as given, or a list indexed by run entry."""
+    items = needs.items() if isinstance(needs, dict) else enumerate(needs)
+    return {k: n for k, n in items if n is not None}
+
+
 class CacheManager:
     """Accounting (integers only, in the C++ host runtime) plus, when ``device``
-    is given, the bytes: per owning entry K as [blocks, kv_heads, block_size,
-    head_dim] and V transposed as [blocks, kv_heads, head_dim, block_size], and
-    one state tensor per entry that needs one."""
+    is given, the bytes: per cache owner the tensors it asks for, each as
+    [blocks, *page shape], and one state tensor per owner of state.
+    ``cache_needs`` and ``state_needs`` map an owner's key (any hashable: the
+    model uses (run entry, mixer index)) to its need; a list stands for the keys
+    0, 1, 2, ... with None where nothing is kept."""
 
-    def __init__(self, cache_needs: list, state_needs: list, n_blocks: int, block_size: int = 16,
+    def __init__(self, cache_needs, state_needs, n_blocks: int, block_size: int = 16,
                  max_requests: int = 64, device=None, dtype=torch.bfloat16):
         if block_size <= 0 or max_requests <= 0:
             raise AlofaError("invalid_argument", "block_size and max_requests must be positive", f"block_size={block_size} max_requests={max_requests}")
@@ -60,9 +70,8 @@ class CacheManager:
         windows: list = []
         entries: list = []
         self.group_of_entry: dict = {}
-        for i, need in enumerate(cache_needs):
-            if need is None:
-                continue
+        cache_needs, state_needs = _keyed(cache_needs), _keyed(state_needs)
+        for i, need in cache_needs.items():
             if need.window not in windows:
                 windows.append(need.window)
                 entries.append([])
@@ -74,22 +83,22 @@ class CacheManager:
                                                              n_blocks, block_size, max_requests))
         self.groups = [Group(w, entries[g], BlockPool(0, _borrowed=self._lib.alofa_cache_pool(self._h, g))) for g, w in enumerate(windows)]
         self.requests: dict = {}      # request key -> its slot
-        self.needs = list(cache_needs)
-        self.state_needs = list(state_needs)
-        self.k: dict = {}
-        self.v: dict = {}
-        self.state: dict = {}
+        self.needs = cache_needs
+        self.state_needs = state_needs
+        self.tensors: dict = {}      # owner key -> {tensor name: [blocks, *page shape]}
+        self.state: dict = {}        # owner key -> [max_requests, *shape]
         self.device = device
         if device is not None:
-            for i, need in enumerate(cache_needs):
-                if need is not None:
-                    # values lie transposed, [channel][slot]: consecutive keys of a channel are contiguous,
-                    # the order in which the matrix cores reduce over keys
-                    self.k[i] = torch.zeros((n_blocks, need.kv_heads, block_size, need.head_dim), dtype=dtype, device=device)
-                    self.v[i] = torch.zeros((n_blocks, need.kv_heads, need.head_dim, block_size), dtype=dtype, device=device)
-            for i, need in enumerate(state_needs):
-                if need is not None:
-                    self.state[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+            for i, need in cache_needs.items():
+                self.tensors[i] = {t.name: torch.zeros((n_blocks, *t.page_shape(block_size)), dtype=t.dtype or dtype, device=device)
+                                   for t in need.tensors}
+            for i, need in state_needs.items():
+                self.state[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+
+    def device_bytes(self) -> int:
+        """Bytes of device memory the pages and the state slots take."""
+        return (sum(t.numel() * t.element_size() for ts in self.tensors.values() for t in ts.values())
+                + sum(t.numel() * t.element_size() for t in self.state.values()))
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -153,7 +162,7 @@ class CacheManager:
         """Let ``dst`` (fresh, empty) hold the whole blocks of ``src``'s first
         ``n_tokens`` tokens as well, by reference count; returns the tokens
         shared. Only groups that keep every key can share; state cannot be shared."""
-        if any(n is not None for n in self.state_needs):
+        if self.state_needs:
             return 0
         return hostlib.check(self._lib.alofa_cache_share_prefix(self._h, self.slot(src), self.slot(dst), ctypes.c_int64(n_tokens)))
 

@@ -23,13 +23,22 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: the arrangement (block) and the parts it arranges.
-    ``prefix`` is where its tensors live in the weight file."""
+    """One layer: the arrangement (``block``, a kind of the "block" family) and
+    the parts it arranges, under the names that block kind gives them (a
+    PartSpec or a tuple of them per name). The built-in "prenorm" block reads
+    ``mixer``, ``feed_forward`` and ``norms`` (two of them); another block kind
+    reads what it likes: several mixers, no feed-forward, other norms.
+    ``prefix`` is where the layer's tensors live in the weight file."""
     prefix: str
     block: PartSpec
-    mixer: PartSpec
-    feed_forward: PartSpec
-    norms: tuple  # PartSpec per norm the block kind asks for, in its order
+    parts: dict
+
+    def part(self, name: str):
+        if name not in self.parts:
+            from ..errors import AlofaError
+            raise AlofaError("invalid_argument", "the layer lacks a part its block kind asks for",
+                             f"prefix={self.prefix} block={self.block.kind} part={name} has={','.join(sorted(self.parts))}")
+        return self.parts[name]
 
 
 @dataclass(frozen=True)

@@ -1,3 +1,3 @@
-from .step import KVView, Span, StepContext, StepEntry, StepFunction
+from .step import CacheView, KVView, Span, StepContext, StepEntry, StepFunction
 
-__all__ = ["KVView", "Span", "StepContext", "StepEntry", "StepFunction"]
+__all__ = ["CacheView", "KVView", "Span", "StepContext", "StepEntry", "StepFunction"]

@@ -18,10 +18,6 @@ from ..cache.manager import CacheManager
 from ..errors import AlofaError
 
 
-SHORT = 4     # rows of one request up to which attention treats them as single tokens
-TILE_ROWS = 64
-
-
 def _pow2_ceil(n: int) -> int:
     return max(64, 1 << (int(n) - 1).bit_length())
 
@@ -46,14 +42,24 @@ class Span:
 
 
 @dataclass
-class KVView:
+class CacheView:
     """What a mixer sees of its cache in one step."""
-    k: torch.Tensor
-    v: torch.Tensor
+    tensors: dict                  # name -> [blocks, *page shape], as the mixer's CacheNeed named them
     block_table: torch.Tensor      # int32 [requests, max_blocks], -1 where no page
-    slots: Optional[torch.Tensor]  # int64 [T] cache slot per row
+    slots: Optional[torch.Tensor]  # int64 [T] cache slot per row (page * page size + place); None for a reader
     owner: bool                    # False: reads another entry's cache, writes nothing
     group: int
+
+    @property
+    def k(self) -> torch.Tensor:
+        return self.tensors["k"]
+
+    @property
+    def v(self) -> torch.Tensor:
+        return self.tensors["v"]
+
+
+KVView = CacheView
 
 
 class StepContext:
@@ -69,43 +75,41 @@ class StepContext:
         # launches, and a coarse value lets captured decode graphs be used again
         self.max_context = _pow2_ceil(max(s.pos0 + s.n for s in spans))
         self.n_positions = fn.n_positions
-        # how attention splits the rows: requests that bring at most SHORT rows are "short"
-        # (served key-head-wise, one token at a time), the others are cut into tiles of
-        # up to 64 rows. short_rows is None when every row is short.
-        self.n_short = sum(s.n for s in spans if s.n <= SHORT)
-        self.short_rows: Optional[torch.Tensor] = None
-        self.long_runs: Optional[list] = None         # (request index, first row, rows <= 64, first position) per tile of rows
-        self._long_tiles: dict = {}
         self.entry_slots = self.entry_tokens = None   # request slot and token count per entry, as arrays
         self.positions: torch.Tensor = None
         self.req_of_token: torch.Tensor = None
         self._tables: list = []
         self._slots: list = []
+        self._memo: dict = {}
+
+    @property
+    def device(self):
+        return self.fn.device
 
     def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
         return self.fn.scratch(name, shape, dtype)
 
-    def prefill_tiles(self, heads: int, window: Optional[int] = None) -> torch.Tensor:
-        """The runs of rows of this step's prompt portions as blocks for the prefill
-        attention kernel, for a mixer with ``heads`` query heads (how the runs share
-        blocks depends on how many blocks there are): built once per step and kind."""
-        key = (heads, window)
-        if key not in self._long_tiles:
-            self._long_tiles[key] = torch.tensor(ops.pair_tiles(self.long_runs, window, heads), dtype=torch.int32, device=self.fn.device)
-        return self._long_tiles[key]
+    def memo(self, key, build):
+        """What a kind of part derives from this step's layout once and uses in every layer
+        (how its kernels share the rows out, index tensors): ``build()`` runs at the first call."""
+        if key not in self._memo:
+            self._memo[key] = build()
+        return self._memo[key]
 
-    def kv(self, entry: int) -> KVView:
-        owner_entry = self.fn.cache_entry[entry]
-        if owner_entry is None:
-            raise AlofaError("invalid_argument", "this entry keeps no cache", f"entry={entry}")
-        g = self.fn.cache.group_of_entry[owner_entry]
-        owns = owner_entry == entry
-        return KVView(self.fn.cache.k[owner_entry], self.fn.cache.v[owner_entry], self._tables[g],
-                      self._slots[g] if owns else None, owns, g)
+    def kv(self, where) -> CacheView:
+        """The cache of the mixer at ``where`` (a run entry, or (entry, k) for the k-th mixer of its block)."""
+        where = where if isinstance(where, tuple) else (where, 0)
+        owner = self.fn.cache_owner.get(where)
+        if owner is None:
+            raise AlofaError("invalid_argument", "this mixer keeps no cache", f"where={where}")
+        g = self.fn.cache.group_of_entry[owner]
+        owns = owner == where
+        return CacheView(self.fn.cache.tensors[owner], self._tables[g], self._slots[g] if owns else None, owns, g)
 
-    def state(self, entry: int) -> torch.Tensor:
-        """Per-request state of an entry: [max_requests, *shape]; row = Span.slot."""
-        return self.fn.cache.state[entry]
+    def state(self, where) -> torch.Tensor:
+        """Per-request state of the mixer at ``where``: [max_requests, *shape]; row = Span.slot."""
+        where = where if isinstance(where, tuple) else (where, 0)
+        return self.fn.cache.state[where]
 
     def identity_rotation(self, head_dim: int):
         return self.fn.identity_rotation(head_dim)
@@ -146,23 +150,17 @@ class StepFunction:
         self._eager_scratch = self._scratch      # buffers of steps that run kernel by kernel
         self._retired: list = []                 # outgrown buffers that captured graphs may still use
         self._identity: dict = {}
-        self.cache_entry = [i if e.cache_of is None else e.cache_of for i, e in enumerate(model.order)]
-        needs = model.cache_needs()
-        self.cache_entry = [c if needs[c] is not None else None for c in self.cache_entry]
+        self.cache_owner = model.cache_owners()      # (entry, k) -> the key of the cache that mixer uses
         self.steps_run = 0
         self.rows_run = 0
         # decode steps (one token per request) replay a captured HIP graph when every
         # part runs native kernels only; ALOFA_GRAPHS=0 switches that off
-        self.use_graphs = os.environ.get("ALOFA_GRAPHS", "1") != "0" and all(
-            getattr(b.mixer, "capturable", False) and getattr(b.feed_forward, "capturable", False) for b in model.blocks)
+        self.use_graphs = os.environ.get("ALOFA_GRAPHS", "1") != "0" and model.capturable
         self._graphs: dict = {}
         self._graph_buffers: dict = {}
         self.graph_replays = 0
-        # build position tables up to the context bound once, so they never move afterwards
-        for b in model.blocks:
-            pos = getattr(b.mixer, "position", None)
-            if pos is not None:
-                pos.table(self.n_positions)
+        # what must not move once steps run (position tables up to the context bound) is built now
+        model.prepare(self.n_positions)
 
     # ------------------------------------------------------------- scratch
     def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
@@ -240,12 +238,6 @@ class StepFunction:
         ctx._tables = [tables_d[g] for g in range(n_groups)]
         ctx._slots = [slots_d[g] for g in range(n_groups)]
         rows = torch.tensor(want_rows, dtype=torch.int32, device=dev) if want_rows else None
-        if ctx.n_short < T:
-            ctx.long_runs = [(i, s.row0 + q0, min(TILE_ROWS, s.n - q0), s.pos0 + q0)
-                             for i, s in enumerate(spans) if s.n > SHORT for q0 in range(0, s.n, TILE_ROWS)]
-            if ctx.n_short:
-                ctx.short_rows = torch.tensor([r for s in spans if s.n <= SHORT for r in range(s.row0, s.row0 + s.n)],
-                                              dtype=torch.int32, device=dev)
         return ctx, ids_d, rows
 
     def finish(self, ctx: StepContext) -> None:

@@ -50,12 +50,52 @@ class Model:
         self.head = build_part("head", spec.head, weights, rt, embedding=self.embedding)
         self.order = list(spec.order)
 
-    # what the cache manager has to provide, one item per run entry
-    def cache_needs(self) -> list:
-        return [None if e.cache_of is not None else self.blocks[e.layer].mixer.cache_need() for e in self.order]
+    # What the cache manager has to provide. The blocks answer; an owner's key is (run entry, index
+    # of the mixer within its block).
+    def cache_needs(self) -> dict:
+        """{(entry, k): CacheNeed} for every mixer that keeps a cache of its own."""
+        return {(i, k): need for i, e in enumerate(self.order) if e.cache_of is None
+                for k, need in enumerate(self.blocks[e.layer].cache_needs()) if need is not None}
 
-    def state_needs(self) -> list:
-        return [self.blocks[e.layer].mixer.state_need() for e in self.order]
+    def state_needs(self) -> dict:
+        """{(entry, k): StateNeed} for every mixer that carries state per request."""
+        return {(i, k): need for i, e in enumerate(self.order)
+                for k, need in enumerate(self.blocks[e.layer].state_needs()) if need is not None}
+
+    def cache_owners(self) -> dict:
+        """{(entry, k): the key whose cache that mixer uses} — its own, or the earlier entry's that
+        ``cache_of`` names; mixers without a cache are left out."""
+        owned = self.cache_needs()
+        out = {}
+        for i, e in enumerate(self.order):
+            src = i if e.cache_of is None else e.cache_of
+            for k in range(len(self.blocks[e.layer].cache_needs())):
+                if (src, k) in owned:
+                    out[(i, k)] = (src, k)
+        return out
+
+    @property
+    def capturable(self) -> bool:
+        return all(b.capturable for b in self.blocks)
+
+    def prepare(self, n_positions: int) -> None:
+        for b in self.blocks:
+            b.prepare(n_positions)
+
+    def weight_bytes(self) -> int:
+        """Bytes of device memory the model's tensors take (a tensor shared by two parts counts once)."""
+        seen, total = set(), 0
+        stack = [self.embedding, self.final_norm, self.head, *self.blocks]
+        while stack:
+            part = stack.pop()
+            for v in vars(part).values():
+                for t in (v if isinstance(v, (list, tuple)) else [v]):
+                    if isinstance(t, torch.Tensor) and t.is_cuda and t.data_ptr() not in seen:
+                        seen.add(t.data_ptr())
+                        total += t.numel() * t.element_size()
+                    elif hasattr(t, "rt") and hasattr(t, "spec") and t is not part:
+                        stack.append(t)
+        return total
 
     def forward(self, ctx, ids: torch.Tensor) -> torch.Tensor:
         """Run the tokens of the step through every entry; returns the float32

@@ -126,9 +126,7 @@ class Qwen2Config(ModelConfig):
         layers = []
         for i in range(self.num_hidden_layers):
             p = f"model.layers.{i}."
-            layers.append(LayerSpec(
-                prefix=p,
-                block=PartSpec("prenorm"),
+            layers.append(LayerSpec(prefix=p, block=PartSpec("prenorm"), parts=dict(
                 mixer=PartSpec("gqa_attention", {
                     "prefix": p + "self_attn.", "hidden": h, "heads": self.num_attention_heads,
                     "kv_heads": self.num_key_value_heads, "head_dim": d, "qkv_bias": True,
@@ -137,7 +135,7 @@ class Qwen2Config(ModelConfig):
                     "prefix": p + "mlp.", "hidden": h, "intermediate": self.intermediate_size}),
                 norms=(PartSpec("rmsnorm", {"name": p + "input_layernorm.weight", "width": h, "eps": self.rms_norm_eps}),
                        PartSpec("rmsnorm", {"name": p + "post_attention_layernorm.weight", "width": h, "eps": self.rms_norm_eps})),
-            ))
+            )))
         return ModelSpec(
             hidden_size=h, vocab_size=self.vocab_size, max_positions=self.max_position_embeddings,
             embedding=PartSpec("token_embedding", {"name": "model.embed_tokens.weight", "vocab": self.vocab_size, "width": h}),

@@ -205,10 +205,13 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
             raise AlofaError("shape_mismatch", "bias length does not fit", f"bias={tuple(bias.shape)} N={N}")
     if add_to_out and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the residual stream is float32", f"out={out.dtype}")
+    if add_to_out and bias is not None:
+        # no kernel's residual epilogue adds a bias: the same call would otherwise give different results by dtype
+        raise AlofaError("unsupported", "a product that adds to the residual stream takes no bias; add the bias in a buffer of its own")
     if not exact and _mfma_operands(a, w):
         _ensure_workspace(a.device)
         _call(_product_entry(kernel, M, N, K), _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
-              _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(None if add_to_out else bias), _I(M), _I(N), _I(K),
+              _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
               _I(ADD_TO_RESIDUAL if add_to_out else STORE), _stream())
         return
     _call("alofa_gemm_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),

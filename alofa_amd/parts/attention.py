@@ -20,6 +20,39 @@ from ..weights.loader import TensorRule
 from .base import CacheNeed, Mixer, build_part, register_part
 
 
+SHORT = ops.DECODE_MAX_Q     # rows of one request up to which they are served as single tokens
+TILE_ROWS = 64               # rows of one block of the prefill kernel
+
+
+class RowPlan:
+    """How this part's bfloat16 kernels share out the rows of one step: requests that bring at
+    most ``SHORT`` rows are "short" (served key-head-wise, one token at a time, by the decode
+    kernel), the others are cut into runs of up to ``TILE_ROWS`` rows for the prefill kernel.
+    Built once per step from the spans and used by every attention layer."""
+
+    def __init__(self, ctx):
+        spans = ctx.spans
+        self.device = ctx.device
+        self.n_short = sum(s.n for s in spans if s.n <= SHORT)
+        self.short_rows = None      # int32 indices of the short rows; None when every row is short (or none is)
+        self.long_runs = None       # (request index, first row, rows, first position) per run; None when every row is short
+        self._tiles: dict = {}
+        if self.n_short < ctx.tokens:
+            self.long_runs = [(i, s.row0 + q0, min(TILE_ROWS, s.n - q0), s.pos0 + q0)
+                              for i, s in enumerate(spans) if s.n > SHORT for q0 in range(0, s.n, TILE_ROWS)]
+            if self.n_short:
+                self.short_rows = torch.tensor([r for s in spans if s.n <= SHORT for r in range(s.row0, s.row0 + s.n)],
+                                               dtype=torch.int32, device=self.device)
+
+    def tiles(self, heads: int, window) -> torch.Tensor:
+        """The runs as blocks of the prefill kernel for a mixer with ``heads`` query heads (how runs
+        share blocks depends on how many blocks there are)."""
+        key = (heads, window)
+        if key not in self._tiles:
+            self._tiles[key] = torch.tensor(ops.pair_tiles(self.long_runs, window, heads), dtype=torch.int32, device=self.device)
+        return self._tiles[key]
+
+
 class GQAAttention(Mixer):
     """params: prefix, hidden, heads, kv_heads, head_dim, qkv_bias, out_bias,
     window (None or a count of keys), position (PartSpec)."""
@@ -65,7 +98,10 @@ class GQAAttention(Mixer):
         self.capturable = self.position.table(1) is not None   # an encoding applied by other code is not captured
 
     def cache_need(self):
-        return CacheNeed(self.kv_heads, self.d, self.window)
+        return CacheNeed.keys_and_values(self.kv_heads, self.d, self.window)
+
+    def prepare(self, n_positions):
+        self.position.table(n_positions)       # built up to the context bound once, so that it never moves afterwards
 
     def forward(self, ctx, entry, x, residual):
         T = x.shape[0]
@@ -73,6 +109,7 @@ class GQAAttention(Mixer):
         qkv = ctx.scratch("qkv", (T, self.qkv_width), self.rt.dtype)
         ops.gemm(qkv, x, self.w_qkv, self.b_qkv, exact=exact)
         kv = ctx.kv(entry)
+        plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
         table = self.position.table(ctx.n_positions)
         if table is None:
             hd = self.heads * self.d
@@ -85,7 +122,7 @@ class GQAAttention(Mixer):
         pow2_pages = kv.k.shape[2] >= ops.MIN_FAST_PAGE and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
         fast_prefill = self.d in ops.PREFILL_HEAD_DIMS
         # one new token per request: the decode kernel rotates it and writes its cache slot itself
-        fused = (not exact and pow2_pages and kv.owner and ctx.max_q_len == 1 and ctx.long_runs is None
+        fused = (not exact and pow2_pages and kv.owner and ctx.max_q_len == 1 and plan.long_runs is None
                  and ops.can_fuse_rope_into_decode(self.d))
         if fused:
             pass
@@ -93,19 +130,19 @@ class GQAAttention(Mixer):
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d, kv.slots, kv.k, kv.v)
         else:
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
-        if exact or not pow2_pages or (ctx.long_runs is not None and not fast_prefill):
+        if exact or not pow2_pages or (plan.long_runs is not None and not fast_prefill):
             # the exact path, and page or head sizes the bfloat16 kernels are not built for
             ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
         else:
-            if ctx.long_runs is not None:       # portions of prompts
-                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, ctx.prefill_tiles(self.heads, self.window), *common)
-            if ctx.n_short:                     # single tokens and very short portions, all query heads of a key head together
-                floats = ops.decode_scratch_floats(ctx.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
+            if plan.long_runs is not None:      # portions of prompts
+                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, plan.tiles(self.heads, self.window), *common)
+            if plan.n_short:                    # single tokens and very short portions, all query heads of a key head together
+                floats = ops.decode_scratch_floats(plan.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
                 partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
                 # (one token per request and nothing else in the step: token i is request i)
-                one_each = ctx.max_q_len == 1 and ctx.short_rows is None and ctx.long_runs is None
+                one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
                 ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, None if one_each else ctx.req_of_token, ctx.positions, *common,
-                                     ctx.max_context, partial, rows=ctx.short_rows, rope=(cos, sin, kv.slots) if fused else None)
+                                     ctx.max_context, partial, rows=plan.short_rows, rope=(cos, sin, kv.slots) if fused else None)
         if self.b_o is not None:
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
             ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)

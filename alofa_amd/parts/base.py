@@ -7,16 +7,19 @@ dtype, ``residual`` the float32 residual stream):
 
   norm          forward(out[n,h], x[T,h] f32, rows=None)         out = norm(x[rows])
   position      table(n_positions) -> (cos, sin) f32 [n, d/2], or apply(ctx, q, k)
-  mixer         forward(ctx, entry, x, residual)                  residual += mix(x)
-                cache_need() -> CacheNeed | None, state_need() -> StateNeed | None
-  feed_forward  forward(ctx, x, residual)                         residual += ff(x)
-  block         forward(ctx, entry, hidden)                       one layer on the stream
+  mixer         forward(ctx, where, x, residual)                  residual += mix(x)
+                cache_need() -> CacheNeed | None, state_need() -> StateNeed | None,
+                prepare(n_positions), capturable
+  feed_forward  forward(ctx, x, residual)                         residual += ff(x); capturable
+  block         built from a LayerSpec; layer_tensors(layer); mixers() (the parts that may keep
+                a cache or state, in a fixed order); cache_needs(), state_needs(), capturable,
+                prepare(n_positions); forward(ctx, entry, hidden)  one layer on the stream
   embedding     forward(ctx, ids) -> hidden[T,h] f32
   head          forward(ctx, y[S,h]) -> logits[S,V] f32
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional
 
 import torch
@@ -45,9 +48,12 @@ def part_class(family: str, kind: str):
 @dataclass(frozen=True)
 class Runtime:
     """Where and how parts compute. ``dtype`` float32 means the exact path:
-    float32 storage, float64 accumulation, no reduced-precision matrix mode."""
+    float32 storage, float64 accumulation, no reduced-precision matrix mode.
+    ``shared`` holds what parts of one model build once and use together (a
+    position table that many layers read)."""
     device: torch.device
     dtype: torch.dtype
+    shared: dict = field(default_factory=dict, compare=False, repr=False)
 
     @property
     def exact(self) -> bool:
@@ -65,13 +71,39 @@ class Runtime:
         return t.to(device=self.device, dtype=torch.float32).contiguous()
 
 
+SLOT = -1     # in CacheTensor.dims: where the token's place within its page goes
+
+
+@dataclass(frozen=True)
+class CacheTensor:
+    """One tensor a mixer keeps per token in pages. ``dims`` is the shape of one page with ``SLOT``
+    standing for the tokens of the page: (kv_heads, SLOT, head_dim) lays the tokens of a page out
+    one after the other per head; (kv_heads, head_dim, SLOT) keeps them transposed; (SLOT, width)
+    is one vector per token. The cache manager allocates [pages, *dims] with the page size in
+    SLOT's place. ``dtype`` None: the runtime's activation dtype."""
+    name: str
+    dims: tuple
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, block_size: int) -> tuple:
+        if tuple(self.dims).count(SLOT) != 1 or any(d <= 0 for d in self.dims if d != SLOT):
+            raise AlofaError("invalid_argument", "a cache tensor's dims hold positive sizes and SLOT exactly once", f"name={self.name} dims={self.dims}")
+        return tuple(block_size if d == SLOT else int(d) for d in self.dims)
+
+
 @dataclass(frozen=True)
 class CacheNeed:
-    """Keys and values per token that a mixer keeps in pages. ``window`` None:
-    every earlier token stays visible; else only the last ``window`` ones."""
-    kv_heads: int
-    head_dim: int
+    """What a mixer keeps per token in pages: any number of named tensors. ``window`` None: every
+    earlier token stays visible; else only the last ``window`` ones, and pages the window has
+    passed go back to the pool. Mixers with the same window share block tables (a group)."""
+    tensors: tuple
     window: Optional[int] = None
+
+    @staticmethod
+    def keys_and_values(kv_heads: int, head_dim: int, window: Optional[int] = None) -> "CacheNeed":
+        """Keys "k" as [kv_heads, slot, head_dim]; values "v" transposed, [kv_heads, head_dim, slot]: consecutive
+        keys of a channel are contiguous, the order in which the matrix cores reduce over keys."""
+        return CacheNeed((CacheTensor("k", (kv_heads, SLOT, head_dim)), CacheTensor("v", (kv_heads, head_dim, SLOT))), window)
 
 
 @dataclass(frozen=True)
@@ -97,7 +129,10 @@ class Part:
 
 
 class Mixer(Part):
+    """``where`` names the mixer's place in the run: the run entry, or (entry, k) for the k-th
+    mixer of a block that has several; it is what ``ctx.kv`` and ``ctx.state`` are asked with."""
     family = "mixer"
+    capturable = False      # True: native kernels on the current stream only, so a decode step may be graph-captured
 
     def cache_need(self) -> Optional[CacheNeed]:
         return None
@@ -105,14 +140,58 @@ class Mixer(Part):
     def state_need(self) -> Optional[StateNeed]:
         return None
 
-    def forward(self, ctx, entry: int, x: torch.Tensor, residual: torch.Tensor) -> None:
+    def prepare(self, n_positions: int) -> None:
+        """Build what must not move once steps run (tables up to the context bound)."""
+
+    def forward(self, ctx, where, x: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
     family = "feed_forward"
+    capturable = False
 
     def forward(self, ctx, x: torch.Tensor, residual: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of parts in one layer. It answers for its parts: what they keep per token
+    and per request, whether a decode step through it may be graph-captured, and what has to be
+    built before the first step. Model, cache manager and step function ask the block and never
+    reach into it, so a block kind with several mixers, or none, or no feed-forward, is an
+    addition. Subclasses set ``self.parts`` (every part, for ``capturable``) and implement
+    ``layer_tensors``, ``mixers`` and ``forward``."""
+    family = "block"
+
+    @classmethod
+    def layer_tensors(cls, layer) -> dict:
+        raise NotImplementedError
+
+    def __init__(self, layer, weights: dict, rt: Runtime):
+        super().__init__(layer.block, weights, rt)
+        self.layer = layer
+        self.parts: list = []
+
+    def mixers(self) -> list:
+        """The parts that may keep a cache or state, in a fixed order; mixer k is reached as (entry, k)."""
+        return []
+
+    def cache_needs(self) -> list:
+        return [m.cache_need() for m in self.mixers()]
+
+    def state_needs(self) -> list:
+        return [m.state_need() for m in self.mixers()]
+
+    @property
+    def capturable(self) -> bool:
+        return all(getattr(p, "capturable", True) for p in self.parts)
+
+    def prepare(self, n_positions: int) -> None:
+        for m in self.mixers():
+            m.prepare(n_positions)
+
+    def forward(self, ctx, entry: int, hidden: torch.Tensor) -> None:
         raise NotImplementedError
 
 

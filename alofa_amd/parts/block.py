@@ -2,33 +2,38 @@
 
 prenorm: a = hidden; a += mixer(norm0(a)); a += feed_forward(norm1(a)) — two
 norms before their sub-layers, two residual sums in float32
-(src/alofa/model/arch/qwen.mojo:1418-1510)."""
+(src/alofa/model/arch/qwen.mojo:1418-1510). It reads the layer's parts
+``mixer``, ``feed_forward`` and ``norms`` (two)."""
 from __future__ import annotations
 
 from ..errors import AlofaError
-from .base import Part, build_part, register_part, tensors_of
+from .base import Block, build_part, register_part, tensors_of
 
 
-class PreNormBlock(Part):
-    family = "block"
+class PreNormBlock(Block):
     n_norms = 2
 
     @classmethod
     def layer_tensors(cls, layer) -> dict:
         out = {}
-        for n in layer.norms:
+        for n in layer.part("norms"):
             out.update(tensors_of("norm", n))
-        out.update(tensors_of("mixer", layer.mixer))
-        out.update(tensors_of("feed_forward", layer.feed_forward))
+        out.update(tensors_of("mixer", layer.part("mixer")))
+        out.update(tensors_of("feed_forward", layer.part("feed_forward")))
         return out
 
     def __init__(self, layer, weights, rt):
-        super().__init__(layer.block, weights, rt)
-        if len(layer.norms) != self.n_norms:
-            raise AlofaError("invalid_argument", "a prenorm block takes two norms", f"prefix={layer.prefix} norms={len(layer.norms)}")
-        self.norms = [build_part("norm", n, weights, rt) for n in layer.norms]
-        self.mixer = build_part("mixer", layer.mixer, weights, rt)
-        self.feed_forward = build_part("feed_forward", layer.feed_forward, weights, rt)
+        super().__init__(layer, weights, rt)
+        norms = layer.part("norms")
+        if len(norms) != self.n_norms:
+            raise AlofaError("invalid_argument", "a prenorm block takes two norms", f"prefix={layer.prefix} norms={len(norms)}")
+        self.norms = [build_part("norm", n, weights, rt) for n in norms]
+        self.mixer = build_part("mixer", layer.part("mixer"), weights, rt)
+        self.feed_forward = build_part("feed_forward", layer.part("feed_forward"), weights, rt)
+        self.parts = [*self.norms, self.mixer, self.feed_forward]
+
+    def mixers(self):
+        return [self.mixer]
 
     def forward(self, ctx, entry, hidden):
         normed = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)

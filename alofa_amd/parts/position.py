@@ -27,7 +27,6 @@ class Rotary(PositionEncoding):
             raise AlofaError("unsupported", "only the half-split pairing (j, j + d/2) is built", f"pairing={spec.params['pairing']}")
         if self.head_dim <= 0 or self.head_dim % 2:
             raise AlofaError("unsupported", "head dimension must be positive and even", f"head_dim={self.head_dim}")
-        self._table = None
 
     def host_table(self, n_positions: int):
         half = self.head_dim // 2
@@ -39,11 +38,18 @@ class Rotary(PositionEncoding):
         return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
 
     def table(self, n_positions: int):
-        if self._table is None or self._table[0].shape[0] < n_positions:
-            n = max(n_positions, 2 * self._table[0].shape[0] if self._table else 0)
+        """One table per (theta, head size) serves every layer of the model (kept on the runtime).
+        A table that has to grow is replaced; the old one is kept alive, since a captured graph
+        may still read it (for positions it covers)."""
+        key = ("rotary", self.theta, self.head_dim)
+        have = self.rt.shared.get(key)
+        if have is None or have[0].shape[0] < n_positions:
+            n = max(n_positions, 2 * have[0].shape[0] if have else 0)
             c, s = self.host_table(n)
-            self._table = (torch.from_numpy(c).to(self.rt.device), torch.from_numpy(s).to(self.rt.device))
-        return self._table
+            if have is not None:
+                self.rt.shared.setdefault("retired tables", []).append(have)
+            have = self.rt.shared[key] = (torch.from_numpy(c).to(self.rt.device), torch.from_numpy(s).to(self.rt.device))
+        return have
 
 
 class NoPosition(PositionEncoding):
@@ -54,14 +60,17 @@ class NoPosition(PositionEncoding):
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         self.head_dim = int(spec.params["head_dim"])
-        self._table = None
 
     def table(self, n_positions: int):
-        if self._table is None or self._table[0].shape[0] < n_positions:
+        key = ("no rotation", self.head_dim)
+        have = self.rt.shared.get(key)
+        if have is None or have[0].shape[0] < n_positions:
             half = self.head_dim // 2
-            self._table = (torch.ones(n_positions, half, dtype=torch.float32, device=self.rt.device),
-                           torch.zeros(n_positions, half, dtype=torch.float32, device=self.rt.device))
-        return self._table
+            if have is not None:
+                self.rt.shared.setdefault("retired tables", []).append(have)
+            have = self.rt.shared[key] = (torch.ones(n_positions, half, dtype=torch.float32, device=self.rt.device),
+                                          torch.zeros(n_positions, half, dtype=torch.float32, device=self.rt.device))
+        return have
 
 
 register_part("position", "rotary", Rotary)

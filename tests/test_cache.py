@@ -32,7 +32,7 @@ def test_pool_order_and_errors():
 
 
 def manager(n_blocks=12, windows=(None, 24, 24, None), state=False, bs=8):
-    needs = [CacheNeed(2, 16, w) for w in windows]
+    needs = [CacheNeed.keys_and_values(2, 16, w) for w in windows]
     states = [StateNeed((4,)) if state else None for _ in windows]
     return CacheManager(needs, states, n_blocks, bs, max_requests=4)
 
@@ -41,7 +41,7 @@ def test_groups_by_need():
     m = manager()
     assert [(g.window, g.entries) for g in m.groups] == [(None, [0, 3]), (24, [1, 2])]
     assert m.group_of_entry == {0: 0, 3: 0, 1: 1, 2: 1}
-    shared = CacheManager([CacheNeed(1, 16), None, CacheNeed(1, 16)], [None] * 3, 4, 8)
+    shared = CacheManager([CacheNeed.keys_and_values(1, 16), None, CacheNeed.keys_and_values(1, 16)], [None] * 3, 4, 8)
     assert shared.groups[0].entries == [0, 2]
 
 

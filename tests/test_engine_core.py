@@ -29,7 +29,7 @@ class FakeStep:
     twice or a wrongly shared page shows in the output."""
 
     def __init__(self, n_blocks, block_size, n_positions=4096, max_requests=64):
-        self.cache = CacheManager([CacheNeed(1, 16, None)], [None], n_blocks, block_size, max_requests=max_requests)
+        self.cache = CacheManager([CacheNeed.keys_and_values(1, 16)], [None], n_blocks, block_size, max_requests=max_requests)
         self.n_positions = n_positions
         self.model = SimpleNamespace(spec=SimpleNamespace(vocab_size=VOCAB))
         self.store = np.full(n_blocks * block_size, -1, dtype=np.int64)

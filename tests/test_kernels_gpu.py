@@ -451,6 +451,12 @@ def test_kernels_refuse_what_they_cannot_take():
         o.rmsnorm(torch.empty(2, 8, device=DEV, dtype=torch.bfloat16), torch.empty(2, 8, device=DEV), torch.empty(8, device=DEV), 1e-6, True)
     with pytest.raises(AlofaError):
         o.argmax(torch.empty(2, dtype=torch.int32, device=DEV), torch.empty(3, 8, device=DEV))
+    # a product that adds to the residual stream takes no bias, in either dtype (no kernel would add it)
+    for dt in (torch.float32, torch.bfloat16):
+        with pytest.raises(AlofaError) as e:
+            o.gemm(torch.zeros(2, 8, device=DEV), torch.zeros(2, 16, device=DEV, dtype=dt), torch.zeros(8, 16, device=DEV, dtype=dt),
+                   torch.zeros(8, device=DEV), add_to_out=True, exact=dt is torch.float32)
+        assert e.value.name == "unsupported"
 
 
 def test_product_kernel_choice():

@@ -102,11 +102,11 @@ def test_attention_without_positions_is_library_attention(tmp_path):
     from alofa_amd.model import Model, expected_tensors, runtime
     from alofa_amd.weights import random_tensors
     h, H, d, V, T = 64, 4, 16, 50, 23
-    layer = LayerSpec("l.", PartSpec("prenorm"),
-                      PartSpec("gqa_attention", {"prefix": "l.att.", "hidden": h, "heads": H, "kv_heads": H, "head_dim": d, "qkv_bias": False,
-                                                 "out_bias": True, "window": None, "position": PartSpec("none", {"head_dim": d})}),
-                      PartSpec("swiglu", {"prefix": "l.ff.", "hidden": h, "intermediate": 32}),
-                      (PartSpec("rmsnorm", {"name": "l.n0", "width": h, "eps": 1e-6}), PartSpec("rmsnorm", {"name": "l.n1", "width": h, "eps": 1e-6})))
+    layer = LayerSpec("l.", PartSpec("prenorm"), dict(
+        mixer=PartSpec("gqa_attention", {"prefix": "l.att.", "hidden": h, "heads": H, "kv_heads": H, "head_dim": d, "qkv_bias": False,
+                                         "out_bias": True, "window": None, "position": PartSpec("none", {"head_dim": d})}),
+        feed_forward=PartSpec("swiglu", {"prefix": "l.ff.", "hidden": h, "intermediate": 32}),
+        norms=(PartSpec("rmsnorm", {"name": "l.n0", "width": h, "eps": 1e-6}), PartSpec("rmsnorm", {"name": "l.n1", "width": h, "eps": 1e-6}))))
     spec = ModelSpec(h, V, 64, PartSpec("token_embedding", {"name": "emb", "vocab": V, "width": h}), (layer,), (RunEntry(0),),
                      PartSpec("rmsnorm", {"name": "nf", "width": h, "eps": 1e-6}), PartSpec("lm_head", {"name": "head", "tied_to": "emb", "vocab": V, "width": h}))
     exp = expected_tensors(spec)
@@ -192,8 +192,9 @@ def register_toy():
             att = PartSpec("gqa_attention", {"prefix": "b.att.", "hidden": h, "heads": self.heads, "kv_heads": 1, "head_dim": self.head_dim,
                                              "qkv_bias": True, "out_bias": False, "window": None,
                                              "position": PartSpec("rotary", {"theta": 10000.0, "head_dim": self.head_dim})})
-            layers = (LayerSpec("a.", PartSpec("prenorm"), PartSpec("toy_running_mean", {"prefix": "a.", "hidden": h}), ff("a."), norms("a.")),
-                      LayerSpec("b.", PartSpec("prenorm"), att, ff("b."), norms("b.")))
+            layers = (LayerSpec("a.", PartSpec("prenorm"), dict(mixer=PartSpec("toy_running_mean", {"prefix": "a.", "hidden": h}),
+                                                               feed_forward=ff("a."), norms=norms("a."))),
+                      LayerSpec("b.", PartSpec("prenorm"), dict(mixer=att, feed_forward=ff("b."), norms=norms("b."))))
             # layer a runs twice (two states), layer b runs twice, the second time reading the first run's cache
             order = (RunEntry(0), RunEntry(1), RunEntry(0), RunEntry(1, cache_of=1))
             return ModelSpec(h, self.vocab, 256, PartSpec("token_embedding", {"name": "emb.weight", "vocab": self.vocab, "width": h}),
@@ -244,9 +245,9 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, dtype):
     assert json.loads((tmp_path / "config.json").read_text())["architectures"] == ["ToyMixForCausalLM"]
     w = pm.read_weights(tmp_path)
     r = Replayer(tmp_path, dtype, 512)
-    assert r.model.state_needs()[0] is not None and r.model.state_needs()[1] is None and r.model.state_needs()[2] is not None
-    assert [n is not None for n in r.model.cache_needs()] == [False, True, False, False]     # entry 3 reads entry 1's cache
-    assert set(r.cache.state) == {0, 2} and set(r.cache.k) == {1}
+    assert set(r.model.state_needs()) == {(0, 0), (2, 0)}
+    assert set(r.model.cache_needs()) == {(1, 0)} and r.model.cache_owners() == {(1, 0): (1, 0), (3, 0): (1, 0)}   # entry 3 reads entry 1's cache
+    assert set(r.cache.state) == {(0, 0), (2, 0)} and set(r.cache.tensors) == {(1, 0)}
     requests = {f"q{i}": random_ids(40 + i, n, 97) for i, n in enumerate([90, 45, 70, 64, 50])}
     refs = {k: toy_plain(w, ids, 3, 16) for k, ids in requests.items()}
     assert_close(collect(r, whole("w", requests["q0"]))["w"], refs["q0"], dtype, "toy whole")
@@ -341,10 +342,13 @@ def register_toy_routed():
             def att(p, position):
                 return PartSpec("gqa_attention", {"prefix": p + "att.", "hidden": h, "heads": self.heads, "kv_heads": 1, "head_dim": self.head_dim,
                                                   "qkv_bias": True, "out_bias": False, "window": None, "position": position})
-            layers = (LayerSpec("a.", PartSpec("prenorm"), att("a.", PartSpec("toy_added_wave", {"head_dim": self.head_dim, "amp": 0.5, "base": 50.0})),
-                                PartSpec("toy_routed", {"prefix": "a.moe.", "hidden": h, "intermediate": self.inter, "experts": TOY_EXPERTS}), norms("a.")),
-                      LayerSpec("b.", PartSpec("prenorm"), att("b.", PartSpec("rotary", {"theta": 10000.0, "head_dim": self.head_dim})),
-                                PartSpec("swiglu", {"prefix": "b.ff.", "hidden": h, "intermediate": self.inter}), norms("b.")))
+            layers = (LayerSpec("a.", PartSpec("prenorm"), dict(
+                          mixer=att("a.", PartSpec("toy_added_wave", {"head_dim": self.head_dim, "amp": 0.5, "base": 50.0})),
+                          feed_forward=PartSpec("toy_routed", {"prefix": "a.moe.", "hidden": h, "intermediate": self.inter, "experts": TOY_EXPERTS}),
+                          norms=norms("a."))),
+                      LayerSpec("b.", PartSpec("prenorm"), dict(
+                          mixer=att("b.", PartSpec("rotary", {"theta": 10000.0, "head_dim": self.head_dim})),
+                          feed_forward=PartSpec("swiglu", {"prefix": "b.ff.", "hidden": h, "intermediate": self.inter}), norms=norms("b."))))
             return ModelSpec(h, self.vocab, 256, PartSpec("token_embedding", {"name": "emb.weight", "vocab": self.vocab, "width": h}),
                              layers, (RunEntry(0), RunEntry(1)), PartSpec("rmsnorm", {"name": "nf.weight", "width": h, "eps": 1e-5}),
                              PartSpec("lm_head", {"name": "head.weight", "tied_to": None, "vocab": self.vocab, "width": h}))
@@ -425,4 +429,158 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(tmp_path, dtype):
     got = collect(r, steps)
     for k in requests:
         assert_close(got[k], refs[k], dtype, f"toy routed mixed {k}")
+    r.cache.check()
+
+
+# ------------------- a toy block with two mixers side by side and no feed-forward; a mixer that caches one vector per token
+
+def register_toy_parallel():
+    """Defined outside the engine: a block kind that runs two mixers on the same normed input and
+    adds both to the stream, with no feed-forward at all, and a mixer that keeps ONE vector per
+    token in pages (not keys and values): its output at position t is the mean of the cached
+    vectors of positions 0..t, times a matrix. The block answers for both mixers' needs; the
+    cache manager allocates the page layout the mixer names."""
+    from alofa_amd.config import LayerSpec, ModelConfig, ModelSpec, PartSpec, RunEntry, register_architecture
+    from alofa_amd.parts import SLOT, Block, CacheNeed, CacheTensor, Mixer, build_part, register_part, tensors_of
+    from alofa_amd.weights import TensorRule
+
+    class LatentMean(Mixer):
+        @classmethod
+        def tensors(cls, spec):
+            p = spec.params
+            return {p["prefix"] + "down.weight": TensorRule((p["rank"], p["hidden"])), p["prefix"] + "up.weight": TensorRule((p["hidden"], p["rank"]))}
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            p = spec.params
+            self.rank = p["rank"]
+            self.down = weights[p["prefix"] + "down.weight"].to(rt.device, torch.float32)
+            self.up = weights[p["prefix"] + "up.weight"].to(rt.device, torch.float32)
+
+        def cache_need(self):
+            return CacheNeed((CacheTensor("latent", (SLOT, self.rank), torch.float32),), None)
+
+        def forward(self, ctx, where, x, residual):
+            view = ctx.kv(where)
+            pages = view.tensors["latent"]                      # [blocks, page, rank]
+            bs = pages.shape[1]
+            flat = pages.view(-1, self.rank)
+            flat[view.slots] = x.float() @ self.down.T          # this step's vectors go to their slots
+            for i, sp in enumerate(ctx.spans):
+                at = torch.arange(sp.pos0 + sp.n, device=x.device)
+                mine = flat[view.block_table[i, at // bs].long() * bs + at % bs]      # read back through the table
+                means = torch.cumsum(mine, dim=0)[sp.pos0:] / (at[sp.pos0:] + 1)[:, None]
+                residual[sp.row0:sp.row0 + sp.n] += means @ self.up.T
+
+    class ParallelBlock(Block):
+        @classmethod
+        def layer_tensors(cls, layer):
+            out = dict(tensors_of("norm", layer.part("norm")))
+            for m in layer.part("mixers"):
+                out.update(tensors_of("mixer", m))
+            return out
+
+        def __init__(self, layer, weights, rt):
+            super().__init__(layer, weights, rt)
+            self.norm = build_part("norm", layer.part("norm"), weights, rt)
+            self.both = [build_part("mixer", m, weights, rt) for m in layer.part("mixers")]
+            self.parts = [self.norm, *self.both]
+
+        def mixers(self):
+            return self.both
+
+        def forward(self, ctx, entry, hidden):
+            normed = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
+            self.norm.forward(normed, hidden)
+            for k, m in enumerate(self.both):
+                m.forward(ctx, (entry, k), normed, hidden)
+
+    @dataclasses.dataclass(frozen=True)
+    class ToyParallelConfig(ModelConfig):
+        hidden: int
+        vocab: int
+        heads: int
+        head_dim: int
+        inter: int
+        rank: int
+        window: int
+        architecture = "ToyParallelForCausalLM"
+
+        @classmethod
+        def from_dict(cls, raw, where="<dict>"):
+            return cls(*(raw[f.name] for f in dataclasses.fields(cls)))
+
+        def to_dict(self):
+            return dict(dataclasses.asdict(self), architectures=[self.architecture])
+
+        def spec(self):
+            h = self.hidden
+
+            def norm(name):
+                return PartSpec("rmsnorm", {"name": name, "width": h, "eps": 1e-5})
+
+            def att(p, window):
+                return PartSpec("gqa_attention", {"prefix": p + "att.", "hidden": h, "heads": self.heads, "kv_heads": 1, "head_dim": self.head_dim,
+                                                  "qkv_bias": True, "out_bias": False, "window": window,
+                                                  "position": PartSpec("rotary", {"theta": 10000.0, "head_dim": self.head_dim})})
+            layers = (LayerSpec("a.", PartSpec("toy_parallel"), dict(
+                          norm=norm("a.n.weight"), mixers=(att("a.", self.window), PartSpec("toy_latent_mean", {"prefix": "a.lat.", "hidden": h, "rank": self.rank})))),
+                      LayerSpec("b.", PartSpec("prenorm"), dict(
+                          mixer=att("b.", None), feed_forward=PartSpec("swiglu", {"prefix": "b.ff.", "hidden": h, "intermediate": self.inter}),
+                          norms=(norm("b.n0.weight"), norm("b.n1.weight")))))
+            return ModelSpec(h, self.vocab, 256, PartSpec("token_embedding", {"name": "emb.weight", "vocab": self.vocab, "width": h}),
+                             layers, (RunEntry(0), RunEntry(1)), norm("nf.weight"),
+                             PartSpec("lm_head", {"name": "head.weight", "tied_to": None, "vocab": self.vocab, "width": h}))
+
+    register_part("mixer", "toy_latent_mean", LatentMean)
+    register_part("block", "toy_parallel", ParallelBlock)
+    register_architecture("ToyParallelForCausalLM", ToyParallelConfig)
+
+
+def toy_parallel_plain(w, ids, heads, d, window):
+    f64 = np.float64
+    hid = pm.embed(w["emb.weight"], ids)
+    T = len(ids)
+    pos = np.arange(T)
+    cos, sin = pm.rope_table(T, d, 10000.0)
+
+    def att(p, n, win):
+        q = pm.rope_apply(pm.linear(n, w[p + "att.q_proj.weight"], w[p + "att.q_proj.bias"]), cos, sin, pos, d)
+        k = pm.rope_apply(pm.linear(n, w[p + "att.k_proj.weight"], w[p + "att.k_proj.bias"]), cos, sin, pos, d)
+        v = pm.linear(n, w[p + "att.v_proj.weight"], w[p + "att.v_proj.bias"])
+        return pm.linear(pm.attention(q, k, v, heads, 1, d, win), w[p + "att.o_proj.weight"])
+    n = pm.rmsnorm(hid, w["a.n.weight"], 1e-5)
+    latent = n.astype(f64) @ w["a.lat.down.weight"].astype(f64).T
+    means = np.cumsum(latent, axis=0) / np.arange(1, T + 1)[:, None]
+    hid = pm.add(pm.add(hid, att("a.", n, window)), (means @ w["a.lat.up.weight"].astype(f64).T).astype(np.float32))   # no feed-forward
+    hid = pm.add(hid, att("b.", pm.rmsnorm(hid, w["b.n0.weight"], 1e-5), None))
+    n = pm.rmsnorm(hid, w["b.n1.weight"], 1e-5)
+    hid = pm.add(hid, pm.linear(pm.swiglu(pm.linear(n, w["b.ff.gate_proj.weight"]), pm.linear(n, w["b.ff.up_proj.weight"])), w["b.ff.down_proj.weight"]))
+    return pm.linear(pm.rmsnorm(hid, w["nf.weight"], 1e-5), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_block_with_two_mixers_and_a_mixer_with_its_own_page_layout(tmp_path, dtype):
+    from helpers import collect, mixed, portions, whole
+    from alofa_amd.replay import Replayer
+    from alofa_amd.weights import write_random_model
+    register_toy_parallel()
+    raw = {"architectures": ["ToyParallelForCausalLM"], "hidden": 48, "vocab": 89, "heads": 3, "head_dim": 16, "inter": 40, "rank": 5, "window": 24}
+    write_random_model(raw, tmp_path, seed=13, std=0.06)
+    w = pm.read_weights(tmp_path)
+    r = Replayer(tmp_path, dtype, 512)
+    # the block answered for both of its mixers; the manager laid the pages out as each asked
+    assert set(r.model.cache_needs()) == {(0, 0), (0, 1), (1, 0)} and not r.model.state_needs()
+    assert [g.window for g in r.cache.groups] == [24, None] and r.cache.groups[1].entries == [(0, 1), (1, 0)]
+    assert tuple(r.cache.tensors[(0, 1)]["latent"].shape[1:]) == (16, 5) and r.cache.tensors[(0, 1)]["latent"].dtype is torch.float32
+    assert set(r.cache.tensors[(0, 0)]) == {"k", "v"} and not r.fn.use_graphs
+    requests = {f"q{i}": random_ids(80 + i, n, 89) for i, n in enumerate([90, 45, 70, 64, 50])}
+    refs = {k: toy_parallel_plain(w, ids, 3, 16, 24) for k, ids in requests.items()}
+    assert_close(collect(r, whole("w", requests["q0"]))["w"], refs["q0"], dtype, "toy parallel whole")
+    assert_close(collect(r, portions("p", requests["q0"]))["p"], refs["q0"], dtype, "toy parallel portions")
+    steps, peak = mixed(requests, seed=4)
+    r = Replayer(tmp_path, dtype, peak)
+    got = collect(r, steps)
+    for k in requests:
+        assert_close(got[k], refs[k], dtype, f"toy parallel mixed {k}")
     r.cache.check()
