@@ -2,6 +2,8 @@
 batches of prompts (token ids; the tokenizer is outside this engine)."""
 from __future__ import annotations
 
+import os
+import sys
 from pathlib import Path
 from typing import Optional
 
@@ -25,10 +27,13 @@ class Engine:
     def __init__(self, model_dir, dtype: str = "bfloat16", max_tokens: int = 256, max_batch: int = 8,
                  kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 2048, max_chunk: int = 512,
                  watermark_permille: int = 900, max_wait_ticks: int = 8, seed: int = 1234, device: str = "cuda:0",
-                 trace_path=None, share_prefixes: bool = False):
+                 trace_path=None, share_prefixes: bool = False, model=None, report=None):
+        """``model``: a (config, Model) pair already on the device, instead of a folder to load.
+        ``report``: a callable that receives one line about device memory at start (default:
+        standard error when ALOFA_REPORT_MEMORY is set)."""
         from .csrc.build import load
         load()
-        self.config, self.model = load_model(Path(model_dir), dtype, device)
+        self.config, self.model = model if model is not None else load_model(Path(model_dir), dtype, device)
         if max_tokens > self.model.spec.max_positions:
             raise AlofaError("out_of_range", "max_tokens passes the model's position bound", f"max_tokens={max_tokens} max_position_embeddings={self.model.spec.max_positions}")
         per_request = (max_tokens + block_size - 1) // block_size
@@ -43,6 +48,19 @@ class Engine:
         self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path, share_prefixes=share_prefixes)
         self.seed = seed
         self._next_id = 1
+        if report is None and os.environ.get("ALOFA_REPORT_MEMORY"):
+            report = lambda line: print(line, file=sys.stderr, flush=True)   # noqa: E731
+        if report is not None:
+            m = self.memory()
+            report(f"[alofa_amd] device memory: weights {m['weights'] / 2**20:.1f} MiB + cache pool {m['cache_pool'] / 2**20:.1f} MiB "
+                   f"({kv_blocks} pages of {block_size} tokens x {len(self.cache.groups)} group(s)) + scratch {m['scratch'] / 2**20:.1f} MiB "
+                   f"(grows to the largest step, then stays) = {m['total'] / 2**20:.1f} MiB")
+
+    def memory(self) -> dict:
+        """Bytes of device memory by use: the rule is weights + cache pool + scratch, nothing else
+        (the reference's gate is resident memory <= 1.15 x weights, tests/unit/test_memory_gate.mojo:49-50)."""
+        weights, pool, scratch = self.model.weight_bytes(), self.cache.device_bytes(), self.step_fn.scratch_bytes()
+        return {"weights": weights, "cache_pool": pool, "scratch": scratch, "total": weights + pool + scratch}
 
     def generate(self, prompts: list, max_new: int = 16, temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0,
                  min_p: float = 0.0, repetition_penalty: float = 1.0, frequency_penalty: float = 0.0,

@@ -181,6 +181,13 @@ class StepFunction:
             self._scratch[key] = buf
         return buf[:n].view(shape)
 
+    def scratch_bytes(self) -> int:
+        """Bytes of the named buffers (eager steps' and the captured graphs'), retired ones included."""
+        bufs = list(self._eager_scratch.values()) + list(self._retired)
+        for b in self._graph_buffers.values():
+            bufs += list(b["scratch"].values()) + [b["dev"]]
+        return sum(t.numel() * t.element_size() for t in bufs)
+
     def identity_rotation(self, head_dim: int):
         key = head_dim
         if key not in self._identity:

@@ -17,16 +17,18 @@ from .safetensors_io import write_safetensors
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
-def random_tensors(expected: dict, seed: int, std: float = 0.02, store_dtype: str = "bfloat16") -> dict:
+def random_tensors(expected: dict, seed: int, std: float = 0.02, store_dtype: str = "bfloat16", device="cpu") -> dict:
+    """``device``: where the tensors are drawn and left (the host by default; a GPU for models whose
+    file would take minutes to write: other values than the host's for the same seed)."""
     if store_dtype not in _DTYPES:
         raise AlofaError("invalid_argument", "weights are stored as bfloat16 or float32", f"store_dtype={store_dtype}")
-    gen = torch.Generator(device="cpu")
+    gen = torch.Generator(device=device)
     gen.manual_seed(int(seed))
     out = {}
     for name, rule in expected.items():
         if rule.optional:
             continue
-        t = torch.randn(tuple(rule.shape), generator=gen, dtype=torch.float32) * std
+        t = torch.randn(tuple(rule.shape), generator=gen, dtype=torch.float32, device=device) * std
         if rule.init == "norm":
             t = t + 1.0
         elif rule.init not in ("matrix", "bias"):

@@ -1,14 +1,33 @@
-"""Decode and prefill throughput of the engine at Qwen2.5-0.5B layer sizes with
-random weights, on one MI355X.
+"""Decode and prefill throughput of the engine at the layer sizes of the
+Qwen2.5 family with random weights, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--dtype bfloat16]
+                    [--config 0.5b|7b|32b]
 
-A step is one decode step of the whole engine loop (scheduler tick, the step
-function over the paged cache, greedy choice, settle) with every request of the
-batch decoding one token. Prints one JSON line; ``value`` is decoded tokens per
-second at the default batch. Peaks are the published MI355X figures."""
+The default (0.5b) is the headline: a step is one decode step of the whole
+engine loop (scheduler tick, the step function over the paged cache, greedy
+choice, settle) with every request of the batch decoding one token; W untimed
+steps, then exactly K timed ones. One JSON line is printed; ``value`` is decoded
+tokens per second at the default batch of 8. Beside it:
+
+  prefill    one 2,048-token prompt: tokens a second, and its flops / time / peak
+  roofline   the decode step's bytes (every weight once + the live requests' cache) / time
+  points     decode at batch 1 and 64, and near the end of the context window
+  spread     median and min..max of the per-step time over interleaved repeats of every point
+             (the reference's method: src/alofa/cli.mojo:212-245, :819-850)
+  roofs      what this GPU gives in this process: a device copy of 1 GiB and a large bf16 matrix
+             product (the reference wants measured roofs, never constants:
+             src/alofa/verify/__init__.mojo:10-17); ``frac`` divides by the published peaks,
+             ``frac_measured`` by these
+  memory     device bytes of weights, cache pool and scratch
+
+``--config 7b`` and ``--config 32b`` run the larger configurations' workloads
+(a continuous batch of 64 requests with prompts of 128..2,048 tokens under
+chunked prefill; 8 prompts of 16,384 tokens and decoding at batch 32 with a
+context of 4,096) through the same engine and print their own line."""
 import argparse
 import json
+import statistics
 import sys
 import tempfile
 import time
@@ -20,14 +39,25 @@ sys.path.insert(0, str(ROOT))
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-# Qwen2.5-0.5B layer sizes (the benchmark configuration)
-QWEN25_05B = {
-    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": 24, "hidden_size": 896,
-    "num_attention_heads": 14, "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936,
-    "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "use_sliding_window": False,
-    "max_position_embeddings": 32768,
+
+def family(layers, hidden, heads, kv_heads, inter, vocab, tied, max_pos=32768):
+    return {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "num_hidden_layers": layers, "hidden_size": hidden,
+            "num_attention_heads": heads, "num_key_value_heads": kv_heads, "intermediate_size": inter, "vocab_size": vocab,
+            "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": tied, "use_sliding_window": False,
+            "max_position_embeddings": max_pos}
+
+
+CONFIGS = {
+    "0.5b": family(24, 896, 14, 2, 4864, 151936, True),
+    "7b": family(28, 3584, 28, 4, 18944, 152064, False),
+    "32b": family(64, 5120, 40, 8, 27648, 152064, False, 40960),
 }
+QWEN25_05B = CONFIGS["0.5b"]
 CONTEXT, PROMPT, BLOCK = 4096, 512, 16
+
+
+def say(text):
+    print(f"[bench] {text}", file=sys.stderr, flush=True)
 
 
 def linear_params_per_layer(c):
@@ -47,10 +77,12 @@ def decode_bytes(c, ctx_lens, dtype_bytes=2):
     return weights + cache
 
 
-def prefill_flops(c, T, wanted=1):
+def prefill_flops(c, T, wanted=1, start=0):
+    """Flops of running T tokens of one request that stand at positions start..start+T-1."""
     h, d, L = c["hidden_size"], c["hidden_size"] // c["num_attention_heads"], c["num_hidden_layers"]
     linear = 2 * T * linear_params_per_layer(c) * L
-    attention = L * 2 * d * c["num_attention_heads"] * T * (T + 1)   # QK^T and PV over the causal half
+    keys = T * start + T * (T + 1) // 2                               # (query, key) pairs under the causal bound
+    attention = L * 4 * d * c["num_attention_heads"] * keys           # QK^T and PV
     return linear + attention + 2 * wanted * h * c["vocab_size"]
 
 
@@ -59,57 +91,345 @@ def sync():
     torch.cuda.synchronize()
 
 
-def measure_decode(model_dir, cfg, dtype, batch, steps, warmup, seed=0, prompt=None):
-    import numpy as np
-    from alofa_amd import Engine
-    rng = np.random.default_rng(seed)
-    per_req = (CONTEXT + BLOCK - 1) // BLOCK
-    eng = Engine(model_dir, dtype=dtype, max_tokens=CONTEXT, max_batch=batch, kv_blocks=per_req * batch + 64,
-                 block_size=BLOCK, token_budget=max(2048, batch), max_chunk=512, watermark_permille=1000)
-    core = eng.core
-    prompt = PROMPT if prompt is None else prompt
-    for r in range(batch):
-        core.submit(r + 1, [int(t) for t in rng.integers(0, cfg["vocab_size"], prompt)], CONTEXT - prompt)
-    while not (core.last_action and len(core.last_action.decode) == batch and not core.last_action.prefill):
-        core.tick()
-    for _ in range(warmup):
-        core.tick()
-    sync()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        rows = core.tick()
-        assert rows == batch, f"a timed step ran {rows} rows, not {batch}"
-    sync()
-    dt = time.perf_counter() - t0
-    ctx_lens = [eng.cache.length(r + 1) for r in range(batch)]
-    for r in range(batch):
-        core.cancel(r + 1)
-    core.tick()
-    del eng
+# ------------------------------------------------------------------ measured roofs
+
+def measure_roofs():
+    """What the GPU gives in this process: GB/s of a device-to-device copy of 1 GiB of bfloat16
+    (bytes read + bytes written over time) and TFLOP/s of a large bfloat16 matrix product (the
+    vendor library's: a yardstick, not part of the engine)."""
     import torch
-    torch.cuda.empty_cache()
-    return dt / steps, ctx_lens
-
-
-def measure_prefill(model_dir, cfg, dtype, T=2048, reps=3, seed=1):
-    import numpy as np
-    from alofa_amd.replay import Replayer
-    rng = np.random.default_rng(seed)
-    r = Replayer(model_dir, dtype, max_tokens=CONTEXT, block_size=BLOCK)
-    best = None
-    for i in range(reps + 1):
-        ids = [int(t) for t in rng.integers(0, cfg["vocab_size"], T)]
-        from alofa_amd.engine.step import StepEntry
-        r.cache.admit(i)
+    n = 1 << 29                                              # 2**29 bfloat16 = 1 GiB
+    src = torch.empty(n, dtype=torch.bfloat16, device="cuda").normal_()
+    dst = torch.empty_like(src)
+    a = torch.randn(8192, 8192, dtype=torch.bfloat16, device="cuda")
+    b = torch.randn(8192, 8192, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty(8192, 8192, dtype=torch.bfloat16, device="cuda")
+    copy_s, gemm_s = [], []
+    for i in range(6):
         sync()
         t0 = time.perf_counter()
-        r.fn.run([StepEntry(i, ids, [T - 1])])
+        for _ in range(4):
+            dst.copy_(src)
+        sync()
+        t1 = time.perf_counter()
+        for _ in range(4):
+            torch.matmul(a, b, out=out)
+        sync()
+        t2 = time.perf_counter()
+        if i:                                                # the first round warms up
+            copy_s.append((t1 - t0) / 4)
+            gemm_s.append((t2 - t1) / 4)
+    del src, dst, a, b, out
+    torch.cuda.empty_cache()
+    return {"hbm_copy_gbs": round(2 * n * 2 / min(copy_s) / 1e9, 1), "gemm_bf16_tflops": round(2 * 8192 ** 3 / min(gemm_s) / 1e12, 1),
+            "how": "best of 5 rounds: copy of 1 GiB bf16 (read + write), 8192^3 bf16 product of the vendor library"}
+
+
+# ------------------------------------------------------------------------ points
+
+class DecodePoint:
+    """Requests of one batch size kept decoding; ``run(n)`` times n more steps."""
+
+    def __init__(self, model, cfg, dtype, batch, prompt, seed=0, context=CONTEXT):
+        import numpy as np
+        from alofa_amd import Engine
+        rng = np.random.default_rng(seed)
+        per_req = (context + BLOCK - 1) // BLOCK
+        self.batch, self.cfg = batch, cfg
+        self.eng = Engine(None, dtype=dtype, max_tokens=context, max_batch=batch, kv_blocks=per_req * batch + 64, block_size=BLOCK,
+                          token_budget=max(2048, batch), max_chunk=512, watermark_permille=1000, model=model)
+        core = self.eng.core
+        for r in range(batch):
+            core.submit(r + 1, [int(t) for t in rng.integers(0, cfg["vocab_size"], prompt)], context - prompt)
+        while not (core.last_action and len(core.last_action.decode) == batch and not core.last_action.prefill):
+            core.tick()
+
+    def run(self, steps):
+        """Seconds per step over ``steps`` decode steps, bracketed by synchronisation."""
+        core = self.eng.core
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            rows = core.tick()
+            assert rows == self.batch, f"a timed step ran {rows} rows, not {self.batch}"
+        sync()
+        return (time.perf_counter() - t0) / steps
+
+    def context_lengths(self):
+        return [self.eng.cache.length(r + 1) for r in range(self.batch)]
+
+    def close(self):
+        import torch
+        for r in range(self.batch):
+            self.eng.core.cancel(r + 1)
+        self.eng.core.tick()
+        self.eng = None
+        torch.cuda.empty_cache()
+
+
+class PrefillPoint:
+    """One prompt of T tokens run whole in one step; ``run()`` times it on fresh pages."""
+
+    def __init__(self, model, cfg, dtype, T=2048, seed=1):
+        import numpy as np
+        from alofa_amd.cache.manager import CacheManager
+        from alofa_amd.engine.step import StepFunction
+        self.T, self.cfg, self.rng = T, cfg, np.random.default_rng(seed)
+        m = model[1]
+        self.cache = CacheManager(m.cache_needs(), m.state_needs(), (T + BLOCK - 1) // BLOCK + 4, BLOCK, max_requests=4,
+                                  device=m.rt.device, dtype=m.rt.dtype)
+        self.fn = StepFunction(m, self.cache, n_positions=max(T, 64))
+        self.n = 0
+
+    def run(self):
+        from alofa_amd.engine.step import StepEntry
+        ids = [int(t) for t in self.rng.integers(0, self.cfg["vocab_size"], self.T)]
+        self.n += 1
+        self.cache.admit(self.n)
+        sync()
+        t0 = time.perf_counter()
+        self.fn.run([StepEntry(self.n, ids, [self.T - 1])])
         sync()
         dt = time.perf_counter() - t0
-        r.cache.free(i)
-        if i > 0:
-            best = dt if best is None else min(best, dt)
-    return best
+        self.cache.free(self.n)
+        return dt
+
+
+def spread(samples):
+    return {"median_ms": round(statistics.median(samples) * 1e3, 4), "min_ms": round(min(samples) * 1e3, 4),
+            "max_ms": round(max(samples) * 1e3, 4), "repeats": len(samples)}
+
+
+def device_model(cfg, dtype, seed):
+    """(config, model) with random weights drawn on the device: for sizes whose file would take minutes to write."""
+    import torch
+    from alofa_amd.config import config_from_dict
+    from alofa_amd.model import Model, expected_tensors, runtime
+    from alofa_amd.weights import random_tensors
+    config = config_from_dict(cfg)
+    spec = config.spec()
+    rt = runtime(dtype)
+    weights = random_tensors(expected_tensors(spec), seed, device=rt.device)
+    model = Model(spec, weights, rt)
+    del weights
+    torch.cuda.empty_cache()
+    return config, model
+
+
+# ------------------------------------------------------------------- the headline
+
+def headline(args):
+    from alofa_amd.model import load_model
+    from alofa_amd.weights import write_random_model
+    cfg = dict(QWEN25_05B, num_hidden_layers=args.layers)
+    dbytes = 2 if args.dtype == "bfloat16" else 4
+    with tempfile.TemporaryDirectory() as d:
+        write_random_model(cfg, d, seed=20260918)
+        model = load_model(d, args.dtype)
+    if args.only_prefill:
+        p = PrefillPoint(model, cfg, args.dtype)
+        p.run()
+        pt = min(p.run() for _ in range(3))
+        print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
+                                      "frac": round(prefill_flops(cfg, 2048) / pt / PEAK_FLOPS[args.dtype], 4)}}))
+        return 0
+    if not 1 <= args.prompt <= CONTEXT - 8 * (args.steps + args.warmup) - 1:
+        print(f"--prompt must leave room for the decode steps within the context of {CONTEXT}")
+        return 2
+    roofs = None if args.no_points else measure_roofs()
+    main_point = DecodePoint(model, cfg, args.dtype, args.batch, args.prompt)
+    memory = main_point.eng.memory()
+    say(f"device memory: weights {memory['weights'] / 2**20:.1f} MiB + cache pool {memory['cache_pool'] / 2**20:.1f} MiB (batch {args.batch} x {CONTEXT} tokens)"
+        f" + scratch {memory['scratch'] / 2**20:.1f} MiB")
+    main_point.run(args.warmup) if args.warmup else None
+    ms = main_point.run(args.steps)                                    # exactly K timed steps after W untimed ones
+    ctx_lens = main_point.context_lengths()
+    memory = main_point.eng.memory()
+    value = args.batch / ms
+    achieved = decode_bytes(cfg, ctx_lens, dbytes) / ms / 1e9
+    out = {
+        "metric": "decode tok/s @ batch 8 (Qwen2.5-0.5B sizes); prefill tok/s @ 2,048 tok; decode @ batch 1/64 under points",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0, 0.02), uniform random token ids)",
+        "config": {"model": "Qwen2.5-0.5B sizes, random weights", "layers": args.layers, "layers_full": QWEN25_05B["num_hidden_layers"],
+                   "hidden": 896, "heads": 14, "kv_heads": 2, "head_dim": 64, "intermediate": 4864, "vocab": 151936,
+                   "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": args.prompt, "decode_context": int(sum(ctx_lens) / len(ctx_lens)),
+                   "kv_block": BLOCK, "tied_embeddings": True, "parallelism": "single GPU"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "memory": {k: int(v) for k, v in memory.items()},
+    }
+    if not args.no_points:
+        T = 2048
+        reps, n = 5, max(8, args.steps // 2)
+        others = {1: DecodePoint(model, cfg, args.dtype, 1, PROMPT), 64: DecodePoint(model, cfg, args.dtype, 64, PROMPT)}
+        prefill = PrefillPoint(model, cfg, args.dtype, T)
+        points = {args.batch: main_point, **{b: p for b, p in others.items() if b != args.batch}}
+        for p in others.values():
+            p.run(max(4, args.warmup // 2))
+        prefill.run()
+        samples = {f"decode_b{b}": [] for b in points}
+        samples["prefill"] = []
+        for _ in range(reps):                                           # interleaved: every point once per round
+            for b, p in points.items():
+                samples[f"decode_b{b}"].append(p.run(n))
+            samples["prefill"].append(prefill.run())
+        pt = statistics.median(samples["prefill"])
+        out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
+                          "frac": round(prefill_flops(cfg, T) / pt / PEAK_FLOPS[args.dtype], 4)}
+        out["points"] = {f"decode_b{b}": round(b / statistics.median(samples[f"decode_b{b}"]), 1) for b in (1, 64)}
+        out["spread"] = {k: spread(v) for k, v in samples.items()}
+        for p in others.values():
+            p.close()
+        main_point.close()
+        # the same near the end of the context window (prompts of 3,840 tokens)
+        for b in (8, 64):
+            p = DecodePoint(model, cfg, args.dtype, b, CONTEXT - 256)
+            p.run(max(4, args.warmup // 4))
+            out["points"][f"decode_b{b}_ctx{CONTEXT - 256}"] = round(b / p.run(max(16, args.steps // 4)), 1)
+            p.close()
+        out["roofs"] = roofs
+        out["roofline"]["frac_measured"] = round(achieved / roofs["hbm_copy_gbs"], 4)
+        if args.dtype == "bfloat16":
+            out["prefill"]["frac_measured"] = round(prefill_flops(cfg, T) / pt / (roofs["gemm_bf16_tflops"] * 1e12), 4)
+    print(json.dumps(out))
+    return 0
+
+
+# --------------------------------------------------------- the larger configurations
+
+def flat_config(name, cfg, layers, **more):
+    d = cfg["hidden_size"] // cfg["num_attention_heads"]
+    return {"model": f"Qwen2.5-{name.upper()} sizes, random weights", "layers": layers, "layers_full": CONFIGS[name]["num_hidden_layers"],
+            "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"], "head_dim": d,
+            "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"], "kv_block": BLOCK,
+            "tied_embeddings": cfg["tie_word_embeddings"], "parallelism": "single GPU", **more}
+
+
+def continuous_batch(args):
+    """64 requests with prompts of uniform random length in [128, 2048] and 256 generated tokens
+    each, all submitted at once, under chunked prefill with chunks of 512 (a budget of 2,048
+    tokens a tick): the whole run through the engine loop, timed from the first tick to the last."""
+    import numpy as np
+    from alofa_amd import Engine
+    name = "7b"
+    layers = args.layers or CONFIGS[name]["num_hidden_layers"]
+    cfg = dict(CONFIGS[name], num_hidden_layers=layers)
+    say(f"drawing {name} weights on the device ({layers} layers)")
+    model = device_model(cfg, args.dtype, 20260918)
+    n_req, new, context = 64, 256, 8192
+    rng = np.random.default_rng(7)
+    lens = [int(n) for n in rng.integers(128, 2049, n_req)]
+    per_req = (max(lens) + new + BLOCK - 1) // BLOCK
+    eng = Engine(None, dtype=args.dtype, max_tokens=context, max_batch=n_req, kv_blocks=per_req * n_req + 64, block_size=BLOCK,
+                 token_budget=2048, max_chunk=512, watermark_permille=1000, model=model, report=say)
+    core = eng.core
+
+    def run():
+        base = (core.ticks + 1) * 1000
+        for r, n in enumerate(lens):
+            core.submit(base + r, [int(t) for t in rng.integers(0, cfg["vocab_size"], n)], new)
+        ticks, decode_s, decode_steps, decode_ctx = 0, 0.0, 0, []
+        sync()
+        t0 = time.perf_counter()
+        while core.has_work():
+            t1 = time.perf_counter()
+            core.tick()
+            act = core.last_action
+            if len(act.decode) == n_req and not act.prefill:
+                sync()
+                decode_s += time.perf_counter() - t1
+                decode_steps += 1
+            ticks += 1
+        sync()
+        dt = time.perf_counter() - t0
+        for r in range(n_req):
+            assert len(core.output(base + r)) == new
+            core.release(base + r)
+        return dt, ticks, decode_s, decode_steps
+    say("warm-up run")
+    run()
+    dt, ticks, decode_s, decode_steps = run()
+    dbytes = 2 if args.dtype == "bfloat16" else 4
+    mean_ctx = [n + new // 2 for n in lens]
+    step_ms = decode_s / max(1, decode_steps) * 1e3
+    out = {"metric": "generated tok/s, continuous batch of 64 requests (prompts U[128,2048], 256 new tokens, chunked prefill 512), Qwen2.5-7B sizes",
+           "value": round(n_req * new / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": ticks, "warmup": ticks, "ms_per_step": round(dt / ticks * 1e3, 4),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic (random weights N(0, 0.02) drawn on the device, uniform random token ids)",
+           "config": flat_config(name, cfg, layers, global_batch=n_req, seq_len=context, prompt_tokens=sum(lens), new_tokens=new, max_chunk=512, token_budget=2048),
+           "total_tok_s": round((sum(lens) + n_req * new) / dt, 1), "seconds": round(dt, 3),
+           "roofline": {"bound": "hbm", "what": "the ticks in which all 64 requests decode and nothing is prefilled", "steps": decode_steps, "ms_per_step": round(step_ms, 4),
+                        "achieved": round(decode_bytes(cfg, mean_ctx, dbytes) / (step_ms / 1e3) / 1e9, 1) if decode_steps else None, "peak": PEAK_HBM_GBS, "unit": "GB/s"},
+           "memory": {k: int(v) for k, v in eng.memory().items()}}
+    if out["roofline"]["achieved"]:
+        out["roofline"]["frac"] = round(out["roofline"]["achieved"] / PEAK_HBM_GBS, 4)
+    print(json.dumps(out))
+    return 0
+
+
+def long_prompts(args):
+    """8 requests, each with a prompt of 16,384 tokens and 128 generated tokens (chunked prefill,
+    chunks of 2,048 under a budget of 4,096 tokens a tick), then decoding at batch 32 with a
+    context of 4,096 tokens, which reads the most cache per step."""
+    import numpy as np
+    from alofa_amd import Engine
+    name = "32b"
+    layers = args.layers or CONFIGS[name]["num_hidden_layers"]
+    cfg = dict(CONFIGS[name], num_hidden_layers=layers)
+    say(f"drawing {name} weights on the device ({layers} layers)")
+    model = device_model(cfg, args.dtype, 20260918)
+    dbytes = 2 if args.dtype == "bfloat16" else 4
+    n_req, plen, new, context = 8, 16384, 128, 32768
+    rng = np.random.default_rng(8)
+    per_req = (plen + new + BLOCK - 1) // BLOCK
+    eng = Engine(None, dtype=args.dtype, max_tokens=context, max_batch=n_req, kv_blocks=per_req * n_req + 64, block_size=BLOCK,
+                 token_budget=4096, max_chunk=2048, watermark_permille=1000, model=model, report=say)
+    core = eng.core
+    for r in range(n_req):
+        core.submit(r + 1, [int(t) for t in rng.integers(0, cfg["vocab_size"], plen)], new)
+    sync()
+    t0 = time.perf_counter()
+    prefill_s, prefill_tokens, prefill_fl, ticks = 0.0, 0, 0.0, 0
+    while core.has_work():
+        t1 = time.perf_counter()
+        core.tick()
+        act = core.last_action
+        if act.prefill and not act.decode:
+            sync()
+            prefill_s += time.perf_counter() - t1
+            prefill_tokens += sum(e - s for _, s, e in act.prefill)
+            prefill_fl += sum(prefill_flops(cfg, e - s, wanted=int(e == plen), start=s) for _, s, e in act.prefill)
+        ticks += 1
+        if ticks % 16 == 0:
+            say(f"tick {ticks}: {prefill_tokens} prompt tokens so far")
+    sync()
+    dt = time.perf_counter() - t0
+    memory = eng.memory()
+    for r in range(n_req):
+        assert len(core.output(r + 1)) == new
+        core.release(r + 1)
+    del eng, core
+    out = {"metric": "prefill tok/s over 8 prompts of 16,384 tokens (chunks of 2,048); decode tok/s @ batch 32, context 4,096 under points; Qwen2.5-32B sizes",
+           "value": round(prefill_tokens / prefill_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": ticks, "warmup": 0, "ms_per_step": round(dt / ticks * 1e3, 3),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic (random weights N(0, 0.02) drawn on the device, uniform random token ids)",
+           "config": flat_config(name, cfg, layers, global_batch=n_req, seq_len=context, prompt_len=plen, new_tokens=new, max_chunk=2048, token_budget=4096),
+           "prefill": {"value": round(prefill_tokens / prefill_s, 1), "tokens": prefill_tokens, "ms": round(prefill_s * 1e3, 1),
+                       "frac": round(prefill_fl / prefill_s / PEAK_FLOPS[args.dtype], 4)},
+           "seconds_whole_run": round(dt, 2), "generated_tok_s_whole_run": round(n_req * new / dt, 1), "memory": {k: int(v) for k, v in memory.items()}}
+    p = DecodePoint(model, cfg, args.dtype, 32, 4096 - 64, context=4096 + 64)
+    p.run(8)
+    ms = p.run(24)
+    ctx_lens = p.context_lengths()
+    achieved = decode_bytes(cfg, ctx_lens, dbytes) / ms / 1e9
+    out["points"] = {"decode_b32_ctx4096": round(32 / ms, 1)}
+    out["roofline"] = {"bound": "hbm", "what": "decode step at batch 32, context about 4,096", "ms_per_step": round(ms * 1e3, 4), "achieved": round(achieved, 1),
+                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    p.close()
+    print(json.dumps(out))
+    return 0
 
 
 def main():
@@ -118,10 +438,11 @@ def main():
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--config", default="0.5b", choices=sorted(CONFIGS), help="layer sizes and workload (default: the headline)")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="prompt length of the timed decode steps' requests (context = prompt + steps so far)")
-    ap.add_argument("--layers", type=int, default=QWEN25_05B["num_hidden_layers"], help="fewer layers than the configuration has, where memory or time needs it")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has, where memory or time needs it")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points, the prefill, the repeats and the roofs")
     ap.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its line")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -130,50 +451,12 @@ def main():
 
     from alofa_amd.csrc.build import load
     load()
-    from alofa_amd.weights import write_random_model
-    cfg = dict(QWEN25_05B, num_hidden_layers=args.layers)
-    with tempfile.TemporaryDirectory() as d:
-        write_random_model(cfg, d, seed=20260918)
-        if args.only_prefill:
-            pt = measure_prefill(d, cfg, args.dtype, 2048)
-            print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
-                                          "frac": round(prefill_flops(cfg, 2048) / pt / PEAK_FLOPS[args.dtype], 4)}}))
-            return 0
-        if not 1 <= args.prompt <= CONTEXT - args.steps - args.warmup - 1:
-            print(f"--prompt must leave room for the decode steps within the context of {CONTEXT}")
-            return 2
-        ms, ctx_lens = measure_decode(d, cfg, args.dtype, args.batch, args.steps, args.warmup, prompt=args.prompt)
-        value = args.batch / ms
-        dbytes = 2 if args.dtype == "bfloat16" else 4
-        achieved = decode_bytes(cfg, ctx_lens, dbytes) / ms / 1e9
-        out = {
-            "metric": "decode tok/s @ batch 8 (Qwen2.5-0.5B sizes); prefill tok/s @ 2,048 tok; decode @ batch 1/64 under points",
-            "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": round(ms * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0, 0.02), uniform random token ids)",
-            "config": {"model": "Qwen2.5-0.5B sizes, random weights", "layers": args.layers, "layers_full": QWEN25_05B["num_hidden_layers"],
-                       "hidden": 896, "heads": 14, "kv_heads": 2, "head_dim": 64, "intermediate": 4864, "vocab": 151936,
-                       "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": args.prompt, "decode_context": int(sum(ctx_lens) / len(ctx_lens)),
-                       "kv_block": BLOCK, "tied_embeddings": True, "parallelism": "single GPU"},
-            "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(achieved / PEAK_HBM_GBS, 4)},
-        }
-        if not args.no_points:
-            T = 2048
-            pt = measure_prefill(d, cfg, args.dtype, T)
-            out["prefill"] = {"value": round(T / pt, 1), "tokens": T, "ms": round(pt * 1e3, 3),
-                              "frac": round(prefill_flops(cfg, T) / pt / PEAK_FLOPS[args.dtype], 4)}
-            points = {}
-            for b in (1, 64):
-                pms, _ = measure_decode(d, cfg, args.dtype, b, max(16, args.steps // 2), max(4, args.warmup // 2))
-                points[f"decode_b{b}"] = round(b / pms, 1)
-            # the same near the end of the context window (prompts of 3,840 tokens)
-            for b in (8, 64):
-                pms, _ = measure_decode(d, cfg, args.dtype, b, max(16, args.steps // 4), max(4, args.warmup // 4), prompt=CONTEXT - 256)
-                points[f"decode_b{b}_ctx{CONTEXT - 256}"] = round(b / pms, 1)
-            out["points"] = points
-    print(json.dumps(out))
-    return 0
+    if args.config == "7b":
+        return continuous_batch(args)
+    if args.config == "32b":
+        return long_prompts(args)
+    args.layers = args.layers or QWEN25_05B["num_hidden_layers"]
+    return headline(args)
 
 
 if __name__ == "__main__":
