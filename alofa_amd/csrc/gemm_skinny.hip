@@ -18,6 +18,12 @@
 // memory (common.h): a block's partial tiles are in memory once its stores have
 // been acknowledged, which every wave waits for before the block is counted.
 //
+// With kNorm the rows of A are the float residual stream and the kernel applies an RMSNorm on the
+// way: a fragment is x * w_norm rounded to bfloat16, the sum of squares of every row is gathered
+// beside the products (each block reads all of A anyway), and the row's factor 1 / sqrt(mean + eps)
+// multiplies the finished sum in the epilogue. Nothing waits for the factor, so the norm costs no
+// trip through memory of its own; a launch of its own it would cost as much as a small product.
+//
 // Operand layout of v_mfma_f32_16x16x32_bf16, lane l: A holds row l % 16,
 // B holds column l % 16, both the 8 reduction indices 8 * (l / 16) .. + 7 of
 // the step; D holds column l % 16, rows 4 * (l / 16) .. + 3.
@@ -45,28 +51,51 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* __restrict__ p, bool o
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// eight values of a row of A as they come from memory: bfloat16, or float with the norm's weights beside them
+struct RawNormed {
+  float4 lo, hi;
+};
+__device__ __forceinline__ void load_raw(RawNormed& dst, const void* row, int k, bool ok) {
+  dst.lo = dst.hi = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (ok) {
+    const float* p = static_cast<const float*>(row) + k;
+    dst.lo = *reinterpret_cast<const float4*>(p);
+    dst.hi = *reinterpret_cast<const float4*>(p + 4);
+  }
+}
+// x * w rounded to bfloat16; the squares of x join the row's sum
+__device__ __forceinline__ bf16x8 to_frag(const RawNormed& x, const RawNormed& w, float& ss) {
+  ss += x.lo.x * x.lo.x + x.lo.y * x.lo.y + x.lo.z * x.lo.z + x.lo.w * x.lo.w;
+  ss += x.hi.x * x.hi.x + x.hi.y * x.hi.y + x.hi.z * x.hi.z + x.hi.w * x.hi.w;
+  const uint4 v = make_uint4(pack_bf16x2(x.lo.x * w.lo.x, x.lo.y * w.lo.y), pack_bf16x2(x.lo.z * w.lo.z, x.lo.w * w.lo.w),
+                             pack_bf16x2(x.hi.x * w.hi.x, x.hi.y * w.hi.y), pack_bf16x2(x.hi.z * w.hi.z, x.hi.w * w.hi.w));
+  return __builtin_bit_cast(bf16x8, v);
+}
+
 // MT: 16-row tiles of A; NT: 16-column tiles per block (kSkSwiglu: tile 0 is the
 // gate matrix, tile 1 the up matrix, same columns); TO: float or bf16_t.
 // kUnroll: steps of 32 along K whose loads are in flight together (twice that with the prefetch).
-template <int MT, int NT, int kWaves, int kEpilogue, typename TO, int kUnroll>
+// kNorm: A is float [M, K] and out = epilogue(rmsnorm(A, norm_w, eps) W^T) (no split of K over blocks then).
+template <int MT, int NT, int kWaves, int kEpilogue, typename TO, int kUnroll, bool kNorm>
 __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
-    TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
+    TO* __restrict__ out, int64_t ldo, const void* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
     const bf16_t* __restrict__ W2, int64_t ldw, const float* __restrict__ bias, int M, int N, int K,
-    f32x4* __restrict__ ws, int* __restrict__ counters) {
+    f32x4* __restrict__ ws, int* __restrict__ counters, const float* __restrict__ norm_w, float eps) {
   __shared__ f32x4 red[kWaves][MT * NT][64];
+  __shared__ float ssq[kNorm ? kWaves : 1][MT][16];
   __shared__ int last_block;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int r = lane % 16, g = lane / 16;
   constexpr int kColsPerBlock = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
   const int n0 = blockIdx.x * kColsPerBlock;
 
-  const bf16_t* a_row[MT];
+  const void* a_row[MT];
   bool a_ok[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + r;
     a_ok[mt] = m < M;
-    a_row[mt] = A + static_cast<int64_t>(a_ok[mt] ? m : 0) * lda;
+    a_row[mt] = static_cast<const char*>(A) + static_cast<int64_t>(a_ok[mt] ? m : 0) * lda * (kNorm ? 4 : 2);
   }
   const bf16_t* w_row[NT];
   bool w_ok[NT];
@@ -110,36 +139,83 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   const int per_split = (all_steps + k_splits - 1) / k_splits;
   const int first_step = blockIdx.y * per_split;
   const int n_steps = (first_step + per_split < all_steps) ? first_step + per_split : all_steps;
-  bf16x8 a_cur[kUnroll][MT], w_cur[kUnroll][NT], a_nxt[kUnroll][MT], w_nxt[kUnroll][NT];
+  float ss[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) ss[mt] = 0.f;
+  if constexpr (!kNorm) {
+    bf16x8 a_cur[kUnroll][MT], w_cur[kUnroll][NT], a_nxt[kUnroll][MT], w_nxt[kUnroll][NT];
 
-  auto load = [&](bf16x8 (&a)[kUnroll][MT], bf16x8 (&w)[kUnroll][NT], int first) {
+    auto load = [&](bf16x8 (&a)[kUnroll][MT], bf16x8 (&w)[kUnroll][NT], int first) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-      const int k = (first + u * kWaves) * 32 + g * 8;
-      const bool k_ok = k < K && first + u * kWaves < n_steps;
+      for (int u = 0; u < kUnroll; ++u) {
+        const int k = (first + u * kWaves) * 32 + g * 8;
+        const bool k_ok = k < K && first + u * kWaves < n_steps;
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) w[u][nt] = load_frag(w_row[nt] + k, k_ok && w_ok[nt]);
+        for (int nt = 0; nt < NT; ++nt) w[u][nt] = load_frag(w_row[nt] + k, k_ok && w_ok[nt]);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) a[u][mt] = load_frag(a_row[mt] + k, k_ok && a_ok[mt]);
+        for (int mt = 0; mt < MT; ++mt) a[u][mt] = load_frag(static_cast<const bf16_t*>(a_row[mt]) + k, k_ok && a_ok[mt]);
+      }
+    };
+
+    load(a_cur, w_cur, first_step + wave);
+    for (int s = first_step + wave; s < n_steps; s += kUnroll * kWaves) {
+      if (s + kUnroll * kWaves < n_steps) load(a_nxt, w_nxt, s + kUnroll * kWaves);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[u][mt], w_cur[u][nt], acc[mt][nt], 0, 0, 0);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) a_cur[u][mt] = a_nxt[u][mt];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) w_cur[u][nt] = w_nxt[u][nt];
+      }
     }
-  };
-
-  load(a_cur, w_cur, first_step + wave);
-  for (int s = first_step + wave; s < n_steps; s += kUnroll * kWaves) {
-    if (s + kUnroll * kWaves < n_steps) load(a_nxt, w_nxt, s + kUnroll * kWaves);
+  } else {
+    // Two sets of operands, each refilled as soon as its steps are done (no copies between sets: a copy
+    // would wait for its load). Everything the first steps need sets out before anything is waited for:
+    // both sets' weights and rows, then the norm's weights, which all waves share through LDS.
+    static_assert(!kNorm || MT == 1, "the norm rides on products of at most 16 rows");
+    extern __shared__ __attribute__((aligned(16))) float norm_lds[];      // K floats
+    RawNormed ra0[kUnroll], ra1[kUnroll];
+    bf16x8 w0[kUnroll][NT], w1[kUnroll][NT];
+    auto issue = [&](RawNormed (&ra)[kUnroll], bf16x8 (&w)[kUnroll][NT], int first) {
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+      for (int u = 0; u < kUnroll; ++u) {
+        const int k = (first + u * kWaves) * 32 + g * 8;
+        const bool k_ok = k < K && first + u * kWaves < n_steps;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+        for (int nt = 0; nt < NT; ++nt) w[u][nt] = load_frag(w_row[nt] + k, k_ok && w_ok[nt]);
+        load_raw(ra[u], a_row[0], k, k_ok && a_ok[0]);
+      }
+    };
+    auto multiply = [&](RawNormed (&ra)[kUnroll], bf16x8 (&w)[kUnroll][NT], int first) {
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[u][mt], w_cur[u][nt], acc[mt][nt], 0, 0, 0);
+      for (int u = 0; u < kUnroll; ++u) {
+        int k = (first + u * kWaves) * 32 + g * 8;
+        k = k < K ? k : 0;                   // (a step past the end holds zeros: any weights will do)
+        const RawNormed nw{*reinterpret_cast<const float4*>(norm_lds + k), *reinterpret_cast<const float4*>(norm_lds + k + 4)};
+        const bf16x8 a = to_frag(ra[u], nw, ss[0]);
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) a_cur[u][mt] = a_nxt[u][mt];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) w_cur[u][nt] = w_nxt[u][nt];
+        for (int nt = 0; nt < NT; ++nt) acc[0][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w[u][nt], acc[0][nt], 0, 0, 0);
+      }
+    };
+    constexpr int kStride = kUnroll * kWaves;
+    int s = first_step + wave;
+    issue(ra0, w0, s);
+    issue(ra1, w1, s + kStride);
+    for (int i = threadIdx.x * 4; i < K; i += kWaves * 64 * 4)
+      *reinterpret_cast<float4*>(norm_lds + i) = *reinterpret_cast<const float4*>(norm_w + i);
+    __syncthreads();
+    for (; s < n_steps; s += 2 * kStride) {
+      multiply(ra0, w0, s);
+      issue(ra0, w0, s + 2 * kStride);
+      multiply(ra1, w1, s + kStride);
+      issue(ra1, w1, s + 3 * kStride);
     }
   }
 
@@ -147,6 +223,14 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) red[wave][mt * NT + nt][lane] = acc[mt][nt];
+  if constexpr (kNorm) {
+    // the four lanes that hold slices of one row meet; the waves' shares of a row are added in wave order below
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const float row_ss = rows_sum(ss[mt]);
+      if (g == 0) ssq[wave][mt][r] = row_ss;
+    }
+  }
   __syncthreads();
 
   if (k_splits > 1) {
@@ -198,6 +282,20 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     }
     const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
     if (n >= N) continue;
+    if constexpr (kNorm) {
+      // rows 4 g .. 4 g + 3 of the tile: their factors 1 / sqrt(mean of squares + eps)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float total = ssq[0][mt][g * 4 + i];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) total += ssq[w][mt][g * 4 + i];
+        // (the hardware's reciprocal square root, good to one unit in the last place: an exact root and an exact
+        // division are some hundred dependent instructions in a kernel that lasts a few microseconds)
+        const float factor = __builtin_amdgcn_rsqf(total / static_cast<float>(K) + eps);
+        sum[i] *= factor;
+        up[i] *= factor;
+      }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = mt * 16 + g * 4 + i;
@@ -215,15 +313,42 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   }
 }
 
+constexpr int kMaxNormK = 8192;    // columns of a product that takes a norm (the norm's weights lie in LDS)
+
+struct NormArgs {
+  const float* weight;   // null: A is bfloat16 and no norm is applied
+  float eps;
+};
+
+// Parts of K that the blocks of a column tile share out (1: no hand-over through the workspace).
+template <int MT, int NT, int kWaves, int kEpilogue>
+static int skinny_splits(int N, int K) {
+  constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
+  const int col_tiles = (N + cols - 1) / cols;
+  int k_splits = 1;
+  const Workspace& g_ws = workspace();
+  if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr) {
+    const int steps = (K + 31) / 32;
+    const int min_steps = (MT == 1) ? 2 * kWaves : kWaves;
+    while (k_splits < 8 && col_tiles * k_splits * 2 <= 512 && steps / (k_splits * 2) >= min_steps) k_splits *= 2;
+    if (col_tiles > kGemmCounters || static_cast<int64_t>(col_tiles) * k_splits * MT * NT * 256 > g_ws.tile_floats) k_splits = 1;
+  }
+  return k_splits;
+}
+
 template <int MT, int NT, int kWaves, int kEpilogue, typename TO>
 static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
-                         const float* bias, int M, int N, int K, hipStream_t stream) {
+                         const float* bias, int M, int N, int K, NormArgs norm, hipStream_t stream, int* splits_only) {
   constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
   const int col_tiles = (N + cols - 1) / cols;
   // split K across blocks while the column tiles alone leave most of the chip idle
   int k_splits = 1;
   const Workspace& g_ws = workspace();
-  if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr) {
+  if (splits_only) {
+    *splits_only = skinny_splits<MT, NT, kWaves, kEpilogue>(N, K);
+    return 0;
+  }
+  if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr && norm.weight == nullptr) {
     const int steps = (K + 31) / 32;
     // (a split costs a trip through memory: only while every wave keeps at least two steps of its own, four
     // with one tile of rows, whose steps are light)
@@ -233,23 +358,34 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
   }
   // loads in flight: many for one row tile (latency is all there is), fewer as row tiles take the registers
   constexpr int unroll = (MT >= 4) ? 2 : 4;
-  gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, unroll><<<dim3(col_tiles, k_splits), kWaves * 64, 0, stream>>>(
-      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
-      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters);
+  if constexpr (kEpilogue != kSkResidual && sizeof(TO) == 2 && MT == 1) {
+    if (norm.weight != nullptr) {
+      // (float rows take twice the registers: two sets of two steps keep two blocks on a compute unit)
+      ALOFA_REQUIRE(K % 4 == 0 && K <= kMaxNormK, "gemm_skinny: the norm's weights must fit in LDS [K=%d, at most %d]", K, kMaxNormK);
+      gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, true><<<dim3(col_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
+          static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
+          reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps);
+      return check_launch("gemm_skinny (with norm)");
+    }
+  }
+  ALOFA_REQUIRE(norm.weight == nullptr, "gemm_skinny: the norm goes with at most 16 rows and the bfloat16 store and swiglu epilogues only");
+  gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, unroll, false><<<dim3(col_tiles, k_splits), kWaves * 64, 0, stream>>>(
+      static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W),
+      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, nullptr, 0.f);
   return check_launch("gemm_skinny");
 }
 
 template <int kEpilogue, typename TO>
 static int dispatch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
-                           const float* bias, int M, int N, int K, hipStream_t stream) {
+                           const float* bias, int M, int N, int K, NormArgs norm, hipStream_t stream, int* splits_only = nullptr) {
   // few columns: one 16-column tile per block and eight waves along K keep more of the chip busy;
   // many columns and many rows: four column tiles per block, so that the rows are read less often
   const bool narrow = (kEpilogue != kSkSwiglu) && N <= 4096;
 #define ALOFA_SKINNY(MT, WIDE)                                                                                        \
   if (kEpilogue == kSkSwiglu)                                                                                         \
-    return launch_skinny<MT, 2, (MT >= 4 ? 4 : 8), kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream); \
-  if (narrow) return launch_skinny<MT, 1, 8, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);     \
-  return launch_skinny<MT, WIDE, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream);
+    return launch_skinny<MT, 2, (MT >= 4 ? 4 : 8), kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm, stream, splits_only); \
+  if (narrow) return launch_skinny<MT, 1, 8, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm, stream, splits_only);     \
+  return launch_skinny<MT, WIDE, 4, kEpilogue, TO>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm, stream, splits_only);
   if (M <= 16) { ALOFA_SKINNY(1, 2) }
   if (M <= 32) { ALOFA_SKINNY(2, 4) }
   ALOFA_SKINNY(4, 4)
@@ -260,11 +396,27 @@ static int dispatch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, c
 
 using namespace alofa;
 
+// Parts of K that alofa_gemm_skinny would share out over blocks for these sizes (1: none).
+extern "C" int alofa_gemm_skinny_splits(int o_dtype, int M, int N, int K, int epilogue) {
+  int splits = 1;
+  const NormArgs none{nullptr, 0.f};
+  if (M <= 0 || M > 64) return 1;
+  if (epilogue == kSkStore && o_dtype == kBF16) dispatch_skinny<kSkStore, bf16_t>(nullptr, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, M, N, K, none, nullptr, &splits);
+  if (epilogue == kSkStore && o_dtype == kF32) dispatch_skinny<kSkStore, float>(nullptr, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, M, N, K, none, nullptr, &splits);
+  if (epilogue == kSkResidual) dispatch_skinny<kSkResidual, float>(nullptr, 0, nullptr, 0, nullptr, nullptr, 0, nullptr, M, N, K, none, nullptr, &splits);
+  return splits;
+}
+
 // bfloat16 A [M, K] (M <= 64) and W [N, K] (W2 for the swiglu epilogue); K a multiple of 8,
 // rows 16-byte aligned. Epilogues: 0 store (+ bias) as o_dtype, 1 add to the float residual, 2 swiglu.
+// norm_w (float [K]) not null: A is float [M, K] and takes an RMSNorm with these weights and eps on
+// its way into the product (bfloat16 store and swiglu epilogues; K is then not shared out over blocks).
 extern "C" int alofa_gemm_skinny(void* out, int o_dtype, int64_t ldo, const void* A, int64_t lda, const void* W,
                                  const void* W2, int64_t ldw, const float* bias, int M, int N, int K, int epilogue,
-                                 hipStream_t stream) {
+                                 const float* norm_w, float eps, hipStream_t stream) {
+  const NormArgs norm{norm_w, eps};
+  ALOFA_REQUIRE(norm_w == nullptr || (reinterpret_cast<uintptr_t>(norm_w) % 16 == 0 && lda % 4 == 0 && eps > 0.f),
+                "gemm_skinny: the norm's weights must be 16-byte aligned, eps positive");
   ALOFA_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: M=%d (1..64) N=%d K=%d", M, N, K);
   ALOFA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K=%d, lda=%lld, ldw=%lld must be multiples of 8", K,
                 static_cast<long long>(lda), static_cast<long long>(ldw));
@@ -272,14 +424,14 @@ extern "C" int alofa_gemm_skinny(void* out, int o_dtype, int64_t ldo, const void
                     reinterpret_cast<uintptr_t>(W2) % 16 == 0, "gemm_skinny: operands must be 16-byte aligned");
   ALOFA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_skinny: a leading dimension is shorter than its row");
   if (epilogue == kSkStore && o_dtype == kBF16)
-    return dispatch_skinny<kSkStore, bf16_t>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream);
+    return dispatch_skinny<kSkStore, bf16_t>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, norm, stream);
   if (epilogue == kSkStore && o_dtype == kF32)
-    return dispatch_skinny<kSkStore, float>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream);
+    return dispatch_skinny<kSkStore, float>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, norm, stream);
   if (epilogue == kSkResidual && o_dtype == kF32)
-    return dispatch_skinny<kSkResidual, float>(out, ldo, A, lda, W, nullptr, ldw, nullptr, M, N, K, stream);
+    return dispatch_skinny<kSkResidual, float>(out, ldo, A, lda, W, nullptr, ldw, nullptr, M, N, K, norm, stream);
   if (epilogue == kSkSwiglu && o_dtype == kBF16) {
     ALOFA_REQUIRE(W2 != nullptr, "gemm_skinny: the swiglu epilogue needs the up matrix");
-    return dispatch_skinny<kSkSwiglu, bf16_t>(out, ldo, A, lda, W, W2, ldw, nullptr, M, N, K, stream);
+    return dispatch_skinny<kSkSwiglu, bf16_t>(out, ldo, A, lda, W, W2, ldw, nullptr, M, N, K, norm, stream);
   }
   ALOFA_REQUIRE(false, "gemm_skinny: unsupported epilogue %d with out dtype %d", epilogue, o_dtype);
 }

@@ -5,6 +5,7 @@ fallback: a tensor that is not on the GPU, or a missing library, is an error."""
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -189,14 +190,55 @@ def _mfma_operands(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+NORM_MAX_ROWS, NORM_MAX_COLUMNS = 16, 8192     # what the streaming kernel's norm form takes (one tile of rows; the norm's weights lie in LDS)
+FUSE_NORMS = os.environ.get("ALOFA_FUSE_NORMS", "1") != "0"   # 0: every norm runs as a kernel of its own
+
+
+def can_fuse_norm(M: int, w: torch.Tensor, out_dtype, swiglu: bool = False) -> bool:
+    """Whether the product of ``M`` float32 rows with the bfloat16 matrix ``w`` can take an RMSNorm
+    of those rows on its way (``gemm(..., norm=)``, ``gemm_swiglu(..., norm=)``): the streaming
+    kernel does, where it is the kernel of choice and does not share K out over blocks."""
+    N, K = w.shape
+    if not FUSE_NORMS:
+        return False
+    if (w.dtype is not torch.bfloat16 or out_dtype is not torch.bfloat16 or M > NORM_MAX_ROWS or K > NORM_MAX_COLUMNS or K % 8 or w.stride(0) % 8
+            or w.data_ptr() % 16 or few_rows_kernel(M, 2 * N if swiglu else N, K, swiglu) != "stream"):
+        return False
+    if swiglu:
+        return True
+    _ensure_workspace(w.device)
+    return load().alofa_gemm_skinny_splits(_I(BF16), _I(M), _I(N), _I(K), _I(STORE)) == 1
+
+
+def _norm_operands(a: torch.Tensor, norm: tuple, K: int):
+    weight, eps = norm
+    _gpu("a", a, torch.float32, 2), _gpu("norm weight", weight, torch.float32, 1), _contig("norm weight", weight)
+    if weight.shape[0] != K or _rows("a", a) % 4 or a.data_ptr() % 16 or weight.data_ptr() % 16 or not eps > 0:
+        raise AlofaError("shape_mismatch", "the fused norm needs float32 rows, 16-byte aligned, one weight per column and a positive eps",
+                         f"a={tuple(a.shape)} weight={tuple(weight.shape)} eps={eps}")
+    return _ptr(weight), _F(eps)
+
+
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         add_to_out: bool = False, exact: bool = False, kernel: Optional[str] = None) -> None:
+         add_to_out: bool = False, exact: bool = False, kernel: Optional[str] = None, norm: Optional[tuple] = None) -> None:
     """out = a @ w.T (+ bias), or out += a @ w.T when ``add_to_out`` (out is then
     the float32 residual stream). w is [out_features, in_features]. ``kernel``
-    names the bfloat16 kernel ("stream" or "tiled") instead of ``few_rows_kernel``."""
+    names the bfloat16 kernel ("stream" or "tiled") instead of ``few_rows_kernel``.
+    ``norm`` = (weight, eps): ``a`` holds float32 rows that take an RMSNorm on their way
+    into the product (only where ``can_fuse_norm`` says so)."""
     _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w", w, None, 2)
     M, K = a.shape
     N = w.shape[0]
+    if norm is not None:
+        if add_to_out or exact or not can_fuse_norm(M, w, out.dtype) or tuple(out.shape) != (M, N) or w.shape[1] != K:
+            raise AlofaError("unsupported", "no kernel takes a norm with this product", f"a={tuple(a.shape)} w={tuple(w.shape)} out={out.dtype}")
+        if bias is not None:
+            _gpu("bias", bias, torch.float32, 1), _contig("bias", bias)
+            if bias.shape[0] != N:
+                raise AlofaError("shape_mismatch", "bias length does not fit", f"bias={tuple(bias.shape)} N={N}")
+        _call("alofa_gemm_skinny", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)),
+              _ptr(bias), _I(M), _I(N), _I(K), _I(STORE), *_norm_operands(a, norm, K), _stream())
+        return
     if w.shape[1] != K or tuple(out.shape) != (M, N):
         raise AlofaError("shape_mismatch", "matrix product shapes do not fit", f"a={tuple(a.shape)} w={tuple(w.shape)} out={tuple(out.shape)}")
     if bias is not None:
@@ -210,9 +252,11 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
         raise AlofaError("unsupported", "a product that adds to the residual stream takes no bias; add the bias in a buffer of its own")
     if not exact and _mfma_operands(a, w):
         _ensure_workspace(a.device)
-        _call(_product_entry(kernel, M, N, K), _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
+        entry = _product_entry(kernel, M, N, K)
+        no_norm = (_ptr(None), _F(0.0)) if entry == "alofa_gemm_skinny" else ()
+        _call(entry, _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
               _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
-              _I(ADD_TO_RESIDUAL if add_to_out else STORE), _stream())
+              _I(ADD_TO_RESIDUAL if add_to_out else STORE), *no_norm, _stream())
         return
     _call("alofa_gemm_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
           _ptr(w), _I(dtype_code(w)), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
@@ -220,8 +264,8 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
 
 
 def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, exact: bool = False,
-                kernel: Optional[str] = None) -> None:
-    """out = silu(a @ w_gate.T) * (a @ w_up.T). ``kernel`` as for ``gemm``."""
+                kernel: Optional[str] = None, norm: Optional[tuple] = None) -> None:
+    """out = silu(a @ w_gate.T) * (a @ w_up.T). ``kernel`` and ``norm`` as for ``gemm``."""
     _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w_gate", w_gate, None, 2), _gpu("w_up", w_up, None, 2)
     M, K = a.shape
     N = w_gate.shape[0]
@@ -229,10 +273,18 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: 
         raise AlofaError("shape_mismatch", "gate/up product shapes do not fit", f"a={tuple(a.shape)} gate={tuple(w_gate.shape)} up={tuple(w_up.shape)} out={tuple(out.shape)}")
     if w_gate.dtype is not w_up.dtype or _rows("w_gate", w_gate) != _rows("w_up", w_up):
         raise AlofaError("invalid_argument", "gate and up matrices must share dtype and layout")
+    if norm is not None:
+        if exact or not can_fuse_norm(M, w_gate, out.dtype, swiglu=True) or w_up.data_ptr() % 16:
+            raise AlofaError("unsupported", "no kernel takes a norm with this product", f"a={tuple(a.shape)} gate={tuple(w_gate.shape)} out={out.dtype}")
+        _call("alofa_gemm_skinny", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
+              _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), *_norm_operands(a, norm, K), _stream())
+        return
     if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up):
         _ensure_workspace(a.device)
-        _call(_product_entry(kernel, M, 2 * N, K, True), _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
-              _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), _stream())
+        entry = _product_entry(kernel, M, 2 * N, K, True)
+        no_norm = (_ptr(None), _F(0.0)) if entry == "alofa_gemm_skinny" else ()
+        _call(entry, _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
+              _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), *no_norm, _stream())
         return
     _call("alofa_gemm_swiglu_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
           _ptr(w_gate), _ptr(w_up), _I(dtype_code(w_gate)), _L(_rows("w_gate", w_gate)), _I(M), _I(N), _I(K), _I(int(exact)), _stream())
@@ -312,13 +364,14 @@ def decode_waves(d: int) -> int:
 
 def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
     """Parts the keys of a (token, key head) are cut into beyond the waves of a block. None while a
-    wave has at most eight steps of 32 keys. Longer contexts: down to about four steps a wave, but
-    only until the blocks fill the chip (a block's fixed cost is paid once per part)."""
+    wave has at most eight steps of 32 keys (a second kernel that merges the parts costs as much as
+    it saves there). Longer contexts: down to about two steps a wave, but only until the blocks fill
+    the chip (a block's fixed cost is paid once per part)."""
     waves = decode_waves(d)
     if max_context <= 32 * waves * 8:
         return 1
     blocks = tokens * kv_heads * -(-(heads // kv_heads) // 16)
-    by_length = -(-max_context // (32 * waves * 4))
+    by_length = -(-max_context // (32 * waves * 2))
     by_chip = max(1, 256 // max(1, blocks))
     return max(1, min(64, by_length, by_chip))
 

@@ -103,11 +103,18 @@ class GQAAttention(Mixer):
     def prepare(self, n_positions):
         self.position.table(n_positions)       # built up to the context bound once, so that it never moves afterwards
 
-    def forward(self, ctx, entry, x, residual):
-        T = x.shape[0]
+    def fuses_norm(self, norm, rows):
+        return (not self.rt.exact and norm.as_rmsnorm() is not None
+                and ops.can_fuse_norm(rows, self.w_qkv, self.rt.dtype))
+
+    def forward(self, ctx, entry, x, residual, norm=None):
+        T = residual.shape[0]
         exact = self.rt.exact
         qkv = ctx.scratch("qkv", (T, self.qkv_width), self.rt.dtype)
-        ops.gemm(qkv, x, self.w_qkv, self.b_qkv, exact=exact)
+        if norm is not None:      # the input norm rides on the product
+            ops.gemm(qkv, residual, self.w_qkv, self.b_qkv, norm=norm.as_rmsnorm())
+        else:
+            ops.gemm(qkv, x, self.w_qkv, self.b_qkv, exact=exact)
         kv = ctx.kv(entry)
         plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
         table = self.position.table(ctx.n_positions)

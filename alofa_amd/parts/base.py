@@ -143,6 +143,12 @@ class Mixer(Part):
     def prepare(self, n_positions: int) -> None:
         """Build what must not move once steps run (tables up to the context bound)."""
 
+    def fuses_norm(self, norm, rows: int) -> bool:
+        """Whether, for a step of ``rows`` rows, this part would rather apply ``norm`` to the
+        residual stream itself (inside its first kernel) than be handed normed rows. A part that
+        says yes is called as ``forward(ctx, where, None, residual, norm=norm)``."""
+        return False
+
     def forward(self, ctx, where, x: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
 
@@ -150,6 +156,10 @@ class Mixer(Part):
 class FeedForward(Part):
     family = "feed_forward"
     capturable = False
+
+    def fuses_norm(self, norm, rows: int) -> bool:
+        """As for a mixer: yes means ``forward(ctx, None, residual, norm=norm)``."""
+        return False
 
     def forward(self, ctx, x: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
@@ -197,6 +207,11 @@ class Block(Part):
 
 class Norm(Part):
     family = "norm"
+
+    def as_rmsnorm(self):
+        """(weight float32 [width], eps) when the norm is x / sqrt(mean(x^2) + eps) * weight, which
+        some kernels can apply on their way; None for any other norm."""
+        return None
 
     def forward(self, out: torch.Tensor, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         raise NotImplementedError

@@ -36,11 +36,19 @@ class PreNormBlock(Block):
         return [self.mixer]
 
     def forward(self, ctx, entry, hidden):
+        rows = hidden.shape[0]
         normed = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
-        self.norms[0].forward(normed, hidden)
-        self.mixer.forward(ctx, entry, normed, hidden)
-        self.norms[1].forward(normed, hidden)
-        self.feed_forward.forward(ctx, normed, hidden)
+        # a part may take the norm into its first kernel (a launch less where launches are what a step costs)
+        if self.mixer.fuses_norm(self.norms[0], rows):
+            self.mixer.forward(ctx, entry, None, hidden, norm=self.norms[0])
+        else:
+            self.norms[0].forward(normed, hidden)
+            self.mixer.forward(ctx, entry, normed, hidden)
+        if self.feed_forward.fuses_norm(self.norms[1], rows):
+            self.feed_forward.forward(ctx, None, hidden, norm=self.norms[1])
+        else:
+            self.norms[1].forward(normed, hidden)
+            self.feed_forward.forward(ctx, normed, hidden)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -31,9 +31,16 @@ class SwiGLU(FeedForward):
         self.w_gate, self.w_up = rt.matrix(gate), rt.matrix(up)
         self.w_down = rt.matrix(weights[pre + "down_proj.weight"])
 
-    def forward(self, ctx, x, residual):
-        act = ctx.scratch("ff_act", (x.shape[0], self.intermediate), self.rt.dtype)
-        ops.gemm_swiglu(act, x, self.w_gate, self.w_up, exact=self.rt.exact)
+    def fuses_norm(self, norm, rows):
+        return (not self.rt.exact and norm.as_rmsnorm() is not None
+                and ops.can_fuse_norm(rows, self.w_gate, self.rt.dtype, swiglu=True))
+
+    def forward(self, ctx, x, residual, norm=None):
+        act = ctx.scratch("ff_act", (residual.shape[0], self.intermediate), self.rt.dtype)
+        if norm is not None:      # the norm before the feed-forward rides on the gate/up product
+            ops.gemm_swiglu(act, residual, self.w_gate, self.w_up, norm=norm.as_rmsnorm())
+        else:
+            ops.gemm_swiglu(act, x, self.w_gate, self.w_up, exact=self.rt.exact)
         ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact)
 
 

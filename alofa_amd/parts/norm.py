@@ -21,6 +21,9 @@ class RMSNorm(Norm):
         self.width = int(spec.params["width"])
         self.weight = rt.vector(weights[spec.params["name"]])
 
+    def as_rmsnorm(self):
+        return self.weight, self.eps
+
     def forward(self, out, x, rows=None):
         ops.rmsnorm(out, x, self.weight, self.eps, self.rt.exact, rows)
 

@@ -396,7 +396,7 @@ def long_prompts(args):
         t1 = time.perf_counter()
         core.tick()
         act = core.last_action
-        if act.prefill and not act.decode:
+        if act.prefill:                     # ticks that bring prompt portions (later ones carry a few decoded tokens beside them)
             sync()
             prefill_s += time.perf_counter() - t1
             prefill_tokens += sum(e - s for _, s, e in act.prefill)

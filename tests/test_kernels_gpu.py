@@ -120,6 +120,45 @@ def test_gemm_bf16(M, N, K, kernel):
     close(outw, pm.linear(a, w32, b), BF16, "f32 weight")
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 1152, 896), (8, 1152, 896), (16, 130, 264), (3, 97, 80), (11, 200, 2040), (16, 176, 1000), (7, 3000, 8192), (5, 4608, 3584), (17, 64, 64), (8, 9000, 8192)])
+def test_product_that_takes_the_norm_with_it(M, N, K):
+    """The streaming product applies the RMSNorm of its float32 rows on the way (x * w rounded to
+    bfloat16 as the operand, the row's factor on the finished sum): against the plain norm followed
+    by the plain product, and against the two kernels run one after the other."""
+    o = ops()
+    rng = np.random.default_rng(8)
+    x = (rng.standard_normal((M, K)) * rng.uniform(0.05, 30.0, (M, 1))).astype(np.float32)     # rows of very different size
+    nw = (1.0 + 0.3 * rng.standard_normal(K)).astype(np.float32)
+    w, w2 = (bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1) for _ in range(2))
+    b = rng.standard_normal(N).astype(np.float32)
+    eps = 1e-5
+    if not o.can_fuse_norm(M, t(w, torch.bfloat16), torch.bfloat16):
+        from alofa_amd.csrc.build import load
+        assert (M > 16 or load().alofa_gemm_skinny_splits(1, M, N, K, 0) > 1 or o.few_rows_kernel(M, N, K) != "stream"), \
+            "only a product that has more than 16 rows, shares K out over blocks or is the tiled kernel's may refuse"
+        with pytest.raises(AlofaError):
+            o.gemm(torch.empty(M, N, device=DEV, dtype=torch.bfloat16), t(x), t(w, torch.bfloat16), t(b), norm=(t(nw), eps))
+        return
+    normed = pm.rmsnorm(x, nw, eps)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm(out, t(x), t(w, torch.bfloat16), t(b), norm=(t(nw), eps))
+    close(out, pm.linear(normed, w, b), BF16, "norm + product + bias")
+    # the two kernels one after the other: the same up to the rounding of the normed rows
+    y = torch.empty(M, K, device=DEV, dtype=torch.bfloat16)
+    o.rmsnorm(y, t(x), t(nw), eps, False)
+    two = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm(two, y, t(w, torch.bfloat16), t(b), kernel="stream")
+    assert (out.float() - two.float()).abs().max().item() <= 2e-2 * max(1.0, two.float().abs().max().item())
+    # rows do not depend on their neighbours: the first row alone gives the same bits
+    one = torch.empty(1, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm(one, t(x[:1]), t(w, torch.bfloat16), t(b), norm=(t(nw), eps))
+    assert torch.equal(one[0], out[0])
+    assert o.can_fuse_norm(M, t(w, torch.bfloat16), torch.bfloat16, swiglu=True)
+    act = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm_swiglu(act, t(x), t(w, torch.bfloat16), t(w2, torch.bfloat16), norm=(t(nw), eps))
+    close(act, pm.swiglu(pm.linear(normed, w), pm.linear(normed, w2)), BF16, "norm + gate/up + swiglu")
+
+
 def test_gemm_split_over_blocks_is_repeatable():
     """Few rows and few columns: K is split over blocks that hand partial sums to the last one
     to arrive. The additions are in a fixed order, so every run gives the same bits; a partial
@@ -269,7 +308,7 @@ def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(5)])
     close(out, ref, BF16, "decode attention")
     if (heads, d, window) == (14, 64, None):
-        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == (1 if bucket == 700 else 8)   # several parts are really in play
+        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == (1 if bucket == 700 else 11)   # several parts are really in play (256 // 22 blocks)
     one = torch.empty(1, heads * d, device=DEV, dtype=torch.bfloat16)        # one token that sees one key
     o.paged_attention(one, c["qcat"][:1], c["kc"], c["vc"], c["table"], c["req"][:1], c["pos"][:1], heads, kv_heads, d, window, scale, False,
                       max_q_len=1, max_context=1)
