@@ -27,10 +27,11 @@ class Engine:
     def __init__(self, model_dir, dtype: str = "bfloat16", max_tokens: int = 256, max_batch: int = 8,
                  kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 2048, max_chunk: int = 512,
                  watermark_permille: int = 900, max_wait_ticks: int = 8, seed: int = 1234, device: str = "cuda:0",
-                 trace_path=None, share_prefixes: bool = False, model=None, report=None):
+                 trace_path=None, share_prefixes: bool = False, model=None, report=None, run_ahead: bool = True):
         """``model``: a (config, Model) pair already on the device, instead of a folder to load.
         ``report``: a callable that receives one line about device memory at start (default:
-        standard error when ALOFA_REPORT_MEMORY is set)."""
+        standard error when ALOFA_REPORT_MEMORY is set). ``run_ahead``: a tick reads the tokens of the
+        tick before only after its own step is launched (``EngineCore``); off, every tick is synchronous."""
         from .csrc.build import load
         load()
         self.config, self.model = model if model is not None else load_model(Path(model_dir), dtype, device)
@@ -45,7 +46,7 @@ class Engine:
         self.step_fn = StepFunction(self.model, self.cache, n_positions=max_tokens)
         self.sched_cfg = SchedConfig(token_budget, max_chunk, block_size, kv_blocks, watermark_permille, max_wait_ticks,
                                      n_slots=max(32, max_batch))
-        self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path, share_prefixes=share_prefixes)
+        self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path, share_prefixes=share_prefixes, run_ahead=run_ahead)
         self.seed = seed
         self._next_id = 1
         if report is None and os.environ.get("ALOFA_REPORT_MEMORY"):
@@ -89,6 +90,7 @@ class Engine:
             ticks += 1
             if ticks > max_ticks:
                 raise AlofaError("capacity", "generation did not finish within the tick limit", f"max_ticks={max_ticks}")
+        self.core.flush()
         outs = {}
         for rid in ids:
             outs[rid] = self.core.output(rid)

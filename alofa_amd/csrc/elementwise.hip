@@ -9,12 +9,19 @@
 namespace alofa {
 
 // ---- embedding -------------------------------------------------------------
-// hidden[t, :] = table[ids[t], :], widened to float. No scaling.
+// hidden[t, :] = table[ids[t], :], widened to float. No scaling. An id below zero stands for a token
+// that never left the device: -(s + 1) means store[s], where the choice of the last step put the
+// token of request slot s (brought into the vocabulary, so that no table row outside it is read).
 template <typename TW>
 __global__ void embed_gather_kernel(float* __restrict__ out, const TW* __restrict__ table,
-                                    const int32_t* __restrict__ ids, int width) {
+                                    const int32_t* __restrict__ ids, int width, const int32_t* __restrict__ store, int vocab) {
   const int t = blockIdx.x;
-  const TW* row = table + static_cast<int64_t>(ids[t]) * width;
+  int id = ids[t];
+  if (id < 0) {
+    id = store[-(id + 1)];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  }
+  const TW* row = table + static_cast<int64_t>(id) * width;
   float* dst = out + static_cast<int64_t>(t) * width;
   for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = load_f32(row + c);
 }
@@ -206,14 +213,16 @@ __global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gate, c
 
 using namespace alofa;
 
+// store: null when every id is a token (the caller has checked them against the vocabulary); else ids below
+// zero name slots of `store` (the caller has checked them against its length)
 extern "C" int alofa_embed_gather(float* out, const void* table, int table_dtype, const int32_t* ids, int tokens,
-                                  int width, hipStream_t stream) {
-  ALOFA_REQUIRE(tokens > 0 && width > 0, "embed_gather: tokens=%d width=%d must be positive", tokens, width);
+                                  int width, const int32_t* store, int vocab, hipStream_t stream) {
+  ALOFA_REQUIRE(tokens > 0 && width > 0 && vocab > 0, "embed_gather: tokens=%d width=%d vocab=%d must be positive", tokens, width, vocab);
   const int threads = width >= 256 ? 256 : 64;
   if (table_dtype == kF32)
-    embed_gather_kernel<float><<<tokens, threads, 0, stream>>>(out, static_cast<const float*>(table), ids, width);
+    embed_gather_kernel<float><<<tokens, threads, 0, stream>>>(out, static_cast<const float*>(table), ids, width, store, vocab);
   else if (table_dtype == kBF16)
-    embed_gather_kernel<bf16_t><<<tokens, threads, 0, stream>>>(out, static_cast<const bf16_t*>(table), ids, width);
+    embed_gather_kernel<bf16_t><<<tokens, threads, 0, stream>>>(out, static_cast<const bf16_t*>(table), ids, width, store, vocab);
   else
     ALOFA_REQUIRE(false, "embed_gather: unknown table dtype %d", table_dtype);
   return check_launch("embed_gather");

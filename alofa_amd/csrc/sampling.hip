@@ -15,7 +15,19 @@ namespace alofa {
 
 constexpr int kPickThreads = 1024;
 
-__global__ void __launch_bounds__(kPickThreads) argmax_kernel(int32_t* __restrict__ out, const float* __restrict__ logits,
+// Where a choice goes: out[r], and, when a store is given, store[store_index[r]] as well (the token
+// of request slot store_index[r], which the next step's embedding reads without a trip to the host).
+struct Choice {
+  int32_t* out;
+  int32_t* store;
+  const int32_t* store_index;
+  __device__ __forceinline__ void put(int r, int token) const {
+    out[r] = token;
+    if (store) store[store_index[r]] = token;
+  }
+};
+
+__global__ void __launch_bounds__(kPickThreads) argmax_kernel(Choice choice, const float* __restrict__ logits,
                                                               int64_t stride, int vocab) {
   __shared__ float best_v[kPickThreads / kWave];
   __shared__ int best_i[kPickThreads / kWave];
@@ -38,7 +50,7 @@ __global__ void __launch_bounds__(kPickThreads) argmax_kernel(int32_t* __restric
   if (threadIdx.x == 0) {
     for (int w = 1; w < kPickThreads / kWave; ++w)
       if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
-    out[blockIdx.x] = bi < vocab ? bi : 0;
+    choice.put(blockIdx.x, bi < vocab ? bi : 0);
   }
 }
 
@@ -77,7 +89,7 @@ __global__ void __launch_bounds__(256) argmax_chunk_kernel(float* __restrict__ p
   }
 }
 
-__global__ void __launch_bounds__(kWave) argmax_final_kernel(int32_t* __restrict__ out, const float* __restrict__ part_v,
+__global__ void __launch_bounds__(kWave) argmax_final_kernel(Choice choice, const float* __restrict__ part_v,
                                                              const int32_t* __restrict__ part_i, int vocab) {
   const int r = blockIdx.x;
   float bv = part_v[r * kArgmaxChunks + threadIdx.x];
@@ -87,10 +99,10 @@ __global__ void __launch_bounds__(kWave) argmax_final_kernel(int32_t* __restrict
     const int oi = __shfl_xor(bi, off, kWave);
     if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
   }
-  if (threadIdx.x == 0) out[r] = bi < vocab ? bi : 0;
+  if (threadIdx.x == 0) choice.put(r, bi < vocab ? bi : 0);
 }
 
-__global__ void __launch_bounds__(kPickThreads) sample_kernel(int32_t* __restrict__ out, const float* __restrict__ logits,
+__global__ void __launch_bounds__(kPickThreads) sample_kernel(Choice choice, const float* __restrict__ logits,
                                                               int64_t stride, int vocab,
                                                               const double* __restrict__ temperature,
                                                               const double* __restrict__ uniform) {
@@ -132,26 +144,40 @@ __global__ void __launch_bounds__(kPickThreads) sample_kernel(int32_t* __restric
     atomicMin(&found, pick);
   }
   __syncthreads();
-  if (tid == 0) out[r] = found;
+  if (tid == 0) choice.put(r, found);
 }
 
 }  // namespace alofa
 
 using namespace alofa;
 
+static int argmax_with(Choice choice, const float* logits, int64_t stride, int rows, int vocab, void* scratch, hipStream_t stream);
+
 // scratch: rows * 64 floats followed by rows * 64 int32 for long rows (null: one block per row)
 extern "C" int alofa_argmax(int32_t* out, const float* logits, int64_t stride, int rows, int vocab, void* scratch,
                             hipStream_t stream) {
+  return argmax_with(Choice{out, nullptr, nullptr}, logits, stride, rows, vocab, scratch, stream);
+}
+
+// The same, and store[store_index[r]] = out[r] as well (store_index: rows int32 indices the caller has checked
+// against the store's length).
+extern "C" int alofa_argmax_to_store(int32_t* out, const float* logits, int64_t stride, int rows, int vocab, void* scratch,
+                                     int32_t* store, const int32_t* store_index, hipStream_t stream) {
+  ALOFA_REQUIRE(store != nullptr && store_index != nullptr, "argmax_to_store: store and store_index must be given");
+  return argmax_with(Choice{out, store, store_index}, logits, stride, rows, vocab, scratch, stream);
+}
+
+static int argmax_with(Choice choice, const float* logits, int64_t stride, int rows, int vocab, void* scratch, hipStream_t stream) {
   ALOFA_REQUIRE(rows > 0 && vocab > 0 && stride >= vocab, "argmax: rows=%d vocab=%d stride=%lld", rows, vocab, static_cast<long long>(stride));
   if (scratch == nullptr) {
-    argmax_kernel<<<rows, kPickThreads, 0, stream>>>(out, logits, stride, vocab);
+    argmax_kernel<<<rows, kPickThreads, 0, stream>>>(choice, logits, stride, vocab);
     return check_launch("argmax");
   }
   float* part_v = static_cast<float*>(scratch);
   int32_t* part_i = reinterpret_cast<int32_t*>(part_v + static_cast<int64_t>(rows) * kArgmaxChunks);
   argmax_chunk_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(part_v, part_i, logits, stride, vocab);
   if (check_launch("argmax_chunk")) return 1;
-  argmax_final_kernel<<<rows, kWave, 0, stream>>>(out, part_v, part_i, vocab);
+  argmax_final_kernel<<<rows, kWave, 0, stream>>>(choice, part_v, part_i, vocab);
   return check_launch("argmax_final");
 }
 
@@ -205,13 +231,16 @@ extern "C" int alofa_argmax_no_alloc(int32_t* out, const float* logits, int64_t 
   int32_t* part_i = reinterpret_cast<int32_t*>(part_v + static_cast<int64_t>(rows) * kArgmaxChunks);
   argmax_chunk_kernel<<<dim3(kArgmaxChunks, rows), 256, 0, stream>>>(part_v, part_i, logits, stride, vocab);
   if (check_launch("argmax_chunk")) return 1;
-  argmax_final_kernel<<<rows, kWave, 0, stream>>>(out, part_v, part_i, vocab);
+  argmax_final_kernel<<<rows, kWave, 0, stream>>>(Choice{out, nullptr, nullptr}, part_v, part_i, vocab);
   return check_launch("argmax_final");
 }
 
+// store and store_index: both null, or as for alofa_argmax_to_store
 extern "C" int alofa_sample(int32_t* out, const float* logits, int64_t stride, int rows, int vocab,
-                            const double* temperature, const double* uniform, hipStream_t stream) {
+                            const double* temperature, const double* uniform, int32_t* store, const int32_t* store_index,
+                            hipStream_t stream) {
   ALOFA_REQUIRE(rows > 0 && vocab > 0 && stride >= vocab, "sample: rows=%d vocab=%d stride=%lld", rows, vocab, static_cast<long long>(stride));
-  sample_kernel<<<rows, kPickThreads, 0, stream>>>(out, logits, stride, vocab, temperature, uniform);
+  ALOFA_REQUIRE((store == nullptr) == (store_index == nullptr), "sample: store and store_index go together");
+  sample_kernel<<<rows, kPickThreads, 0, stream>>>(Choice{out, store, store_index}, logits, stride, vocab, temperature, uniform);
   return check_launch("sample");
 }

@@ -11,11 +11,22 @@ settle, one scheduler action per tick (src/alofa/engine/core.mojo:382-694).
            requests that have produced ``max_new`` tokens: their pages go back
            at once and the scheduler hears of it on the next tick.
 
+A token chosen on the device stays there: the choice writes it to the step
+function's token store, where the next step's embedding finds it. What the host
+needs of it is only its value for the output, and nothing the scheduler decides
+depends on values (requests end by count). So the engine runs ahead: a tick
+lays out and launches its step, launches the choice and an asynchronous copy
+of the chosen tokens, and only then reads back the tokens of the tick before;
+the GPU never waits for the host between steps. Outputs lag the ticks by one
+until ``flush`` (``run`` and ``is_done`` see to that). Requests whose sampling
+needs the host (filters, penalties) make their tick synchronous.
+
 Preemption is recompute: the victim loses its pages, its generated tokens and
 its generator state, and is fed again from its first prompt token. There is no
 end-of-sequence check: a request ends by count or by cancel (core.mojo:659-665)."""
 from __future__ import annotations
 
+from collections import deque
 from dataclasses import dataclass, field
 from typing import Optional
 
@@ -26,7 +37,7 @@ from .. import ops
 from ..errors import AlofaError
 from ..sampling.sampler import SampleParams, Sampler, SplitMix64
 from .scheduler import Action, SchedConfig, SchedInput, Scheduler, blocks_for
-from .step import StepEntry, StepFunction
+from .step import TOKEN_ON_DEVICE, StepEntry, StepFunction
 from .trace import config_line, trace_line
 
 QUEUED, RESIDENT, DONE = "queued", "resident", "done"
@@ -46,11 +57,18 @@ class Request:
     reported: bool = False
     preemptions: int = 0
     shared: int = 0                  # prompt tokens taken over from another request's pages
+    pending: int = 0                 # tokens chosen on the device whose values have not been read back yet
+    on_device: bool = False          # the last chosen token lies in the step function's token store
 
 
 class EngineCore:
-    def __init__(self, step_fn: StepFunction, sched_cfg: SchedConfig, trace_path=None, share_prefixes: bool = False):
+    def __init__(self, step_fn: StepFunction, sched_cfg: SchedConfig, trace_path=None, share_prefixes: bool = False,
+                 run_ahead: bool = True):
         self.fn = step_fn
+        # read the tokens of a tick back only after the next tick's step has been launched
+        self.run_ahead = bool(run_ahead)
+        self._inflight: deque = deque()      # (owed [(request id, preemptions)], pinned tokens, count, event), oldest first
+        self._staging = None
         # a new request starts on the whole pages of a resident request with the same first tokens
         # (by reference count) instead of computing them again; off unless asked for
         self.share_prefixes = bool(share_prefixes)
@@ -105,19 +123,21 @@ class EngineCore:
             self._cancels.append(req)
 
     def is_done(self, req: int) -> bool:
-        return self.requests[req].state == DONE
+        """Finished, and every token's value has arrived."""
+        r = self.requests[req]
+        return r.state == DONE and r.pending == 0
 
     def output(self, req: int) -> list:
         return list(self.requests[req].out)
 
     def release(self, req: int) -> None:
-        if self.requests[req].state != DONE:
+        if not self.is_done(req):
             raise AlofaError("invalid_argument", "only a finished request can be released", f"request={req}")
         del self.requests[req]
 
     def has_work(self) -> bool:
         return (bool(self._arrivals) or bool(self._cancels) or bool(self._to_report) or self._freed_blocks > 0
-                or any(r.state != DONE for r in self.requests.values()))
+                or bool(self._inflight) or any(r.state != DONE for r in self.requests.values()))
 
     def _scheduler_let_go(self, cancelled: list, finished: list) -> None:
         """What follows from the scheduler's phases 1 and 2: a cancelled request loses its pages here
@@ -165,6 +185,7 @@ class EngineCore:
             r = self.requests[p]
             self._drop(r)
             r.out, r.fed, r.state, r.rng = [], 0, QUEUED, SplitMix64(r.seed)
+            r.pending, r.on_device = 0, False          # a token of its still on its way is dropped when it arrives
             r.preemptions += 1
         entries, owes = [], []
         for req, start, end in act.prefill:
@@ -184,9 +205,9 @@ class EngineCore:
             r = self.requests[req]
             if req in act.preempted or r.state == DONE:
                 continue
-            if r.state != RESIDENT or not r.out:
+            if r.state != RESIDENT or not (r.out or r.pending):
                 raise AlofaError("invalid_argument", "decode for a request that is not resident", f"request={req}")
-            entries.append(StepEntry(req, [r.out[-1]], [0]))
+            entries.append(StepEntry(req, [TOKEN_ON_DEVICE if r.on_device else r.out[-1]], [0]))
             owes.append(req)
         return entries, owes
 
@@ -214,45 +235,121 @@ class EngineCore:
         self.shared_tokens += got
         return got
 
-    def choose(self, logits: torch.Tensor, owes: list) -> list:
-        """One token per row of ``logits``, for the requests in ``owes`` (in order)."""
-        reqs = [self.requests[o] for o in owes]
-        chosen = [None] * len(reqs)
-        dev = [i for i, r in enumerate(reqs) if r.params.plain]
-        if dev:
-            greedy = [i for i in dev if r_is_greedy(reqs[i])]
-            drawn = [i for i in dev if not r_is_greedy(reqs[i])]
-            if greedy:
-                rows = logits if len(greedy) == len(reqs) else logits[torch.tensor(greedy, device=logits.device)]
-                out = torch.empty(len(greedy), dtype=torch.int32, device=logits.device)
-                ops.argmax(out, rows)
-                for i, t in zip(greedy, out.tolist()):
-                    chosen[i] = int(t)
-            if drawn:
-                rows = logits[torch.tensor(drawn, device=logits.device)].contiguous()
-                temp = torch.tensor([reqs[i].params.temperature for i in drawn], dtype=torch.float64, device=logits.device)
-                u = torch.tensor([reqs[i].rng.next_uniform() for i in drawn], dtype=torch.float64, device=logits.device)
-                out = torch.empty(len(drawn), dtype=torch.int32, device=logits.device)
-                ops.sample(out, rows, temp, u)
-                for i, t in zip(drawn, out.tolist()):
-                    chosen[i] = int(t)
-        host = [i for i in range(len(reqs)) if chosen[i] is None]
-        if host:
-            rows = logits[torch.tensor(host, device=logits.device)].cpu().numpy()
-            for k, i in enumerate(host):
-                r = reqs[i]
-                self.sampler.build(rows[k], r.params, r.prompt + r.out)
-                chosen[i] = self.sampler.pick(r.rng.next_uniform()) if not r.params.greedy else int(np.argmax(self.sampler.weights))
-        return chosen
+    # ------------------------------------------------------------------ choice
+    def _stage(self):
+        """Small pinned blocks (taking turns, as a block's copy runs only when the GPU gets there)
+        and their mirror on the device: request slots of the rows that choose on the device,
+        temperatures and uniform numbers going up, chosen tokens coming down."""
+        if self._staging is None:
+            cap, dev = self.cache.max_requests, self.fn.device
+            up_bytes = 4 * cap + 16 * cap                       # int32 slots, float64 temperatures, float64 uniforms
 
-    def settle(self, owes: list, chosen: list) -> None:
-        it = iter(chosen)
+            def views(block, host):
+                v = {"slots": block[:4 * cap].view(torch.int32), "temperature": block[4 * cap:12 * cap].view(torch.float64),
+                     "uniform": block[12 * cap:].view(torch.float64)}
+                return {k: t.numpy() for k, t in v.items()} if host else v
+            mirror = torch.empty(up_bytes, dtype=torch.uint8, device=dev)
+            turns = []
+            for _ in range(3):
+                up = torch.empty(up_bytes, dtype=torch.uint8, pin_memory=True)
+                down = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+                turns.append({"up": up, "down": down, "tokens": down.numpy(), "event": torch.cuda.Event(), **views(up, True)})
+            self._staging = {"turns": turns, "turn": 0, "mirror": mirror, "chosen": torch.empty(cap, dtype=torch.int32, device=dev),
+                             **views(mirror, False)}
+        return self._staging
+
+    def choose(self, logits: torch.Tensor, owes: list) -> Optional[list]:
+        """One token per row of ``logits``, for the requests in ``owes`` (in order). Requests that
+        sample plainly (greedy, or temperature alone) choose on the device; the tokens go to the
+        token store and set out for the host, and None is returned: ``collect`` reads them later.
+        With a request that needs the host's chain the whole tick is synchronous and the tokens
+        are returned."""
+        reqs = [self.requests[o] for o in owes]
+        n = len(reqs)
+        host = [i for i, r in enumerate(reqs) if not r.params.plain]
+        greedy = [i for i, r in enumerate(reqs) if r.params.plain and r_is_greedy(r)]
+        drawn = [i for i, r in enumerate(reqs) if r.params.plain and not r_is_greedy(r)]
+        order = greedy + drawn
+        if order:
+            st = self._stage()
+            turn = st["turns"][st["turn"]]
+            st["turn"] = (st["turn"] + 1) % len(st["turns"])
+            turn["event"].synchronize()                          # this block's last use (three ticks ago) is over
+            ctx = self.fn.last_context
+            ng, nd = len(greedy), len(drawn)
+            slots = [self.cache.slot(reqs[i].id) for i in order]
+            if ng == n and ctx.request_slots is not None and ctx.request_slots.shape[0] == n:
+                slots_dev = ctx.request_slots                    # a decode step keeps its requests' slots on the device
+            else:
+                turn["slots"][:ng + nd] = slots
+                for k, i in enumerate(drawn):
+                    turn["temperature"][k] = reqs[i].params.temperature
+                    turn["uniform"][k] = reqs[i].rng.next_uniform()
+                st["mirror"].copy_(turn["up"], non_blocking=True)
+                slots_dev = st["slots"][:ng + nd]
+            chosen = st["chosen"]
+            if ng:
+                rows = logits if ng == n else logits[torch.tensor(greedy, device=logits.device)]
+                ops.argmax(chosen[:ng], rows, store=self.fn.token_store, store_index=slots_dev[:ng])
+            if nd:
+                rows = logits[torch.tensor(drawn, device=logits.device)].contiguous()
+                ops.sample(chosen[ng:ng + nd], rows, st["temperature"][:nd], st["uniform"][:nd],
+                           store=self.fn.token_store, store_index=slots_dev[ng:ng + nd])
+            turn["down"][:ng + nd].copy_(chosen[:ng + nd], non_blocking=True)
+            turn["event"].record()
+            for i in order:
+                reqs[i].on_device = True
+            sent = ([(reqs[i].id, reqs[i].preemptions) for i in order], turn["tokens"], ng + nd, turn["event"])
+            if not host:
+                self._inflight.append(sent)
+                return None
+        if not host:
+            return None
+        # the host's chain needs the logits now: this tick is synchronous, every value is returned
+        self.collect()
+        values = [None] * n
+        if order:
+            sent[3].synchronize()
+            for i, tok in zip(order, sent[1][:sent[2]].tolist()):
+                values[i] = int(tok)
+        rows = logits[torch.tensor(host, device=logits.device)].cpu().numpy()
+        for k, i in enumerate(host):
+            r = reqs[i]
+            self.sampler.build(rows[k], r.params, r.prompt + r.out)
+            values[i] = self.sampler.pick(r.rng.next_uniform()) if not r.params.greedy else int(np.argmax(self.sampler.weights))
+            r.on_device = False
+        return values
+
+    def collect(self, keep: int = 0) -> None:
+        """Read back the tokens that earlier choices sent on their way, oldest first, all but the
+        newest ``keep`` sets. A request that was preempted since, or released, no longer takes its token."""
+        while len(self._inflight) > keep:
+            owed, tokens, n, event = self._inflight.popleft()
+            event.synchronize()
+            for (rid, life), tok in zip(owed, tokens[:n].tolist()):
+                r = self.requests.get(rid)
+                if r is not None and r.preemptions == life and r.pending > 0:
+                    r.out.append(int(tok))
+                    r.pending -= 1
+
+    def flush(self) -> None:
+        """Every token chosen so far is in its request's output afterwards."""
+        self.collect()
+
+    def settle(self, owes: list, chosen: Optional[list]) -> None:
+        """``chosen``: the tokens (one per owing request, None where the value is still on its way) or
+        None when all are on their way. Ends requests by count; a token's value is not needed for that."""
+        it = iter(chosen) if chosen is not None else None
         for o in owes:
             if o is None:
                 continue
             r = self.requests[o]
-            r.out.append(next(it))
-            if len(r.out) >= r.max_new:
+            tok = next(it) if it is not None else None
+            if tok is None:
+                r.pending += 1
+            else:
+                r.out.append(tok)
+            if len(r.out) + r.pending >= r.max_new:
                 self._drop(r)
                 r.state = DONE
                 if self.sched.find(r.id) >= 0 and r.id not in self.last_action.finished:
@@ -264,7 +361,8 @@ class EngineCore:
                 r.state = DONE
 
     def tick(self) -> int:
-        """One whole tick; returns the rows that ran."""
+        """One whole tick; returns the rows that ran. When it returns, the tokens of the tick
+        before are in the outputs (all of them with ``run_ahead`` off)."""
         entries, owes = self.prepare()
         self.ticks += 1
         self.last_rows = sum(len(e.tokens) for e in entries)
@@ -273,8 +371,10 @@ class EngineCore:
             wanted = [o for o in owes if o is not None]
             chosen = self.choose(logits, wanted) if wanted else []
             self.settle(owes, chosen)
+            self.collect(keep=1 if self.run_ahead else 0)
         else:
             self.settle([], [])
+            self.collect()
         return self.last_rows
 
     def run(self, max_ticks: int = 1 << 30) -> None:
@@ -284,6 +384,7 @@ class EngineCore:
                 raise AlofaError("capacity", "the engine did not finish within the tick limit", f"max_ticks={max_ticks}")
             self.tick()
             n += 1
+        self.flush()
 
 
 def r_is_greedy(r: Request) -> bool:

@@ -22,10 +22,15 @@ def _pow2_ceil(n: int) -> int:
     return max(64, 1 << (int(n) - 1).bit_length())
 
 
+TOKEN_ON_DEVICE = -1     # as a StepEntry's only token: the token the last choice for this request left on the device
+
+
 @dataclass
 class StepEntry:
     """Next tokens of one request. ``want``: places among these tokens whose
-    logits are asked for (may be empty)."""
+    logits are asked for (may be empty). ``tokens == [TOKEN_ON_DEVICE]``: the one
+    token that the last choice for this request wrote to the step function's
+    ``token_store`` (``ops.argmax(..., store=)``); it never visits the host."""
     request: object
     tokens: list
     want: list = field(default_factory=list)
@@ -81,6 +86,8 @@ class StepContext:
         self._tables: list = []
         self._slots: list = []
         self._memo: dict = {}
+        self.token_store = fn.token_store
+        self.request_slots: Optional[torch.Tensor] = None   # int32 [entries] on the device, where the step keeps them there (decode graphs)
 
     @property
     def device(self):
@@ -150,9 +157,12 @@ class StepFunction:
         self._eager_scratch = self._scratch      # buffers of steps that run kernel by kernel
         self._retired: list = []                 # outgrown buffers that captured graphs may still use
         self._identity: dict = {}
+        # the last token chosen for the request in each slot, for choices that stay on the device
+        self.token_store = torch.zeros(cache.max_requests, dtype=torch.int32, device=self.device)
         self.cache_owner = model.cache_owners()      # (entry, k) -> the key of the cache that mixer uses
         self.steps_run = 0
         self.rows_run = 0
+        self.last_context: Optional[StepContext] = None
         # decode steps (one token per request) replay a captured HIP graph when every
         # part runs native kernels only; ALOFA_GRAPHS=0 switches that off
         self.use_graphs = os.environ.get("ALOFA_GRAPHS", "1") != "0" and model.capturable
@@ -207,7 +217,14 @@ class StepFunction:
             raise AlofaError("invalid_argument", "an entry brings no tokens", f"request={entries[int(n_tokens.argmin())].request}")
         slots = np.fromiter((self.cache.slot(e.request) for e in entries), dtype=np.int32, count=len(entries))
         ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=int(n_tokens.sum()))
-        if ids.min() < 0 or ids.max() >= vocab:
+        if ids.min() < 0:
+            # a token left on the device: the embedding is told the request's slot, as -(slot + 1)
+            starts = np.cumsum(n_tokens) - n_tokens
+            carried = ids[starts] == TOKEN_ON_DEVICE
+            if (ids < 0).sum() != carried.sum() or (n_tokens[carried] != 1).any():
+                raise AlofaError("out_of_range", "token id outside the vocabulary (a token left on the device is an entry's only token)", f"min={ids.min()}")
+            ids[starts[carried]] = -(slots[carried].astype(np.int64) + 1)
+        if ids.max() >= vocab:
             raise AlofaError("out_of_range", "token id outside the vocabulary", f"vocab={vocab} min={ids.min()} max={ids.max()}")
         for e, n in zip(entries, n_tokens):
             for w in e.want:
@@ -256,25 +273,29 @@ class StepFunction:
 
     # ---------------------------------------------------------- decode graphs
     def _decode_buffers(self, B: int) -> dict:
-        """Static device buffers of the decode graphs for batch B, and the pinned
-        host block that is copied over them in one piece before a replay."""
+        """Static device buffers of the decode graphs for batch B, and the pinned host blocks that
+        are copied over them in one piece before a replay. The host blocks take turns: a step may
+        be laid out while the copy of the step before has not run yet (it runs when the GPU gets
+        there), so that the host never has to wait for the GPU in order to prepare the next step."""
         if B not in self._graph_buffers:
             W = max(1, (self.n_positions + self.cache.block_size - 1) // self.cache.block_size)
             G = len(self.cache.groups)
-            n32 = 3 * B + G * B * W                      # ids, positions, req_of_token, tables
+            n32 = 4 * B + G * B * W                      # ids, positions, req_of_token, request slots, tables
             n32 += n32 % 2                               # keep the int64 part 8-byte aligned
-            nbytes = 4 * n32 + 8 * G * B                 # + slots
-            host = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+            nbytes = 4 * n32 + 8 * G * B                 # + cache slots
+
+            def views(block, host):
+                b32, b64 = block[:4 * n32].view(torch.int32), block[4 * n32:].view(torch.int64)
+                v = {"ids": b32[:B], "positions": b32[B:2 * B], "req_of_token": b32[2 * B:3 * B], "request_slots": b32[3 * B:4 * B],
+                     "tables": b32[4 * B:4 * B + G * B * W].view(G, B, W), "slots": b64.view(G, B)}
+                return {k: t.numpy() for k, t in v.items()} if host else v
             devb = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
-            h32, d32 = host[:4 * n32].view(torch.int32), devb[:4 * n32].view(torch.int32)
-            h64, d64 = host[4 * n32:].view(torch.int64), devb[4 * n32:].view(torch.int64)
-            buf = {"host": host, "dev": devb, "W": W, "scratch": {},
-                   "h_ids": h32[:B].numpy(), "h_pos": h32[B:2 * B].numpy(), "h_req": h32[2 * B:3 * B].numpy(),
-                   "h_tables": h32[3 * B:3 * B + G * B * W].view(G, B, W).numpy(), "h_slots": h64.view(G, B).numpy(),
-                   "ids": d32[:B], "positions": d32[B:2 * B], "req_of_token": d32[2 * B:3 * B],
-                   "tables": d32[3 * B:3 * B + G * B * W].view(G, B, W), "slots": d64.view(G, B),
-                   "rows": torch.arange(B, dtype=torch.int32, device=self.device), "copied": torch.cuda.Event()}
-            buf["h_req"][:] = np.arange(B, dtype=np.int32)
+            buf = {"dev": devb, "W": W, "scratch": {}, "turn": 0, "hosts": [], **views(devb, False),
+                   "rows": torch.arange(B, dtype=torch.int32, device=self.device)}
+            for _ in range(3):
+                host = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+                buf["hosts"].append({"block": host, "copied": torch.cuda.Event(), **views(host, True)})
+                buf["hosts"][-1]["req_of_token"][:] = np.arange(B, dtype=np.int32)
             self._graph_buffers[B] = buf
         return self._graph_buffers[B]
 
@@ -283,19 +304,23 @@ class StepFunction:
         cache = self.cache
         B = len(entries)
         buf = self._decode_buffers(B)
-        buf["copied"].synchronize()                      # the last copy out of the host block is done
+        host = buf["hosts"][buf["turn"]]
+        buf["turn"] = (buf["turn"] + 1) % len(buf["hosts"])
+        host["copied"].synchronize()                     # this block's last copy (three steps ago) is done
         pos0 = np.empty(B, dtype=np.int64)
         # the layout goes straight into the pinned block that is copied to the device in one piece
-        cache.plan_step_into(slots, n_tokens, self.n_positions, pos0, buf["h_pos"], buf["h_req"], buf["h_tables"], buf["h_slots"])
-        buf["h_ids"][:] = ids
+        cache.plan_step_into(slots, n_tokens, self.n_positions, pos0, host["positions"], host["req_of_token"], host["tables"], host["slots"])
+        host["ids"][:] = ids
+        host["request_slots"][:] = slots
         spans = self._spans(entries, slots, n_tokens, pos0)
-        ctx = StepContext(self, spans, buf["h_pos"].copy())
+        ctx = StepContext(self, spans, host["positions"].copy())
         ctx.entry_slots, ctx.entry_tokens = slots, n_tokens
         ctx.positions, ctx.req_of_token = buf["positions"], buf["req_of_token"]
+        ctx.request_slots = buf["request_slots"]
         ctx._tables = [buf["tables"][g] for g in range(len(cache.groups))]
         ctx._slots = [buf["slots"][g] for g in range(len(cache.groups))]
-        buf["dev"].copy_(buf["host"], non_blocking=True)
-        buf["copied"].record()
+        buf["dev"].copy_(host["block"], non_blocking=True)
+        host["copied"].record()
         key = (B, ctx.max_context)
         saved, self._scratch = self._scratch, buf["scratch"]   # graphs of one batch size share their own buffers
         try:
@@ -320,6 +345,7 @@ class StepFunction:
         finally:
             self._scratch = saved
         self.finish(ctx)
+        self.last_context = ctx
         return logits
 
     def run(self, entries: list) -> Optional[torch.Tensor]:
@@ -333,4 +359,5 @@ class StepFunction:
             hidden = self.model.forward(ctx, ids)
             logits = self.model.logits(ctx, hidden, rows) if rows is not None else None
             self.finish(ctx)
+            self.last_context = ctx
             return logits

@@ -93,15 +93,20 @@ def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
 
 # ----------------------------------------------------------------- embedding
 
-def embed_gather(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+def embed_gather(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, store: Optional[torch.Tensor] = None) -> None:
     """out[t] = table[ids[t]] widened to float32. ``ids`` must already be
-    checked against the vocabulary on the host."""
+    checked against the vocabulary on the host. With ``store`` (int32) an id
+    below zero, -(s + 1), stands for the token store[s] that an earlier choice
+    left on the device (``argmax`` and ``sample`` with ``store=``); the caller has
+    checked such s against the store's length."""
     _gpu("out", out, torch.float32, 2), _gpu("table", table, None, 2), _gpu("ids", ids, torch.int32, 1)
     _contig("out", out), _contig("table", table), _contig("ids", ids)
     T, h = out.shape
     if table.shape[1] != h or ids.shape[0] != T:
         raise AlofaError("shape_mismatch", "embedding width or token count does not fit", f"out={tuple(out.shape)} table={tuple(table.shape)} ids={tuple(ids.shape)}")
-    _call("alofa_embed_gather", _ptr(out), _ptr(table), _I(dtype_code(table)), _ptr(ids), _I(T), _I(h), _stream())
+    if store is not None:
+        _gpu("store", store, torch.int32, 1), _contig("store", store)
+    _call("alofa_embed_gather", _ptr(out), _ptr(table), _I(dtype_code(table)), _ptr(ids), _I(T), _I(h), _ptr(store), _I(table.shape[0]), _stream())
 
 
 # ---------------------------------------------------------------------- norm
@@ -539,22 +544,50 @@ def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_he
 
 # ------------------------------------------------------------------ sampling
 
-def argmax(out: torch.Tensor, logits: torch.Tensor) -> None:
-    """out[r] = first index of the maximum of logits[r] (lowest index on ties)."""
+_argmax_scratch: dict = {}
+
+
+def _store_operands(store, store_index, n: int):
+    if (store is None) != (store_index is None):
+        raise AlofaError("invalid_argument", "a token store goes with the index of every row's place in it")
+    if store is not None:
+        _gpu("store", store, torch.int32, 1), _contig("store", store), _gpu("store_index", store_index, torch.int32, 1), _contig("store_index", store_index)
+        if store_index.shape[0] != n:
+            raise AlofaError("shape_mismatch", "one place in the store per row", f"store_index={tuple(store_index.shape)} rows={n}")
+
+
+def argmax(out: torch.Tensor, logits: torch.Tensor, store: Optional[torch.Tensor] = None,
+           store_index: Optional[torch.Tensor] = None) -> None:
+    """out[r] = first index of the maximum of logits[r] (lowest index on ties); with ``store``
+    also store[store_index[r]] = out[r] (indices the caller has checked against the store)."""
     _gpu("out", out, torch.int32, 1), _gpu("logits", logits, torch.float32, 2), _contig("out", out)
-    if out.shape[0] != logits.shape[0]:
+    n = logits.shape[0]
+    if out.shape[0] != n:
         raise AlofaError("shape_mismatch", "one choice per row")
-    # long rows are searched by 64 blocks each, through a small scratch (values, then indices)
-    scratch = torch.empty(2 * 64 * logits.shape[0], dtype=torch.float32, device=logits.device) if logits.shape[1] >= 8192 else None
-    _call("alofa_argmax", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(logits.shape[0]), _I(logits.shape[1]), _ptr(scratch), _stream())
+    _store_operands(store, store_index, n)
+    # long rows are searched by 64 blocks each, through a small scratch (values, then indices) that is kept
+    scratch = None
+    if logits.shape[1] >= 8192:
+        key = logits.device
+        scratch = _argmax_scratch.get(key)
+        if scratch is None or scratch.numel() < 2 * 64 * n:
+            scratch = _argmax_scratch[key] = torch.empty(2 * 64 * max(n, 64), dtype=torch.float32, device=logits.device)
+    if store is None:
+        _call("alofa_argmax", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(n), _I(logits.shape[1]), _ptr(scratch), _stream())
+    else:
+        _call("alofa_argmax_to_store", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(n), _I(logits.shape[1]), _ptr(scratch),
+              _ptr(store), _ptr(store_index), _stream())
 
 
-def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor) -> None:
-    """out[r] = inverse-CDF draw from softmax(logits[r] / temperature[r]) at uniform[r] in [0, 1)."""
+def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
+           store: Optional[torch.Tensor] = None, store_index: Optional[torch.Tensor] = None) -> None:
+    """out[r] = inverse-CDF draw from softmax(logits[r] / temperature[r]) at uniform[r] in [0, 1); ``store`` as for ``argmax``."""
     _gpu("out", out, torch.int32, 1), _gpu("logits", logits, torch.float32, 2), _contig("out", out)
     _gpu("temperature", temperature, torch.float64, 1), _gpu("uniform", uniform, torch.float64, 1)
     _contig("temperature", temperature), _contig("uniform", uniform)
     n = logits.shape[0]
     if out.shape[0] != n or temperature.shape[0] != n or uniform.shape[0] != n:
         raise AlofaError("shape_mismatch", "one choice, temperature and uniform number per row")
-    _call("alofa_sample", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(n), _I(logits.shape[1]), _ptr(temperature), _ptr(uniform), _stream())
+    _store_operands(store, store_index, n)
+    _call("alofa_sample", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(n), _I(logits.shape[1]), _ptr(temperature), _ptr(uniform),
+          _ptr(store), _ptr(store_index), _stream())

@@ -28,7 +28,7 @@ class TokenEmbedding(Part):
 
     def forward(self, ctx, ids):
         hidden = ctx.scratch("hidden", (ids.shape[0], self.width), torch.float32)
-        ops.embed_gather(hidden, self.table, ids)
+        ops.embed_gather(hidden, self.table, ids, getattr(ctx, "token_store", None))
         return hidden
 
 

@@ -23,7 +23,8 @@ def test_product_kernel_by_shape():
 def test_decode_splits_follow_the_context():
     short = ops.decode_splits(8, 14, 2, 64, 1024)
     assert short == 1                                                             # the waves of one block cover a short context
-    assert ops.decode_splits(8, 14, 2, 64, 1 << 16) > ops.decode_splits(8, 14, 2, 64, 1 << 13) >= 1
+    assert ops.decode_splits(8, 14, 2, 64, 1 << 13) > ops.decode_splits(8, 14, 2, 64, 1 << 12) > 1   # about two steps of 32 keys a wave
+    assert ops.decode_splits(8, 14, 2, 64, 1 << 16) == 256 // 16                   # until the blocks fill the chip
     assert ops.decode_splits(64, 14, 2, 64, 1 << 13) <= ops.decode_splits(8, 14, 2, 64, 1 << 13)    # many blocks already: fewer parts
     assert ops.decode_waves(64) == 8 and ops.decode_waves(128) == 4 and ops.decode_waves(256) == 4
 

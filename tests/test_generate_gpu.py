@@ -169,7 +169,7 @@ def test_decode_time_preemption_recomputes(tiny_dirs):
     for i, p in enumerate(prompts):
         core.submit(i + 1, p, 25)                     # 3 x 3 blocks
     core.tick(), core.tick()
-    assert core.sched.blocks_used == 3 and all(len(r.out) == 2 for r in core.requests.values())
+    assert core.sched.blocks_used == 3 and all(len(r.out) + r.pending == 2 for r in core.requests.values())
     core.sched.cfg = SchedConfig(64, 32, 16, 5, 1000, 8, 32)     # five blocks: the second page of all three does not fit
     seen = []
     for _ in range(400):
@@ -234,6 +234,43 @@ def test_engine_shares_prefixes_when_asked(tiny_dirs):
     for i in range(5):
         core.release(i + 1)
     held_nothing(eng)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_ahead_changes_no_token(tiny_dirs, dtype):
+    """The engine launches a step before it has read the tokens of the step before (they stay on
+    the device for the next step's embedding). The same requests tick by tick with and without
+    running ahead, greedy and with a temperature, among them one that samples on the host (top-k),
+    which makes its ticks synchronous: the same tokens; and outputs lag a tick by at most one token."""
+    from alofa_amd import Engine
+    from alofa_amd.sampling.sampler import SampleParams
+    prompts = [random_ids(90 + i, n, 512) for i, n in enumerate((3, 19, 40, 8, 27))]
+    params = [SampleParams(temperature=0.0), SampleParams(temperature=0.7), SampleParams(temperature=0.0),
+              SampleParams(temperature=0.9, top_k=12), SampleParams(temperature=1.3)]
+
+    def play(run_ahead, late=()):
+        eng = Engine(tiny_dirs["B"], dtype=dtype, max_tokens=96, max_chunk=16, token_budget=40, run_ahead=run_ahead)
+        core, lag = eng.core, 0
+        for i, (p, sp) in enumerate(zip(prompts, params)):
+            if i not in late:
+                core.submit(i + 1, p, 14, sp, seed=77)
+        ticks = 0
+        while core.has_work():
+            core.tick()
+            ticks += 1
+            if ticks == 6:
+                for i in late:      # joins while the others decode; without the top-k request every tick runs ahead
+                    core.submit(i + 1, prompts[i], 14, params[i], seed=77)
+            lag = max(lag, max(r.pending for r in core.requests.values()))
+        outs = [core.output(i + 1) for i in range(5)]
+        assert all(core.is_done(i + 1) and len(outs[i]) == 14 for i in range(5))
+        held_nothing(eng)
+        return outs, lag, eng.step_fn.graph_replays
+    straight, lag0, _ = play(False)
+    ahead, lag1, replays = play(True)
+    assert lag0 == 0 and straight == ahead
+    joined, lag2, replays = play(True, late=(3,))
+    assert joined == straight and lag2 == 1 and (replays > 0 or dtype == "float32")
 
 
 def test_tight_pool_serves_requests_one_after_another(tiny_dirs):
