@@ -115,7 +115,8 @@ def main(argv=None) -> int:
                     watermark_permille=env_int("ALOFA_WATERMARK_PERMILLE", 900, 1, 1000),
                     max_wait_ticks=env_int("ALOFA_MAX_WAIT_TICKS", 8, 0, 1 << 20), seed=seed,
                     trace_path=env_str("ALOFA_TRACE", "") or None,
-                    share_prefixes=bool(env_int("ALOFA_SHARE_PREFIX", 0, 0, 1)))
+                    share_prefixes=bool(env_int("ALOFA_SHARE_PREFIX", 0, 0, 1)),
+                    report=lambda line: print(line, file=sys.stderr, flush=True))
     outs = engine.generate(prompts, max_new=max_new,
                            temperature=env_float("ALOFA_TEMPERATURE", 0.0, 0.0, 1e6),
                            top_k=env_int("ALOFA_TOP_K", 0, 0, 1 << 30), top_p=env_float("ALOFA_TOP_P", 1.0, 1e-9, 1.0),

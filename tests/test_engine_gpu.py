@@ -138,6 +138,40 @@ def test_wider_model_in_every_cutting(replayers, tiny_dirs, dtype):
     assert_close(collect(r, portions("p", ids, sizes=(70, 2, 130, 9, 33, 2)))["p"], ref, dtype, "D portions")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_peaky_attention_in_every_cutting(tiny_dirs, tmp_path, name, dtype):
+    """Random weights of size 0.02 make attention nearly uniform: one key among hundreds hardly
+    shows. Here the query and key matrices are scaled by eight, so that the scores are 64 times as
+    large and most queries put nearly all their weight on one key, often far behind them, across
+    page ends and (configuration C) at the edge of the window: a key dropped, doubled or taken from
+    the wrong page moves the logits by far more than rounding does, in bfloat16 too."""
+    import torch
+    from safetensors.torch import load_file, save_file
+    from alofa_amd.replay import Replayer
+    for f in ("config.json", "model.safetensors"):
+        (tmp_path / f).write_bytes((tiny_dirs[name] / f).read_bytes())
+    st = load_file(tmp_path / "model.safetensors")
+    for k in st:
+        if k.endswith("q_proj.weight") or k.endswith("k_proj.weight"):
+            st[k] = (st[k].float() * 8.0).to(st[k].dtype)
+    save_file(st, tmp_path / "model.safetensors")
+    ids = ids_of(name, seed=13, n=200)
+    ref = plain_logits(tmp_path, tuple(ids))
+    flat = plain_logits(tiny_dirs[name], tuple(ids))
+    assert np.abs(ref - flat).max() > 0.05 * np.abs(flat).max(), "the scaling changes what the model computes"
+    r = Replayer(tmp_path, dtype, 512)
+    assert_close(collect(r, whole("w", ids))["w"], ref, dtype, f"{name} peaky whole")
+    assert_close(collect(r, bulk_and_tail("t", ids, tail=90))["t"], ref, dtype, f"{name} peaky bulk+tail")
+    assert_close(collect(r, portions("p", ids))["p"], ref, dtype, f"{name} peaky portions")
+    requests = {f"r{i}": random_ids(300 + i, n, TINY[name]["vocab_size"]) for i, n in enumerate([200, 41, 150, 64, 35])}
+    steps, peak = mixed(requests, seed=9)
+    r = Replayer(tmp_path, dtype, peak)
+    got = collect(r, steps)
+    for k, v in requests.items():
+        assert_close(got[k], plain_logits(tmp_path, tuple(v)), dtype, f"{name} peaky mixed {k}")
+
+
 def random_config(rnd):
     """A Qwen2 configuration drawn at random: head sizes in steps of 16 up to 256, any head and
     group counts, widths and vocabularies that are no powers of two, windows on some layers."""
