@@ -233,7 +233,8 @@ def headline(args):
         print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
                                       "frac": round(prefill_flops(cfg, 2048) / pt / PEAK_FLOPS[args.dtype], 4)}}))
         return 0
-    if not 1 <= args.prompt <= CONTEXT - 8 * (args.steps + args.warmup) - 1:
+    timed = args.steps + args.warmup + (0 if args.no_points else 5 * max(8, args.steps // 2))      # steps this batch's requests decode
+    if not 1 <= args.prompt <= CONTEXT - timed - 1:
         print(f"--prompt must leave room for the decode steps within the context of {CONTEXT}")
         return 2
     roofs = None if args.no_points else measure_roofs()
