@@ -6,6 +6,7 @@ the order given (src/alofa/engine/executor.mojo:555-609 for the row layout,
 :665-859 for the pass)."""
 from __future__ import annotations
 
+import gc
 import os
 from dataclasses import dataclass, field
 from typing import Optional
@@ -331,9 +332,21 @@ class StepFunction:
                 logits = self.model.logits(ctx, hidden, buf["rows"])
                 torch.cuda.current_stream().synchronize()
                 graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph), ops.stream_scope():
-                    hidden = self.model.forward(ctx, buf["ids"])
-                    captured = self.model.logits(ctx, hidden, buf["rows"])
+                # No garbage collection while the stream is capturing: a collected object that owns device
+                # or pinned memory, an event or an older graph (a step function that went out of use, for
+                # one: it and its last context refer to each other) frees it with calls that a capturing
+                # stream forbids, and an error in a destructor ends the process. What is garbage already
+                # goes before the capture begins.
+                collecting = gc.isenabled()
+                gc.collect()
+                gc.disable()
+                try:
+                    with torch.cuda.graph(graph), ops.stream_scope():
+                        hidden = self.model.forward(ctx, buf["ids"])
+                        captured = self.model.logits(ctx, hidden, buf["rows"])
+                finally:
+                    if collecting:
+                        gc.enable()
                 if captured.data_ptr() != logits.data_ptr():
                     raise AlofaError("invalid_argument", "a buffer moved between the eager run and the capture")
                 self._graphs[key] = (graph, captured)

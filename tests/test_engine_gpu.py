@@ -87,6 +87,38 @@ def test_mixed_requests_with_pages_used_again(tiny_dirs, name, dtype):
         assert_close(got[k], plain_logits(tiny_dirs[name], tuple(ids)), dtype, f"{name} mixed {k}")
 
 
+def test_no_garbage_is_collected_while_a_decode_step_is_captured(tiny_dirs):
+    """A step function that went out of use is garbage that only the collector finds (it and its
+    last context refer to each other), and it owns pinned memory, events and graphs, which must not
+    be freed while a stream is capturing. With the collector set to run at every chance, none of
+    its runs may fall into the capture of a new decode step, and the step's logits are right."""
+    import gc
+    import torch
+    from alofa_amd.replay import Replayer
+    ids = ids_of("A", seed=21, n=70)
+    during = []
+
+    def watch(phase, info):
+        if phase == "start" and torch.cuda.is_current_stream_capturing():
+            during.append(info["generation"])
+
+    thresholds = gc.get_threshold()
+    gc.callbacks.append(watch)
+    try:
+        old = Replayer(tiny_dirs["A"], "bfloat16", 256)
+        collect(old, bulk_and_tail("o", ids, tail=4))        # decode steps: pinned blocks, events, a graph
+        del old
+        new = Replayer(tiny_dirs["A"], "bfloat16", 256)
+        gc.set_threshold(1, 1, 1)
+        got = collect(new, bulk_and_tail("n", ids, tail=4))["n"]
+    finally:
+        gc.set_threshold(*thresholds)
+        gc.callbacks.remove(watch)
+    assert during == []
+    assert new.fn.graph_replays > 0
+    assert_close(got, plain_logits(tiny_dirs["A"], tuple(ids)), "bfloat16", "A decoded beside garbage")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(replayers, tiny_dirs, dtype):
     ids = ids_of("C", seed=3, n=400)                     # crosses many pages and the window many times

@@ -182,6 +182,36 @@ def test_gemm_split_over_blocks_is_repeatable():
     assert int(differing) == 0
 
 
+@pytest.mark.parametrize("M,N,K", [(130, 200, 256), (257, 97, 64), (1100, 1100, 640), (65, 70, 128), (2048, 896, 896)])
+def test_gemm_tiled_with_slabs_straight_into_lds(M, N, K):
+    """Small tiles, K a multiple of 64 and not shared out: the form of the tiled product whose
+    slabs go from memory straight into LDS (rows past M and N are fetched from the last valid row,
+    the chunks of a row lie permuted). Every epilogue it has, edges in both directions, one slab
+    and many, and rows that are a strided view."""
+    rng = np.random.default_rng(47)
+    a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
+    b = rng.standard_normal(N).astype(np.float32)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm(out, t(a, torch.bfloat16), t(w, torch.bfloat16), t(b), kernel="tiled")
+    close(out, pm.linear(a, w, b), BF16, "bf16 out")
+    outf = torch.empty(M, N, device=DEV)
+    ops().gemm(outf, t(a, torch.bfloat16), t(w, torch.bfloat16), kernel="tiled")
+    close(outf, pm.linear(a, w), 1e-4, "f32 out")
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    acc = t(res)
+    ops().gemm(acc, t(a, torch.bfloat16), t(w, torch.bfloat16), add_to_out=True, kernel="tiled")
+    close(acc, pm.add(res, pm.linear(a, w)), 1e-4, "residual")
+    wide = torch.zeros(M, K + 72, device=DEV, dtype=torch.bfloat16)
+    wide[:, 8:8 + K] = t(a, torch.bfloat16)
+    ops().gemm(outf, wide[:, 8:8 + K], t(w, torch.bfloat16), kernel="tiled")
+    close(outf, pm.linear(a, w), 1e-4, "rows that are a view")
+    # a row's result does not depend on what else is in the batch, beyond the order of the additions (one row
+    # alone makes few tiles, whose K may be shared out among blocks)
+    one = torch.empty(1, N, device=DEV)
+    ops().gemm(one, t(a[M - 1:], torch.bfloat16), t(w, torch.bfloat16), kernel="tiled")
+    assert (one[0] - outf[M - 1]).abs().max().item() <= 2e-6 * outf[M - 1].abs().max().item()
+
+
 def test_gemm_takes_a_strided_view():
     rng = np.random.default_rng(4)
     big = rng.standard_normal((6, 300)).astype(np.float32)
