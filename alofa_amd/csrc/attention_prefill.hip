@@ -1,8 +1,13 @@
 // Paged causal grouped-query attention for prompt portions, bfloat16 on MFMA,
 // with a running softmax so that no score matrix is ever stored.
 //
-// A block serves 64 consecutive query rows of one request and one query head
-// with TEAMS teams of four wavefronts; within a team every wave owns 16 rows.
+// A block serves, with TEAMS teams of WPT wavefronts each, either (kShare false)
+// 64 consecutive query rows of one request and one query head, every wave of a
+// team owning 16 rows (WPT = 4); or (kShare true) 16 consecutive query rows and
+// up to WPT query heads of one key head, every wave of a team owning one head:
+// the heads of a group read the same keys and values, so a tile that is fetched
+// and staged once serves all of them (a fetch and a staging per head cost about
+// as much as the head's arithmetic).
 // The visible keys are walked in tiles of 64 that start at absolute multiples
 // of 64; the teams take the tiles in turn (a row's chain of dependent tiles is
 // TEAMS times shorter, and the teams' waves fill one another's stalls) and
@@ -38,8 +43,9 @@ constexpr int KPAD = 8, VPAD = 8;
 // tiles: int32 [n_blocks, 2, 4]: a block serves up to two runs of rows, one after the other, each
 // (request index, first row in the packed batch, rows (<= 64; 0: none), position of the first row). The caller
 // pairs long runs with short ones so that blocks carry about the same number of key tiles.
-template <int DT, int TEAMS>  // DT = d / 16
-__global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
+// kShare: blockIdx.y = key head * chunks + chunk of up to WPT query heads of its group; blockIdx.z = which 16 rows of the run.
+template <int DT, int TEAMS, int WPT, bool kShare>  // DT = d / 16
+__global__ void __launch_bounds__(64 * WPT * TEAMS) attention_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
     int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int bs_shift, int window,
@@ -49,26 +55,36 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
   constexpr int KROW = d + KPAD, VROW = BKV + VPAD;
   // per team: its key tile and its transposed value tile; at the end the same room takes the team's
   // running state (per lane its maximum, its sum and its 4 * DT channels)
-  constexpr int kStageBytes = (BKV * KROW + d * VROW) * 2, kStateBytes = 256 * (4 * DT + 2) * 4;
-  constexpr int kTeamBytes = ((kStageBytes > kStateBytes ? kStageBytes : kStateBytes) + 15) / 16 * 16;
+  constexpr int kTeamThreads = 64 * WPT;
+  static_assert(kShare || WPT == 4, "without sharing a team's four waves own the four 16-row groups of a run");
+  constexpr int kStageBytes = (BKV * KROW + d * VROW) * 2, kStateBytes = kTeamThreads * (4 * DT + 2) * 4;
+  constexpr int kTeamBytes = (((TEAMS > 1 && kStateBytes > kStageBytes) ? kStateBytes : kStageBytes) + 15) / 16 * 16;   // (one team hands no state over)
   __shared__ __attribute__((aligned(16))) char team_room[TEAMS * kTeamBytes];
-  const int team = threadIdx.x / 256;
+  const int team = threadIdx.x / kTeamThreads;
   bf16_t* Ks = reinterpret_cast<bf16_t*>(team_room + team * kTeamBytes);
   bf16_t* Vt = Ks + BKV * KROW;
 
-  const int tid = threadIdx.x % 256, wave = tid / 64, lane = tid % 64;
+  const int tid = threadIdx.x % kTeamThreads, wave = tid / 64, lane = tid % 64;
   const int c16 = lane % 16, g = lane / 16;
-  const int head = blockIdx.y, hk = head / (heads / kv_heads);
+  const int group = heads / kv_heads, chunks = (group + WPT - 1) / WPT;
+  // the query head this wave serves (kShare: a wave past the group's end helps with staging only), and its key head
+  const int hk = kShare ? blockIdx.y / chunks : blockIdx.y / group;
+  const bool head_ok = !kShare || (blockIdx.y % chunks) * WPT + wave < group;
+  const int head = kShare ? hk * group + (head_ok ? (blockIdx.y % chunks) * WPT + wave : 0) : blockIdx.y;
   for (int part = 0; part < 2; ++part) {
   const int32_t* tile = tiles + 8 * blockIdx.x + 4 * part;
-  const int req = tile[0], row0 = tile[1], n_rows = tile[2], pos0 = tile[3];
-  if (n_rows <= 0) break;     // uniform over the block
+  // kShare: the block takes rows 16 z .. of the run (fewer at the run's end; none: the block has nothing to do in this run)
+  const int sub = kShare ? 16 * blockIdx.z : 0;
+  const int req = tile[0], row0 = tile[1] + sub, pos0 = tile[3] + sub;
+  const int n_rows = kShare ? min(tile[2] - sub, 16) : tile[2];
+  if (tile[2] <= 0) break;    // uniform over the block
+  if (n_rows <= 0) continue;
   __syncthreads();            // the first run's last tile has been read by every wave
   const int32_t* table = block_table + static_cast<int64_t>(req) * max_blocks;
 
   // this lane's query row and its fragments of Q
-  const int my_row = wave * 16 + c16;                 // within the tile
-  const bool row_ok = my_row < n_rows;
+  const int my_row = kShare ? c16 : wave * 16 + c16;  // within the block's rows
+  const bool row_ok = my_row < n_rows && head_ok;
   const int my_pos = pos0 + my_row;
   bf16x8 qf[DS];
 #pragma unroll
@@ -97,12 +113,12 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
   // issued can stay on their way while the tile before is worked on, a load under a branch is waited for at
   // once. The page numbers of a tile are looked up one tile ahead of its keys and values for the same reason.
   constexpr int kChunks = BKV * d / 8;
-  constexpr int kPerThread = (kChunks + 255) / 256;
+  constexpr int kPerThread = (kChunks + kTeamThreads - 1) / kTeamThreads;
   const int page_mask = (1 << bs_shift) - 1;
   const int v_first = first_key & ~7, v_last = last_pos & ~7;    // first and last visible group of eight keys
   uint4 k_reg[kPerThread], v_reg[kPerThread];
   int k_page[kPerThread], v_page[kPerThread];
-  auto chunk_of = [&](int j) { const int c = tid + 256 * j; return c < kChunks ? c : kChunks - 1; };
+  auto chunk_of = [&](int j) { const int c = tid + kTeamThreads * j; return c < kChunks ? c : kChunks - 1; };
   auto k_key = [&](int t, int j) { return t * BKV + chunk_of(j) / (d / 8); };
   auto v_key0 = [&](int t, int j) { return t * BKV + (chunk_of(j) % 8) * 8; };
   auto clamp = [](int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); };
@@ -130,7 +146,7 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
     const bool whole = t * BKV >= first_key && t * BKV + BKV - 1 <= last_pos;   // uniform over the team
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
-      const int c = tid + 256 * j;
+      const int c = tid + kTeamThreads * j;
       if (c < kChunks) {
         uint4 kv = k_reg[j], vv = v_reg[j];
         if (!whole) {
@@ -171,6 +187,7 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
     if (!mine) continue;
     fetch(t + TEAMS);
     lookup(t + 2 * TEAMS);
+    if (!head_ok) continue;     // (a wave without a head of its own has done its share of the staging)
 
     // S^T for the four 16-key quarters of the tile
     f32x4 s[4];
@@ -297,10 +314,29 @@ __global__ void __launch_bounds__(256 * TEAMS) attention_prefill_kernel(
 
 using namespace alofa;
 
-// Teams per block: as many as the registers (128 per lane with four teams, and no spills) and the LDS of a
+// Teams per block: as many as the registers (128 per lane with 1,024 threads, and no spills) and the LDS of a
 // compute unit hold at this head size.
 template <int DT>
 constexpr int kTeams = (DT <= 2 || DT == 4) ? 4 : DT <= 8 ? 2 : 1;
+// ... where the heads of a group share the tiles: teams of as many waves as the block serves heads (six to eight)
+// (two teams of seven waves of head size 64 would spill)
+template <int DT>
+constexpr int kShareTeams = DT <= 2 ? 2 : 1;
+
+// How many heads of a group share their tiles in one block (0: none do; every head has blocks of its own). A
+// shared tile serves 16 rows of each of these heads where an unshared one serves 64 rows of one head, so fewer
+// than six heads save no staging (measured: five lose a fifth at 40/8 heads of size 128 and 16k keys, seven
+// win an eighth to a fifth at 28/4). Larger groups go in equal chunks of at most eight heads. Sharing cuts a
+// run of 64 rows into four blocks of 16, each of which walks the run's tiles with fewer teams: it pays when
+// there are enough blocks to fill the chip twice anyway, and loses when the longest block's walk is what the
+// launch waits for. Eight waves of head size 256 would not keep their state in registers.
+extern "C" int alofa_attention_prefill_share(int heads, int kv_heads, int d, int runs, int compute_units) {
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || d > 128) return 0;
+  const int group = heads / kv_heads, chunks = (group + 7) / 8, width = (group + chunks - 1) / chunks;
+  if (width < 6) return 0;
+  const int64_t blocks = static_cast<int64_t>(runs) * kv_heads * chunks * 4;
+  return blocks >= 2 * static_cast<int64_t>(compute_units) ? width : 0;
+}
 
 extern "C" int alofa_attention_prefill_supports(int d) {
   return d == 16 || d == 32 || d == 48 || d == 64 || d == 96 || d == 128 || d == 256;
@@ -309,7 +345,7 @@ extern "C" int alofa_attention_prefill_supports(int d) {
 extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                        const void* k_cache, const void* v_cache, const int32_t* block_table,
                                        int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
-                                       int block_size, int window, float scale, hipStream_t stream) {
+                                       int block_size, int window, float scale, int share, hipStream_t stream) {
   ALOFA_REQUIRE(n_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_prefill: tiles=%d heads=%d kv_heads=%d (kv_heads must divide heads)", n_tiles, heads, kv_heads);
   ALOFA_REQUIRE(alofa_attention_prefill_supports(d), "attention_prefill: head size %d is not built (16, 32, 48, 64, 96, 128, 256 are)", d);
@@ -319,11 +355,20 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
   while ((1 << bs_shift) < block_size) ++bs_shift;
   ALOFA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
                 "attention_prefill: q rows must be 16-byte aligned and out rows 8-byte aligned");
-  dim3 grid(n_tiles, heads);
-#define ALOFA_PREFILL(DT)                                                                                                 \
-  attention_prefill_kernel<DT, kTeams<DT>><<<grid, 256 * kTeams<DT>, 0, stream>>>(                                           \
+  const int group = heads / kv_heads, width = share;
+  ALOFA_REQUIRE(width == 0 || (width >= 6 && width <= 8 && d <= 128 && width <= group),
+                "attention_prefill: %d heads of a group of %d cannot share their tiles at head size %d (six to eight can, up to size 128)",
+                width, group, d);
+  const int chunks = width ? (group + width - 1) / width : 0;
+#define ALOFA_PREFILL_AS(DT, TEAMS, WPT, SHARE, GRID)                                                                         \
+  attention_prefill_kernel<DT, TEAMS, WPT, SHARE><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(                                    \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
       static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
+#define ALOFA_PREFILL_WIDE(DT, WPT)                                                                            \
+  if (width == WPT && DT <= 8) ALOFA_PREFILL_AS((DT <= 8 ? DT : 8), (kShareTeams<(DT <= 8 ? DT : 8)>), WPT, true, dim3(n_tiles, kv_heads * chunks, 4))
+#define ALOFA_PREFILL(DT)                                                                         \
+  ALOFA_PREFILL_WIDE(DT, 8); else ALOFA_PREFILL_WIDE(DT, 7); else ALOFA_PREFILL_WIDE(DT, 6);   \
+  else ALOFA_PREFILL_AS(DT, kTeams<DT>, 4, false, dim3(n_tiles, heads))
   switch (d / 16) {
     case 1: ALOFA_PREFILL(1); break;
     case 2: ALOFA_PREFILL(2); break;
@@ -334,5 +379,7 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
     case 16: ALOFA_PREFILL(16); break;
   }
 #undef ALOFA_PREFILL
+#undef ALOFA_PREFILL_WIDE
+#undef ALOFA_PREFILL_AS
   return check_launch("attention_prefill");
 }

@@ -505,10 +505,26 @@ def compute_units() -> int:
     return _compute_units
 
 
+def prefill_share(heads: int, kv_heads: int, d: int, runs: int) -> int:
+    """How many query heads of a group share their key and value tiles in one block of the prefill
+    attention kernel when it serves ``runs`` runs of up to 64 rows (the kernel's own rule: six to
+    eight heads, when the launch has blocks enough to fill the chip twice): 0 when every head has
+    blocks of its own."""
+    return int(load().alofa_attention_prefill_share(_I(heads), _I(kv_heads), _I(d), _I(runs), _I(compute_units())))
+
+
+def prefill_blocks_per_run(heads: int, kv_heads: int, share: int) -> int:
+    """Blocks of the prefill attention kernel that serve one run of up to 64 rows: one per query
+    head, or, where ``share`` heads of a group share their tiles, four blocks of 16 rows per chunk
+    of that many heads."""
+    return kv_heads * -(-(heads // kv_heads) // share) * 4 if share else heads
+
+
 def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = None) -> list:
     """``runs``: (request index, first row, rows <= 64, position of the first
     row) per run of rows. Returns per block two runs (the second may be empty).
-    When there are more blocks (runs x ``heads``) than compute units, the run
+    When there are more blocks (runs x ``heads``, the blocks that serve one run)
+    than compute units, the run
     that walks the most key tiles shares a block with the one that walks the
     fewest, and so on, so that blocks carry about the same work; with fewer,
     every run has a block of its own (a portion deep in a long context would
@@ -527,10 +543,12 @@ def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = 
     return out
 
 
-def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale) -> None:
+def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale, share: int = 0) -> None:
     """bfloat16 attention for portions of prompts. ``tiles`` is int32 [n, 2, 4]
     from ``pair_tiles``: per block up to two runs of rows, each (request index,
-    first row, rows <= 64 or 0 for none, position of the first row)."""
+    first row, rows <= 64 or 0 for none, position of the first row). ``share``
+    (from ``prefill_share``; the tiles were paired for its count of blocks):
+    that many heads of a group are served from one staged tile."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     if d not in PREFILL_HEAD_DIMS:
         raise AlofaError("unsupported", "the prefill attention kernel is not built for this head size", f"head_dim={d} built={PREFILL_HEAD_DIMS}")
@@ -539,7 +557,7 @@ def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_he
         raise AlofaError("shape_mismatch", "tiles must be [n, 2, 4]", f"tiles={tuple(tiles.shape)}")
     _call("alofa_attention_prefill", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
           _ptr(block_table), _I(block_table.shape[1]), _ptr(tiles), _I(tiles.shape[0]), _I(heads), _I(kv_heads), _I(d), _I(bs),
-          _I(int(window or 0)), _F(scale), _stream())
+          _I(int(window or 0)), _F(scale), _I(share), _stream())
 
 
 # ------------------------------------------------------------------ sampling

@@ -421,11 +421,15 @@ def test_decode_attention_with_many_splits(heads, kv_heads, d):
     assert err <= 1e-2 * np.abs(ref).max(), f"{err} vs {np.abs(ref).max()}"
 
 
-@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 96, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (3, 1, 32, 64)])
+@pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 96, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (3, 1, 32, 64),
+                                                 (22, 2, 32, 16), (6, 1, 256, 16), (28, 4, 128, 16), (7, 1, 16, 8), (16, 2, 64, 16), (6, 1, 96, 16)])
 @pytest.mark.parametrize("window", [None, 21, 300])
 def test_prefill_attention(heads, kv_heads, d, bs, window):
     """The tiled kernel for portions of prompts: whole prompts, portions deep in
-    a context, runs of exactly 64 and 65 rows, several tiles per request."""
+    a context, runs of exactly 64 and 65 rows, several tiles per request. A block serves 64 rows of
+    one head, or, in launches with many blocks and six or more query heads per key head (head sizes up
+    to 128), 16 rows of the heads of a group, which share the staged tiles (groups of six to eight in
+    teams of as many waves, eleven in chunks of six and five): both forms are run where the second exists."""
     rng = np.random.default_rng(23)
     lens, q_lens = [37, 130, 700, 64, 65, 200], [37, 5, 100, 64, 65, 200]
     c = paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16)
@@ -437,14 +441,25 @@ def test_prefill_attention(heads, kv_heads, d, bs, window):
     scale = float(np.float32(1) / np.sqrt(np.float32(d)))
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(len(lens))])
     # two runs per block (many blocks) and a block per run (fewer blocks than compute units)
-    paired, single = ops().pair_tiles(tiles, window), ops().pair_tiles(tiles, window, heads)
+    paired, single = ops().pair_tiles(tiles, window), ops().pair_tiles(tiles, window, 1)
     assert sorted(tuple(r) for b in paired for r in b if r[2]) == sorted(tiles) and len(paired) == (len(tiles) + 1) // 2
     assert [tuple(b[0]) for b in single] == tiles and all(b[1][2] == 0 for b in single)
     assert len(ops().pair_tiles(tiles * 40, window, heads)) == len(tiles) * 20
-    for name, blocks in (("paired", paired), ("single", single)):
-        out.zero_()
-        ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(blocks, np.int32), torch.int32), heads, kv_heads, d, window, scale)
-        close(out, ref, BF16, f"prefill attention, {name}")
+    # the kernel's own choice for a launch of few runs and of very many
+    group = heads // kv_heads
+    wide = ops().prefill_share(heads, kv_heads, d, 1 << 20)
+    assert ops().prefill_share(heads, kv_heads, d, 1) == 0
+    assert wide == {1: 0, 2: 0, 3: 0, 5: 0, 6: 6 if d <= 128 else 0, 7: 7, 8: 8, 11: 6}[group]
+    assert ops().prefill_blocks_per_run(heads, kv_heads, wide) == (kv_heads * -(-group // wide) * 4 if wide else heads)
+    for share in sorted({0, wide}):
+        for name, blocks in (("paired", paired), ("single", single)):
+            out.zero_()
+            ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(blocks, np.int32), torch.int32), heads, kv_heads, d, window, scale,
+                                    share=share)
+            close(out, ref, BF16, f"prefill attention, {name}, {share} heads share")
+    with pytest.raises(Exception, match="cannot share"):
+        ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(single, np.int32), torch.int32), heads, kv_heads, d, window, scale,
+                                share=5)
 
 
 def test_prefill_attention_far_key():
