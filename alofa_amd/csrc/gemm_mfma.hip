@@ -299,7 +299,8 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 
 // The same product with the slabs brought from memory straight into LDS (global_load_lds_dwordx4: every lane's
 // 16 bytes land at consecutive LDS addresses, 1 KB per wave and instruction, no registers and no LDS writes in
-// between) into a ring of S slabs. For K a multiple of 64 and no K shares.
+// between) into a ring of S slabs, S - 1 of them on their way while one is multiplied. For K a multiple of 64 and
+// no K shares. Which products take it: see launch_mfma.
 // A slab is 64 WTM rows of A and 64 WTN rows of W, 128 bytes each, unpadded; the eight 16-byte chunks of a row are
 // permuted by the row's number (chunk c of row r lies at place c ^ swz(r)), which the lane that fetches place p
 // of row r undoes by fetching chunk p ^ swz(r), so that the 16 or 32 rows whose fragments are read together
@@ -343,12 +344,18 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
       src[j] = base + static_cast<int64_t>(min(n, N - 1)) * ldw + c * 8;
     }
   }
+  // The fetches are written out as instructions: the compiler, which cannot tell the ring's slabs apart, would wait
+  // for every fetch on its way before any read from LDS, and the slabs set out ahead would be waited for at once.
+  // (M0 holds the LDS address of the wave's first lane; the instruction adds 16 bytes per lane.)
+  const unsigned ring_at = static_cast<unsigned>(reinterpret_cast<uintptr_t>(ring));
   auto fetch = [&](int slab) {     // uniform over the block
-    char* stage = ring + (slab % S) * kStageBytes + wave * 1024;
+    const unsigned stage = ring_at + (slab % S) * kStageBytes + wave * 1024;
 #pragma unroll
-    for (int j = 0; j < kLoads; ++j)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[j] + static_cast<int64_t>(slab) * TK),
-                                       (__attribute__((address_space(3))) void*)(stage + j * 4096), 16, 0, 0);
+    for (int j = 0; j < kLoads; ++j) {
+      const bf16_t* from = src[j] + static_cast<int64_t>(slab) * TK;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :: "s"(__builtin_amdgcn_readfirstlane(stage + j * 4096)), "v"(from), "r"(ring) : "memory", "m0");
+    }
   };
 
   f32x16 acc[WTM][WTN];
@@ -393,16 +400,24 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
   };
 
   // Slab k + S - 1 is set out once every wave has read slab k - 1 (whose place it takes), i.e. after the barrier
-  // of step k, and has the multiplications of S - 1 steps to arrive. A wave waits for its own fetches before the
-  // barrier; behind the barrier all of the slab is there.
+  // of step k, and has the multiplications of S - 1 steps to arrive. A wave waits for its own fetches of slab k
+  // (the S - 2 slabs behind it stay on their way) before the barrier; behind the barrier all of the slab is there.
+  constexpr int kLead = S - 1;
 #pragma unroll
-  for (int p = 0; p < S - 1; ++p)
+  for (int p = 0; p < kLead; ++p)
     if (p < slabs) fetch(p);
-  for (int k = 0; k < slabs; ++k) {
+  int k = 0;
+  for (; k + kLead < slabs; ++k) {
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLoads * (kLead - 1)) : "memory");
+    __syncthreads();
+    read(k);
+    fetch(k + kLead);
+    multiply();
+  }
+  for (; k < slabs; ++k) {      // nothing more to set out: the last slabs as they come
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     read(k);
-    if (k + S - 1 < slabs) fetch(k + S - 1);
     multiply();
   }
   tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out, ldo, bias, M, N, m0, n0, wm, wn, lane);
@@ -420,20 +435,21 @@ static int launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t 
   // operands beyond what the eight L2s hold together (4 MB each)
   const int w_rows = (kEpilogue == kMfSwiglu) ? 2 * N : N;
   const int by_die = (static_cast<int64_t>(M) + w_rows) * K * 2 > (32 << 20);
-  // Small tiles with K a multiple of the slab: the slabs go straight into LDS (measured against the kernel below at
-  // 2,048 rows: 13.1 against 15.4 us for N = 1,152, K = 896; 86 against 98 for 3,584 x 3,584; 399 against 468 for
-  // N = 3,584, K = 18,944; no gain at 128 x 128 tiles, where a ring of two slabs leaves room for two blocks per
-  // compute unit instead of three: 71 against 61 us for N = 9,728, K = 896).
-  if constexpr (!kSplitK && WTM == 1 && WTN == 1 && kEpilogue != kMfSwiglu) if (K % TK == 0) {
-    gemm_dma_kernel<kEpilogue, TO, 1, 1, 2><<<tiles_n * tiles_m, 256, 0, stream>>>(
-        static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
-        static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, tiles_m, tiles_n, by_die);
-    return 0;
-  }
   gemm_mfma_kernel<kEpilogue, TO, WTM, WTN, PF, kSplitK><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
       static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, tiles_m, tiles_n, shares, kSplitK ? g_ws.tiles : nullptr,
       kSplitK ? g_ws.counters : nullptr, by_die);
+  return 0;
+}
+
+template <int kEpilogue, typename TO, int WTM, int WTN, int S>
+static int launch_dma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
+                      hipStream_t stream) {
+  const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
+  const int by_die = (static_cast<int64_t>(M) + N) * K * 2 > (32 << 20);
+  gemm_dma_kernel<kEpilogue, TO, WTM, WTN, S><<<tiles_n * tiles_m, 256, 0, stream>>>(
+      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, bias, M, N, K,
+      tiles_m, tiles_n, by_die);
   return 0;
 }
 
@@ -472,11 +488,23 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 127) / 128, 1, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     } else if (big_blocks >= 512) {
       if (launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 127) / 128, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
+    } else if (big_blocks >= 256 && K % TK == 0) {
+      // One to two big tiles per compute unit: a ring of two slabs filled straight from memory, two blocks per
+      // compute unit, all of them resident at once. (2,048 rows, weights from memory, against the small tiles
+      // below: 71 against 102 us for 3,584 x 3,584, 335 against 513 for N = 3,584, K = 18,944. With more tiles
+      // than two per compute unit the three resident blocks of the kernel above do better: 107 against 137 us
+      // for N = 4,608, K = 3,584.)
+      if (launch_dma<kEpilogue, TO, 2, 2, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
     } else {
       const int tiles_n = (N + 63) / 64, tiles_m = (M + 63) / 64;
       const int shares = k_shares(static_cast<int64_t>(tiles_n) * tiles_m, 64 * 64, K);
       if (shares > 1) {
         if (launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
+      } else if (K % TK == 0) {
+        // small tiles, slabs straight from memory into a ring of three (against the kernel below, same conditions:
+        // 13.3 against 15.8 us for N = 1,152, K = 896; 10.4 against 12.2 for 896 x 896; 38.8 against 44.6 for
+        // N = 896, K = 4,864; a ring of two is slower than either when the weights come from memory: 60 us)
+        if (launch_dma<kEpilogue, TO, 1, 1, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
       } else {
         if (launch_tile<kEpilogue, TO, 1, 1, 2, false>(tiles_n, tiles_m, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
       }
