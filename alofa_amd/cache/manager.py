@@ -208,6 +208,12 @@ class CacheManager:
             row_slots.ctypes.data_as(lp), ctypes.c_int64(T)))
         return pos0, positions, req_of_token, tables, row_slots
 
+    def step_width(self, slots: np.ndarray, n_tokens: np.ndarray) -> int:
+        """How many blocks the longest request of a step will hold once the step's tokens are in:
+        the width its block tables need."""
+        ip = ctypes.POINTER(ctypes.c_int)
+        return hostlib.check(self._lib.alofa_cache_step_width(self._h, int(slots.shape[0]), slots.ctypes.data_as(ip), n_tokens.ctypes.data_as(ip)))
+
     def plan_step_into(self, slots: np.ndarray, n_tokens: np.ndarray, max_positions: int, pos0: np.ndarray, positions: np.ndarray,
                        req_of_token: np.ndarray, tables: np.ndarray, row_slots: np.ndarray) -> None:
         """``plan_step`` into arrays the caller keeps (contiguous; tables [groups, n, width])."""

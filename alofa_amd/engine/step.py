@@ -157,6 +157,8 @@ class StepFunction:
         self._scratch: dict = {}
         self._eager_scratch = self._scratch      # buffers of steps that run kernel by kernel
         self._retired: list = []                 # outgrown buffers that captured graphs may still use
+        self._eager_hosts: list = []             # pinned blocks the eager steps are laid out in, taking turns
+        self._eager_turn = 0
         self._identity: dict = {}
         # the last token chosen for the request in each slot, for choices that stay on the device
         self.token_store = torch.zeros(cache.max_requests, dtype=torch.int32, device=self.device)
@@ -247,23 +249,50 @@ class StepFunction:
         entry gets its pages or nothing is changed (capacity error)."""
         slots, n_tokens, ids = self.plan(entries)
         cache = self.cache
-        pos0, positions, req_of_token, tables, row_slots = cache.plan_step(slots, n_tokens, self.n_positions)
+        n, T, G = len(entries), int(n_tokens.sum()), len(cache.groups)
+        want = [(i, int(w)) for i, e in enumerate(entries) for w in e.want]
+        width = cache.step_width(slots, n_tokens)
+        # one pinned block, laid out in place, and one copy that the host does not wait for:
+        # ids, positions, request of every token, wanted rows, block tables (int32); cache slots (int64)
+        n32 = 3 * T + len(want) + G * n * width
+        n32 += n32 % 2
+        nbytes = 4 * n32 + 8 * G * T
+        host = self._eager_host(nbytes)
+        h32, h64 = host["block"][:4 * n32].view(torch.int32).numpy(), host["block"][4 * n32:nbytes].view(torch.int64).numpy()
+        at_rows, at_tables = 3 * T, 3 * T + len(want)
+        pos0 = np.empty(n, dtype=np.int64)
+        cache.plan_step_into(slots, n_tokens, self.n_positions, pos0, h32[T:2 * T], h32[2 * T:3 * T],
+                             h32[at_tables:at_tables + G * n * width].reshape(G, n, width), h64.reshape(G, T))
+        h32[:T] = ids
         spans = self._spans(entries, slots, n_tokens, pos0)
-        T = int(positions.shape[0])
-        want_rows = [s.row0 + int(w) for e, s in zip(entries, spans) for w in e.want]
-        ctx = StepContext(self, spans, positions)
+        if want:
+            h32[at_rows:at_tables] = [spans[i].row0 + w for i, w in want]
+        ctx = StepContext(self, spans, h32[T:2 * T].copy())
         ctx.entry_slots, ctx.entry_tokens = slots, n_tokens
-        n_groups = len(cache.groups)
-        dev = self.device
-        ids_d = torch.from_numpy(ids).to(dev)
-        ctx.positions = torch.from_numpy(positions).to(dev)
-        ctx.req_of_token = torch.from_numpy(req_of_token).to(dev)
-        tables_d = torch.from_numpy(tables).to(dev)
-        slots_d = torch.from_numpy(row_slots).to(dev)
-        ctx._tables = [tables_d[g] for g in range(n_groups)]
-        ctx._slots = [slots_d[g] for g in range(n_groups)]
-        rows = torch.tensor(want_rows, dtype=torch.int32, device=dev) if want_rows else None
+        block = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        block.copy_(host["block"][:nbytes], non_blocking=True)
+        host["copied"].record()
+        d32, d64 = block[:4 * n32].view(torch.int32), block[4 * n32:].view(torch.int64)
+        ids_d, ctx.positions, ctx.req_of_token = d32[:T], d32[T:2 * T], d32[2 * T:3 * T]
+        tables_d, slots_d = d32[at_tables:at_tables + G * n * width].view(G, n, width), d64.view(G, T)
+        ctx._tables = [tables_d[g] for g in range(G)]
+        ctx._slots = [slots_d[g] for g in range(G)]
+        rows = d32[at_rows:at_tables] if want else None
         return ctx, ids_d, rows
+
+    def _eager_host(self, nbytes: int) -> dict:
+        """The pinned block an eager step is laid out in: three take turns (a block is written again
+        only when its last copy has run), and one that is too small is replaced by a bigger one."""
+        ring = self._eager_hosts
+        if len(ring) < 3:
+            ring.append({"block": torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, pin_memory=True), "copied": torch.cuda.Event()})
+            return ring[-1]
+        host = ring[self._eager_turn]
+        self._eager_turn = (self._eager_turn + 1) % len(ring)
+        host["copied"].synchronize()
+        if host["block"].numel() < nbytes:
+            host["block"] = torch.empty(2 * nbytes, dtype=torch.uint8, pin_memory=True)
+        return host
 
     def finish(self, ctx: StepContext) -> None:
         """The step's tokens are written: lengths advance and pages that a window
