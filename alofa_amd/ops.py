@@ -146,7 +146,9 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
     its time grows with M; the tiled kernel's hardly does, but it needs more work
     per block to get going. Measured on one MI355X at the projection sizes of
     0.5B, 7B and 32B models, the tiled kernel wins from these weight sizes on
-    (w_rows * K, in elements): 64 M at 5..8 rows, 24 M at 9..16 rows, 10 M above;
+    (w_rows * K, in elements): 64 M at 5..8 rows, 24 M at 9..16 rows, 8 M above
+    (the gate and up matrices of the 0.5B sizes, 8.7 M: 12.0 against 13.5 us at 32
+    rows, 12.2 against 15.0 at 64; its down matrix, 4.4 M: 18.4 against 13.1);
     and against a matrix as long as a vocabulary (256 column tiles of 128 or more)
     from the first row on."""
     if M > SKINNY_MAX_ROWS:
@@ -160,7 +162,7 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
         return "tiled" if elements >= 64 << 20 else "stream"
     if M <= 16:
         return "tiled" if elements >= 24 << 20 else "stream"
-    return "tiled" if elements >= 10 << 20 else "stream"
+    return "tiled" if elements >= 8 << 20 else "stream"
 
 
 def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int, swiglu: bool = False) -> str:

@@ -550,7 +550,8 @@ def test_product_kernel_choice():
     o = ops()
     assert o.few_rows_kernel(1, 151936, 896) == "tiled" and o.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "stream"
     assert o.few_rows_kernel(4, 4608, 3584) == "stream" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
-    assert o.few_rows_kernel(64, 2 * 4864, 896) == "stream" and o.few_rows_kernel(32, 3584, 3584) == "tiled"
+    assert o.few_rows_kernel(64, 2 * 4864, 896, swiglu=True) == "tiled" and o.few_rows_kernel(16, 2 * 4864, 896, swiglu=True) == "stream"
+    assert o.few_rows_kernel(64, 896, 4864) == "stream" and o.few_rows_kernel(32, 3584, 3584) == "tiled"
     assert o.few_rows_kernel(65, 8, 8) == "tiled"
     a, w = torch.zeros(70, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(16, 64, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(AlofaError):
