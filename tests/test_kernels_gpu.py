@@ -182,12 +182,13 @@ def test_gemm_split_over_blocks_is_repeatable():
     assert int(differing) == 0
 
 
-@pytest.mark.parametrize("M,N,K", [(130, 200, 256), (257, 97, 64), (1100, 1100, 640), (65, 70, 128), (2048, 896, 896), (2050, 2100, 192), (2048, 2176, 64)])
+@pytest.mark.parametrize("M,N,K", [(130, 200, 256), (257, 97, 64), (1100, 1100, 640), (65, 70, 128), (2048, 896, 896), (2050, 2100, 192), (2048, 2176, 64), (1990, 890, 2048)])
 def test_gemm_tiled_with_slabs_straight_into_lds(M, N, K):
     """K a multiple of 64 and not shared out: the forms of the tiled product whose slabs go from
     memory straight into a ring in LDS (rows past M and N are fetched from the last valid row, the
     chunks of a row lie permuted): small tiles with a ring of three, and big tiles with a ring of
-    two where there are one to two of them per compute unit (the last two shapes). Every epilogue
+    two where there are one to two of them per compute unit (the two shapes before the last), tiles
+    of 128 x 64 with a ring of four where those fill the chip once and K is long (the last). Every epilogue
     they have, edges in both directions, one slab and many, and rows that are a strided view."""
     rng = np.random.default_rng(47)
     a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
