@@ -446,7 +446,9 @@ template <int kEpilogue, typename TO, int WTM, int WTN, int S>
 static int launch_dma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
                       hipStream_t stream) {
   const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
-  const int by_die = (static_cast<int64_t>(M) + N) * K * 2 > (32 << 20);
+  // (tiles dealt out die by die at every size: with weights that come from memory it is 3 to 9 % faster here than row
+  // by row also where the operands would fit the L2s: 12.4 against 13.3 us for N = 1,152, K = 896 at 2,048 rows)
+  const int by_die = 1;
   gemm_dma_kernel<kEpilogue, TO, WTM, WTN, S><<<tiles_n * tiles_m, 256, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, bias, M, N, K,
       tiles_m, tiles_n, by_die);
