@@ -44,8 +44,10 @@ class Engine:
         self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), kv_blocks, block_size,
                                   max_requests=max(32, max_batch), device=self.model.rt.device, dtype=self.model.rt.dtype)
         self.step_fn = StepFunction(self.model, self.cache, n_positions=max_tokens)
+        # (pages are counted per request by what the group of layers that holds the most holds: everything,
+        # or, where every layer sees a window only, the window and a step's tokens)
         self.sched_cfg = SchedConfig(token_budget, max_chunk, block_size, kv_blocks, watermark_permille, max_wait_ticks,
-                                     n_slots=max(32, max_batch))
+                                     n_slots=max(32, max_batch), held_tokens=self.cache.held_tokens_bound(max_chunk))
         self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path, share_prefixes=share_prefixes, run_ahead=run_ahead)
         self.seed = seed
         self._next_id = 1

@@ -208,6 +208,17 @@ class CacheManager:
             row_slots.ctypes.data_as(lp), ctypes.c_int64(T)))
         return pos0, positions, req_of_token, tables, row_slots
 
+    def held_tokens_bound(self, step_tokens: int) -> int:
+        """The most tokens a request holds pages for at any time, in the group that holds the most,
+        when a step brings it at most ``step_tokens``: -1 for no bound (some group keeps every key),
+        0 where no group keeps pages at all, else the longest window plus the step plus the two pages
+        that a window's ends may lie in. What the scheduler counts a request's pages by."""
+        if not self.groups:
+            return 0
+        if any(g.window is None for g in self.groups):
+            return -1
+        return max(g.window for g in self.groups) + int(step_tokens) + 2 * self.block_size
+
     def step_width(self, slots: np.ndarray, n_tokens: np.ndarray) -> int:
         """How many blocks the longest request of a step will hold once the step's tokens are in:
         the width its block tables need."""

@@ -148,7 +148,13 @@ constexpr int64_t DIGEST_MOD = 2147483647, DIGEST_MUL = 1000003;
 struct SchedConfig {
   int64_t token_budget, max_chunk, block_size, capacity_blocks, watermark_permille, max_wait_ticks;
   int n_slots;
+  // The most tokens a request holds pages for at any time, in the group of layers that holds the most: below
+  // zero for no bound (a group that keeps every key, the reference's only case), a window's length plus what
+  // a step adds where every group gives back what a window has passed, 0 where no layer keeps pages at all.
+  int64_t held_tokens;
   int64_t threshold() const { return capacity_blocks * watermark_permille / 1000; }
+  // pages a request of this many tokens holds
+  int64_t blocks(int64_t tokens) const { return blocks_for(held_tokens < 0 ? tokens : std::min(tokens, held_tokens), block_size); }
 };
 
 struct Action {
@@ -173,13 +179,13 @@ struct Sched {
   int64_t blocks_held() const {
     int64_t t = 0;
     for (int i = 0; i < cfg.n_slots; ++i)
-      if (state[i] != ST_FREE) t += blocks_for(done[i] + generated[i], cfg.block_size);
+      if (state[i] != ST_FREE) t += cfg.blocks(done[i] + generated[i]);
     return t;
   }
   int64_t blocks_wanted() const {
     int64_t t = 0;
     for (int i = 0; i < cfg.n_slots; ++i)
-      if (state[i] == ST_WAITING) t += std::max<int64_t>(0, blocks_for(prompt_len[i], cfg.block_size) - blocks_for(done[i], cfg.block_size));
+      if (state[i] == ST_WAITING) t += std::max<int64_t>(0, cfg.blocks(prompt_len[i]) - cfg.blocks(done[i]));
     return t;
   }
   int64_t digest() const {
@@ -193,15 +199,15 @@ struct Sched {
   int64_t committed() const {
     int64_t t = 0;
     for (int i = 0; i < cfg.n_slots; ++i)
-      if (state[i] != ST_FREE) t += blocks_for(prompt_len[i] + max_new[i], cfg.block_size);
+      if (state[i] != ST_FREE) t += cfg.blocks(prompt_len[i] + max_new[i]);
     return t;
   }
   int admit(int64_t req, int64_t p_len, int64_t m_new) {
     if (p_len <= 0) return fail(kInvalidArgument, "prompt_len must be positive [request=%lld]", (long long)req);
     if (m_new <= 0) return fail(kInvalidArgument, "max_new must be positive [request=%lld]", (long long)req);
     if (find(req) >= 0) return fail(kInvalidArgument, "duplicate request id [request=%lld]", (long long)req);
-    if (blocks_for(p_len, cfg.block_size) > cfg.capacity_blocks) return fail(kCapacity, "prompt does not fit in the kv pool [request=%lld]", (long long)req);
-    if (committed() + blocks_for(p_len + m_new, cfg.block_size) > cfg.threshold())
+    if (cfg.blocks(p_len) > cfg.capacity_blocks) return fail(kCapacity, "prompt does not fit in the kv pool [request=%lld]", (long long)req);
+    if (committed() + cfg.blocks(p_len + m_new) > cfg.threshold())
       return fail(kCapacity, "concurrent sequences exceed the kv watermark [request=%lld]", (long long)req);
     int slot = -1;
     for (int i = 0; i < cfg.n_slots && slot < 0; ++i)
@@ -213,9 +219,9 @@ struct Sched {
     return 0;
   }
   void release(int slot, bool to_cache) {
-    const int64_t held = blocks_for(done[slot] + generated[slot], cfg.block_size);
+    const int64_t held = cfg.blocks(done[slot] + generated[slot]);
     if (to_cache) {
-      const int64_t whole = blocks_for(prompt_len[slot] + max_new[slot], cfg.block_size);
+      const int64_t whole = cfg.blocks(prompt_len[slot] + max_new[slot]);
       blocks_used += whole - held;
       cached_blocks += whole;
     } else {
@@ -228,7 +234,7 @@ struct Sched {
     for (int i = cfg.n_slots - 1; i >= 0; --i) {
       if (i != protect && state[i] == ST_RUNNING && done[i] + generated[i] > 0) {
         act.preempted.push_back(ids[i]);
-        blocks_used -= blocks_for(done[i] + generated[i], cfg.block_size);
+        blocks_used -= cfg.blocks(done[i] + generated[i]);
         done[i] = generated[i] = wait_ticks[i] = 0;
         ++preempt_count[i];
         ++preempt_total;
@@ -243,7 +249,7 @@ struct Sched {
     const int64_t chunk = std::min({cfg.max_chunk, prompt_len[slot] - done[slot], budget});
     if (chunk <= 0) return budget;
     const int64_t new_done = done[slot] + chunk;
-    const int64_t need = blocks_for(new_done, cfg.block_size) - blocks_for(done[slot], cfg.block_size);
+    const int64_t need = cfg.blocks(new_done) - cfg.blocks(done[slot]);
     if (blocks_used + need > cfg.capacity_blocks) return budget;  // pages ran out: this request waits for a later tick
     act.prefill.insert(act.prefill.end(), {ids[slot], done[slot], new_done});
     blocks_used += need;
@@ -293,7 +299,7 @@ struct Sched {
     for (int i = 0; i < n && budget > 0; ++i) {  // 6
       if (state[i] != ST_RUNNING) continue;
       const int64_t seq = done[i] + generated[i];
-      const int64_t need = blocks_for(seq + 1, cfg.block_size) - blocks_for(seq, cfg.block_size);
+      const int64_t need = cfg.blocks(seq + 1) - cfg.blocks(seq);
       if (need > 0)
         while (blocks_used + need > cfg.capacity_blocks)
           if (!preempt_one(act, i)) return fail(kCapacity, "kv pool too small for this batch");
@@ -560,15 +566,16 @@ int alofa_cache_commit_step(void* cv, int n_entries, const int* slots, const int
 }
 
 // ---- scheduler
-void* alofa_sched_new(const int64_t* cfg7) {
-  return new Sched(SchedConfig{cfg7[0], cfg7[1], cfg7[2], cfg7[3], cfg7[4], cfg7[5], static_cast<int>(cfg7[6])});
+// cfg8: token_budget, max_chunk, block_size, capacity_blocks, watermark_permille, max_wait_ticks, n_slots, held_tokens
+void* alofa_sched_new(const int64_t* cfg8) {
+  return new Sched(SchedConfig{cfg8[0], cfg8[1], cfg8[2], cfg8[3], cfg8[4], cfg8[5], static_cast<int>(cfg8[6]), cfg8[7]});
 }
 void alofa_sched_free(void* s) { delete static_cast<Sched*>(s); }
 // a new configuration for the next ticks (the slot count cannot change)
-int alofa_sched_set_config(void* sv, const int64_t* cfg7) {
+int alofa_sched_set_config(void* sv, const int64_t* cfg8) {
   Sched* s = static_cast<Sched*>(sv);
-  if (cfg7[6] != s->cfg.n_slots) return fail(kInvalidArgument, "the slot count of a scheduler cannot change");
-  s->cfg = SchedConfig{cfg7[0], cfg7[1], cfg7[2], cfg7[3], cfg7[4], cfg7[5], static_cast<int>(cfg7[6])};
+  if (cfg8[6] != s->cfg.n_slots) return fail(kInvalidArgument, "the slot count of a scheduler cannot change");
+  s->cfg = SchedConfig{cfg8[0], cfg8[1], cfg8[2], cfg8[3], cfg8[4], cfg8[5], static_cast<int>(cfg8[6]), cfg8[7]};
   return 0;
 }
 // out: prefill triples, then decode, preempted, finished ids, each at offset k * cap of `out` (4 * cap long);
@@ -591,10 +598,10 @@ int alofa_sched_find(void* s, int64_t req) { return static_cast<Sched*>(s)->find
 int alofa_sched_would_admit(void* sv, int64_t p_len, int64_t m_new, const int64_t* pending, int n_pending) {
   Sched* s = static_cast<Sched*>(sv);
   const SchedConfig& c = s->cfg;
-  if (p_len <= 0 || m_new <= 0 || blocks_for(p_len, c.block_size) > c.capacity_blocks) return 0;
+  if (p_len <= 0 || m_new <= 0 || c.blocks(p_len) > c.capacity_blocks) return 0;
   int64_t committed = s->committed();
-  for (int i = 0; i < n_pending; ++i) committed += blocks_for(pending[2 * i] + pending[2 * i + 1], c.block_size);
-  if (committed + blocks_for(p_len + m_new, c.block_size) > c.threshold()) return 0;
+  for (int i = 0; i < n_pending; ++i) committed += c.blocks(pending[2 * i] + pending[2 * i + 1]);
+  if (committed + c.blocks(p_len + m_new) > c.threshold()) return 0;
   return s->n_live() + n_pending < c.n_slots;
 }
 // which: 0 ids, 1 prompt_len, 2 done, 3 generated, 4 max_new, 5 state, 6 wait_ticks, 7 preempt_count

@@ -36,7 +36,7 @@ import torch
 from .. import ops
 from ..errors import AlofaError
 from ..sampling.sampler import SampleParams, Sampler, SplitMix64
-from .scheduler import Action, SchedConfig, SchedInput, Scheduler, blocks_for
+from .scheduler import Action, SchedConfig, SchedInput, Scheduler
 from .step import TOKEN_ON_DEVICE, StepEntry, StepFunction
 from .trace import config_line, trace_line
 
@@ -110,7 +110,7 @@ class EngineCore:
             raise AlofaError("out_of_range", "token id outside the vocabulary", f"request={req} vocab={vocab}")
         self.requests[req] = Request(req, [int(t) for t in prompt], int(max_new), params or SampleParams(temperature=0.0), int(seed),
                                      rng=SplitMix64(seed))
-        self._charge[req] = blocks_for(len(prompt) + int(max_new), self.sched.cfg.block_size)
+        self._charge[req] = self.sched.cfg.blocks(len(prompt) + int(max_new))
         self._arrivals.append(req)
 
     def can_admit(self, prompt_len: int, max_new: int) -> bool:

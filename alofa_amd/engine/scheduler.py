@@ -45,6 +45,10 @@ class SchedConfig:
     watermark_permille: int = 900
     max_wait_ticks: int = 8
     n_slots: int = 32
+    # The most tokens a request holds pages for at any time, in the group of layers that holds the most (not in
+    # the reference, whose layers all keep every key): below zero for no bound, a window's length plus what a
+    # step adds where every group gives back what its window has passed, 0 where no layer keeps pages.
+    held_tokens: int = -1
 
     def __post_init__(self):
         if self.token_budget < 0 or self.max_chunk <= 0 or self.block_size <= 0 or self.capacity_blocks <= 0:
@@ -55,6 +59,10 @@ class SchedConfig:
     @property
     def threshold_blocks(self) -> int:
         return self.capacity_blocks * self.watermark_permille // 1000
+
+    def blocks(self, tokens: int) -> int:
+        """Pages that a request of ``tokens`` tokens holds (in the group that holds the most)."""
+        return blocks_for(tokens if self.held_tokens < 0 else min(tokens, self.held_tokens), self.block_size)
 
 
 @dataclass
@@ -103,7 +111,7 @@ class Scheduler:
     @staticmethod
     def _cfg_array(cfg: SchedConfig):
         return hostlib.long_array([cfg.token_budget, cfg.max_chunk, cfg.block_size, cfg.capacity_blocks,
-                                   cfg.watermark_permille, cfg.max_wait_ticks, cfg.n_slots])
+                                   cfg.watermark_permille, cfg.max_wait_ticks, cfg.n_slots, cfg.held_tokens])
 
     @property
     def cfg(self) -> SchedConfig:

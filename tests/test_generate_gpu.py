@@ -286,6 +286,36 @@ def test_tight_pool_serves_requests_one_after_another(tiny_dirs):
     assert e.value.name == "capacity"
 
 
+def test_a_model_of_windows_only_is_admitted_by_what_it_holds(tmp_path):
+    """Every layer sees the last 40 keys only, so a request never holds more pages than the
+    window and a step's tokens take: four requests of 200 tokens run side by side in a pool that
+    holds 40 pages of 16 tokens, where their lengths alone would ask for 56, and give the tokens
+    each gives alone (float32: exactly those of the plain implementation)."""
+    from alofa_amd import Engine
+    from alofa_amd.weights import write_random_model
+    cfg = dict(TINY["C"], max_window_layers=0)
+    d = tmp_path / "windows_only"
+    write_random_model(cfg, d, seed=77)
+    prompts = [random_ids(300 + i, 170 + 10 * i, cfg["vocab_size"]) for i in range(4)]
+    want = [plain_greedy(d, p, 24) for p in prompts]
+    eng = Engine(d, dtype="float32", max_tokens=256, max_batch=4, kv_blocks=40, block_size=16, max_chunk=32, token_budget=64)
+    assert eng.sched_cfg.held_tokens == 40 + 32 + 2 * 16 and [g.window for g in eng.cache.groups] == [40]
+    core = eng.core
+    for i, p in enumerate(prompts):
+        core.submit(i + 1, p, 24)
+    side_by_side = 0
+    while core.has_work():
+        core.tick()
+        side_by_side = max(side_by_side, len(core.last_action.decode))
+        assert eng.cache.groups[0].pool.high_water <= 40
+    assert side_by_side == 4
+    assert [core.output(i + 1) for i in range(4)] == want
+    for i in range(4):
+        core.release(i + 1)
+    core.run(10)
+    held_nothing(eng)
+
+
 def test_cancel_and_request_verbs(tiny_dirs):
     from alofa_amd import Engine
     from alofa_amd.errors import AlofaError

@@ -110,6 +110,45 @@ def test_pages_run_out():
     assert e.value.name == "capacity"
 
 
+def test_pages_are_counted_by_what_a_request_holds():
+    """Not in the reference, whose layers all keep every key: where every group of layers gives back
+    what a window has passed, a request is counted by the window and a step's tokens, not by its
+    length; where no layer keeps pages, by nothing. The default (no bound) is the reference's count."""
+    long_ones = [(1, 200, 50), (2, 200, 50), (3, 200, 50)]
+    # the reference's count: a prompt of 50 pages does not fit a pool of 24
+    s = Scheduler(SchedConfig(token_budget=64, max_chunk=16, block_size=4, capacity_blocks=24, watermark_permille=1000))
+    with pytest.raises(AlofaError) as e:
+        s.step(SchedInput(arrivals=long_ones[:1]))
+    assert e.value.name == "capacity" and "does not fit" in str(e.value)
+    # at most 28 tokens held (a window of 4, a step of 16, two pages): 7 pages each, three fit in 24 and run side by side
+    cfg = SchedConfig(token_budget=64, max_chunk=16, block_size=4, capacity_blocks=24, watermark_permille=1000, held_tokens=28)
+    assert cfg.blocks(10) == 3 and cfg.blocks(28) == 7 and cfg.blocks(250) == 7
+    s = Scheduler(cfg)
+    a = s.step(SchedInput(arrivals=long_ones))
+    assert a.prefill == [(1, 0, 16), (2, 0, 16), (3, 0, 16)]
+    peak, finished, ticks = 0, [], 0
+    while s.n_live() and ticks < 400:
+        a = s.step(SchedInput())
+        ticks += 1
+        peak = max(peak, s.blocks_used)
+        finished += a.finished
+        assert s.blocks_used == s.blocks_held() + s.cached_blocks <= 24 and a.preempted == []
+    assert sorted(finished) == [1, 2, 3] and peak == 21 and s.cached_blocks == 21
+    assert s.step(SchedInput(freed_blocks=21)).tick_seq == ticks + 2 and s.blocks_used == 0
+    # a fourth would pass the watermark: refused by name, as ever
+    s = Scheduler(cfg)
+    with pytest.raises(AlofaError) as e:
+        s.step(SchedInput(arrivals=long_ones + [(4, 200, 50)]))
+    assert e.value.name == "capacity" and "watermark" in str(e.value)
+    # no layer keeps pages: the pool is never what refuses
+    s = Scheduler(SchedConfig(token_budget=64, max_chunk=16, block_size=4, capacity_blocks=1, watermark_permille=1000, held_tokens=0, n_slots=8))
+    a = s.step(SchedInput(arrivals=[(i, 1000, 10) for i in range(1, 9)]))
+    assert len(a.prefill) == 4 and s.blocks_used == 0       # the token budget cuts, not the pages
+    with pytest.raises(AlofaError) as e:
+        s.step(SchedInput(arrivals=[(9, 5, 5)]))
+    assert "scheduler is full" in str(e.value)
+
+
 def test_cancel_blocks_arrival_in_the_same_tick_and_refusals_are_named():
     s = Scheduler(SchedConfig())
     a = s.step(SchedInput(arrivals=[(7, 5, 2)], cancelled=[7]))
