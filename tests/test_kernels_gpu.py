@@ -305,6 +305,47 @@ def paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, dtype, scale_key=None)
                 qcat=t(np.concatenate(qs), dtype))
 
 
+def test_exact_attention_on_the_reference_paged_vectors():
+    """The reference's eleven paged-attention cases (tests/fixtures/paged/ there; its own test
+    compares at one part in 1e5, tests/unit/test_paged_attention.mojo:66-70) as one batch of eleven
+    requests through the float32 kernel: their gathered keys and values laid out in this engine's
+    pages (whole pages of 16 slots in shuffled order, values transposed), the queries at the last
+    positions; and its wrong-head-mapping control must not match."""
+    from conftest import FIXTURES
+    d_ = FIXTURES / "paged"
+    floats = lambda f: np.array([float(x) for x in (d_ / f).read_text().split()], dtype=np.float32)      # noqa: E731
+    cfg = dict(l.split("\t") for l in (d_ / "config.tsv").read_text().splitlines())
+    bs, cols, H, Hkv, hd = (int(cfg[k]) for k in ("block_size", "kv_cols", "n_heads", "n_kv_heads", "head_dim"))
+    cases = [l.split("\t") for l in (d_ / "cases.tsv").read_text().splitlines() if not l.startswith("#")]
+    rng = np.random.default_rng(5)
+    ks, vs, qs, wants = [], [], [], []
+    for name, _s, _r, _o, q_len, _n, *_runs in cases:
+        kv = floats(f"{name}.kv.tsv")
+        L = kv.size // (2 * cols)
+        ks.append(kv[:L * cols].reshape(L, cols)), vs.append(kv[L * cols:].reshape(L, cols))
+        qs.append(floats(f"{name}.q.tsv").reshape(int(q_len), H * hd)), wants.append(floats(f"{name}.y.tsv").reshape(int(q_len), H * hd))
+    per = [(k.shape[0] + bs - 1) // bs for k in ks]
+    order = rng.permutation(sum(per) + 2)
+    kc = np.full((sum(per) + 2, Hkv, bs, hd), np.nan, np.float32)
+    vc = np.full_like(kc, np.nan)
+    table = np.full((len(cases), max(per)), -1, np.int32)
+    pos, req, used = [], [], 0
+    for r, (k, v, q) in enumerate(zip(ks, vs, qs)):
+        table[r, :per[r]] = order[used:used + per[r]]
+        used += per[r]
+        for p_ in range(k.shape[0]):
+            kc[table[r, p_ // bs], :, p_ % bs] = k[p_].reshape(Hkv, hd)
+            vc[table[r, p_ // bs], :, p_ % bs] = v[p_].reshape(Hkv, hd)
+        pos.extend(range(k.shape[0] - q.shape[0], k.shape[0])), req.extend([r] * q.shape[0])
+    out = torch.empty(len(pos), H * hd, device=DEV)
+    ops().paged_attention(out, t(np.concatenate(qs)), t(kc), t(vc.transpose(0, 1, 3, 2)), t(table, torch.int32), t(np.array(req, np.int32), torch.int32),
+                          t(np.array(pos, np.int32), torch.int32), H, Hkv, hd, None, float(np.float32(1) / np.sqrt(np.float32(hd))), True)
+    want = np.concatenate(wants)
+    close(out, want, 1e-5, "the reference's paged vectors")
+    wrong = floats("expected_hmap.tsv").reshape(wants[0].shape)
+    assert np.abs(out[:wrong.shape[0]].cpu().numpy() - wrong).max() > 1e-3
+
+
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 80, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16)])
 @pytest.mark.parametrize("dtype,exact", [(torch.float32, True), (torch.bfloat16, False)])
 @pytest.mark.parametrize("window", [None, 21])

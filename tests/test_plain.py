@@ -65,6 +65,42 @@ def test_attention_vector(l0):
     assert not close(pm.attention(l0["q_rot"], kk, vv, 14, 14, 64), l0["attn_out"])
 
 
+def _floats(path):
+    return np.array([float(x) for x in path.read_text().split()], dtype=np.float32)
+
+
+def test_attention_vectors_through_page_tables():
+    """The reference's paged-attention vectors (tests/fixtures/paged/ there, written by an
+    independent implementation, scripts/dump_paged_reference.py:116-160; used by
+    tests/unit/test_paged_attention.mojo:48-70 at one part in 1e5): a cache of 4 blocks x 16 slots,
+    4 query heads on 2 key heads of size 8, eleven cases whose keys and values are gathered through
+    tables of (block, first slot, length) runs, some starting in the middle of a block; the queries
+    are the last q_len positions. Both of its exported negative controls must fail: the first
+    expected value moved by 0.05, and query head h mapped to key head h % 2 instead of h // 2."""
+    d = FIXTURES / "paged"
+    cfg = dict(l.split("\t") for l in (d / "config.tsv").read_text().splitlines())
+    bs, cols, H, Hkv, hd = (int(cfg[k]) for k in ("block_size", "kv_cols", "n_heads", "n_kv_heads", "head_dim"))
+    kc = _floats(d / "k_cache.tsv").reshape(-1, bs, cols)
+    vc = _floats(d / "v_cache.tsv").reshape(-1, bs, cols)
+    assert kc.shape[0] == int(cfg["n_blocks"])
+    cases = [l.split("\t") for l in (d / "cases.tsv").read_text().splitlines() if not l.startswith("#")]
+    assert len(cases) == int(cfg["n_cases"]) and sum(c[1] == "-" for c in cases) == 3
+    first = None
+    for name, _scenario, _req, _ops, q_len, n_entries, *runs in cases:
+        q_len, runs = int(q_len), [tuple(int(x) for x in runs[3 * i:3 * i + 3]) for i in range(int(n_entries))]
+        k = np.concatenate([kc[b, s:s + n] for b, s, n in runs])
+        v = np.concatenate([vc[b, s:s + n] for b, s, n in runs])
+        assert np.array_equal(np.concatenate([k.ravel(), v.ravel()]), _floats(d / f"{name}.kv.tsv")), name      # the gather itself
+        q, want = _floats(d / f"{name}.q.tsv").reshape(q_len, H * hd), _floats(d / f"{name}.y.tsv").reshape(q_len, H * hd)
+        got = pm.attention(q, k, v, H, Hkv, hd)
+        assert np.abs(got - want).max() <= 1e-5 * max(1.0, np.abs(want).max()), name
+        first = first or (got, want)
+    got, want = first
+    for control in ("expected_bad.tsv", "expected_hmap.tsv"):
+        wrong = _floats(d / control).reshape(want.shape)
+        assert np.abs(got - wrong).max() > 1e-3 * max(1.0, np.abs(want).max()), control
+
+
 def test_residual_and_activation_vectors(l0):
     assert close(pm.add(l0["embed_out"], l0["o_out"]), l0["hidden1"])
     assert close(pm.silu(l0["gate_out"]), l0["silu_out"])
