@@ -29,7 +29,10 @@ __global__ void embed_gather_kernel(float* __restrict__ out, const TW* __restric
 // ---- RMSNorm ---------------------------------------------------------------
 // y = x * 1/sqrt(mean(x^2) + eps) * w per row; row r of the output is made from
 // row rows[r] of x when `rows` is given. x is the float residual stream.
-template <typename TO, typename Acc>
+// K4 > 0: the row (a multiple of four wide, at most 1,024 K4 values, 16-byte aligned) stays in registers as K4
+// groups of four per thread between the sum of its squares and the scaling, and its weights are on their way
+// meanwhile; K4 = 0: any row, read twice.
+template <typename TO, typename Acc, int K4>
 __global__ void __launch_bounds__(256) rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x,
                                                       const float* __restrict__ w,
                                                       const int32_t* __restrict__ rows, int width, float eps) {
@@ -37,29 +40,35 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(TO* __restrict__ out, cons
   const int r = blockIdx.x;
   const float* src = x + static_cast<int64_t>(rows ? rows[r] : r) * width;
   TO* dst = out + static_cast<int64_t>(r) * width;
-  // rows of up to 256 * kKeep values stay in registers between the two passes, and their weights are on
-  // their way while the squares are summed; wider rows are read twice
-  constexpr int kKeep = 8;
-  if (width <= 256 * kKeep) {
-    float xs[kKeep], ws[kKeep];
+  if constexpr (K4 > 0) {
+    float4 xs[K4], ws[K4];
+    const int groups = width / 4;
+#pragma unroll
+    for (int i = 0; i < K4; ++i) {
+      const int g = threadIdx.x + 256 * i;
+      xs[i] = g < groups ? reinterpret_cast<const float4*>(src)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+      ws[i] = g < groups ? reinterpret_cast<const float4*>(w)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     Acc ss = 0;
 #pragma unroll
-    for (int i = 0; i < kKeep; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      xs[i] = c < width ? src[c] : 0.f;
-      ws[i] = c < width ? w[c] : 0.f;
-    }
-#pragma unroll
-    for (int i = 0; i < kKeep; ++i) {      // ascending c, as the strided loop below
-      const Acc v = static_cast<Acc>(xs[i]);
-      ss += v * v;
+    for (int i = 0; i < K4; ++i) {      // ascending columns within the thread
+      const Acc a = static_cast<Acc>(xs[i].x), b = static_cast<Acc>(xs[i].y), c = static_cast<Acc>(xs[i].z), d = static_cast<Acc>(xs[i].w);
+      ss += a * a;
+      ss += b * b;
+      ss += c * c;
+      ss += d * d;
     }
     ss = block_sum<Acc, 256>(ss, scratch);
     const Acc scale = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(width) + static_cast<Acc>(eps));
 #pragma unroll
-    for (int i = 0; i < kKeep; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      if (c < width) store_f32(dst + c, static_cast<float>(static_cast<Acc>(xs[i]) * scale * static_cast<Acc>(ws[i])));
+    for (int i = 0; i < K4; ++i) {
+      const int g = threadIdx.x + 256 * i;
+      if (g < groups) {
+        store_f32(dst + 4 * g + 0, static_cast<float>(static_cast<Acc>(xs[i].x) * scale * static_cast<Acc>(ws[i].x)));
+        store_f32(dst + 4 * g + 1, static_cast<float>(static_cast<Acc>(xs[i].y) * scale * static_cast<Acc>(ws[i].y)));
+        store_f32(dst + 4 * g + 2, static_cast<float>(static_cast<Acc>(xs[i].z) * scale * static_cast<Acc>(ws[i].z)));
+        store_f32(dst + 4 * g + 3, static_cast<float>(static_cast<Acc>(xs[i].w) * scale * static_cast<Acc>(ws[i].w)));
+      }
     }
     return;
   }
@@ -231,14 +240,27 @@ extern "C" int alofa_embed_gather(float* out, const void* table, int table_dtype
 extern "C" int alofa_rmsnorm(void* out, int out_dtype, const float* x, const float* w, const int32_t* rows,
                              int n_rows, int width, float eps, int exact, hipStream_t stream) {
   ALOFA_REQUIRE(n_rows > 0 && width > 0, "rmsnorm: rows=%d width=%d must be positive", n_rows, width);
-  if (out_dtype == kF32 && exact)
-    rmsnorm_kernel<float, double><<<n_rows, 256, 0, stream>>>(static_cast<float*>(out), x, w, rows, width, eps);
-  else if (out_dtype == kF32)
-    rmsnorm_kernel<float, float><<<n_rows, 256, 0, stream>>>(static_cast<float*>(out), x, w, rows, width, eps);
-  else if (out_dtype == kBF16 && !exact)
-    rmsnorm_kernel<bf16_t, float><<<n_rows, 256, 0, stream>>>(static_cast<bf16_t*>(out), x, w, rows, width, eps);
-  else
+  // rows that stay in registers: up to 8,192 wide, a multiple of four, 16-byte aligned (x rows, w and width * 4 bytes)
+  const bool vec = width % 4 == 0 && width <= 8192 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
+  const int k4 = !vec ? 0 : width <= 1024 ? 1 : width <= 2048 ? 2 : width <= 4096 ? 4 : 8;
+#define ALOFA_RMSNORM(TO, ACC)                                                                                                   \
+  switch (k4) {                                                                                                                   \
+    case 1: rmsnorm_kernel<TO, ACC, 1><<<n_rows, 256, 0, stream>>>(static_cast<TO*>(out), x, w, rows, width, eps); break;         \
+    case 2: rmsnorm_kernel<TO, ACC, 2><<<n_rows, 256, 0, stream>>>(static_cast<TO*>(out), x, w, rows, width, eps); break;         \
+    case 4: rmsnorm_kernel<TO, ACC, 4><<<n_rows, 256, 0, stream>>>(static_cast<TO*>(out), x, w, rows, width, eps); break;         \
+    case 8: rmsnorm_kernel<TO, ACC, 8><<<n_rows, 256, 0, stream>>>(static_cast<TO*>(out), x, w, rows, width, eps); break;         \
+    default: rmsnorm_kernel<TO, ACC, 0><<<n_rows, 256, 0, stream>>>(static_cast<TO*>(out), x, w, rows, width, eps);               \
+  }
+  if (out_dtype == kF32 && exact) {
+    ALOFA_RMSNORM(float, double)
+  } else if (out_dtype == kF32) {
+    ALOFA_RMSNORM(float, float)
+  } else if (out_dtype == kBF16 && !exact) {
+    ALOFA_RMSNORM(bf16_t, float)
+  } else {
     ALOFA_REQUIRE(false, "rmsnorm: unsupported out dtype %d with exact=%d", out_dtype, exact);
+  }
+#undef ALOFA_RMSNORM
   return check_launch("rmsnorm");
 }
 

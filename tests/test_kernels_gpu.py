@@ -48,7 +48,7 @@ def test_embed_gather(dtype):
     assert np.array_equal(out.cpu().numpy(), pm.embed(table, ids))
 
 
-@pytest.mark.parametrize("width", [80, 896, 1000])
+@pytest.mark.parametrize("width", [80, 896, 1000, 1026, 2044, 3584, 5120, 8192, 9000])     # rows kept in registers (multiples of four up to 8,192) and rows read twice
 def test_rmsnorm(width):
     rng = np.random.default_rng(1)
     x = (rng.standard_normal((9, width)) * 3).astype(np.float32)
