@@ -155,6 +155,11 @@ int check_launch(const char* what);
 
 }  // namespace alofa
 
+// (sampling.hip) the last stage of an argmax over candidates that another kernel left
+extern "C" int alofa_argmax_parts(int32_t* out, int32_t* store, const int32_t* store_index, const float* part_v,
+                                  const int32_t* part_i, int rows, int n_parts, int vocab, hipStream_t stream);
+
+
 #define ALOFA_REQUIRE(cond, ...)          \
   do {                                    \
     if (!(cond)) {                        \

@@ -31,7 +31,7 @@ namespace alofa {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-enum MfmaEpilogue : int { kMfStore = 0, kMfResidual = 1, kMfSwiglu = 2 };
+enum MfmaEpilogue : int { kMfStore = 0, kMfResidual = 1, kMfSwiglu = 2, kMfArgmax = 3 };
 
 constexpr int TK = 64, PAD = 8;
 constexpr int kRow = TK + PAD;  // LDS row length in elements
@@ -58,6 +58,42 @@ __device__ __forceinline__ TilePlace place_tile(int block, int tiles_m, int tile
   const int per_group = kGroup * tiles_n, first_m = (t / per_group) * kGroup, within = t % per_group;
   const int rows = min(tiles_m - first_m, kGroup);
   return {first_m + within % rows, within / rows, step / tiles};
+}
+
+// Instead of the outputs, a wave leaves per row the highest of its columns and that column's number (the lowest
+// among equals): candidate 2 bn + wn of `parts` per row, values at out[m * parts + ..], column numbers as int32
+// behind the M * parts values. A column past N is no candidate (its number reads as INT_MAX).
+template <int WTM, int WTN>
+__device__ __forceinline__ void tile_argmax(f32x16 (&acc)[WTM][WTN], float* __restrict__ out, int parts, int M, int N, int m0, int n0,
+                                            int bn, int wm, int wn, int lane) {
+  const int col = lane % 32, half = lane / 32;
+  int32_t* numbers = reinterpret_cast<int32_t*>(out + static_cast<int64_t>(M) * parts);
+#pragma unroll
+  for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      if (m0 + wm * 32 * WTM + i * 32 + 8 * (e / 4) >= M) continue;     // (uniform over the wave) rows past M: with 8 rows, 4 of a wave's 16 registers count
+      float bv = -3.402823466e+38f;
+      int bi = 0x7fffffff;
+#pragma unroll
+      for (int j = 0; j < WTN; ++j) {      // ascending columns: an equal value further right does not take over
+        const int n = n0 + wn * 32 * WTN + j * 32 + col;
+        const float v = acc[i][j][e];
+        if (n < N && v > bv) { bv = v; bi = n; }
+      }
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) {     // the 32 lanes that hold this row's columns
+        const float ov = __shfl_xor(bv, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+      }
+      const int m = m0 + wm * 32 * WTM + i * 32 + 8 * (e / 4) + 4 * half + e % 4;
+      if (col == 0 && m < M) {
+        out[static_cast<int64_t>(m) * parts + 2 * bn + wn] = bv;
+        numbers[static_cast<int64_t>(m) * parts + 2 * bn + wn] = bi;
+      }
+    }
+  }
 }
 
 // What a wave does with its finished tiles (WTM x WTN of 32 x 32, the block's tile at m0, n0 of the output).
@@ -294,7 +330,12 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
       }
   }
 
-  tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out, ldo, bias, M, N, m0, n0, wm, wn, lane);
+  if constexpr (kEpilogue == kMfArgmax) {
+    tile_argmax<WTM, WTN>(acc, out, static_cast<int>(ldo), M, N, m0, n0, place.bn, wm, wn, lane);
+    return;
+  } else {
+    tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out, ldo, bias, M, N, m0, n0, wm, wn, lane);
+  }
 }
 
 // The same product with the slabs brought from memory straight into LDS (global_load_lds_dwordx4: every lane's
@@ -547,4 +588,22 @@ extern "C" int alofa_gemm_mfma(void* out, int o_dtype, int64_t ldo, const void* 
     return launch_mfma<kMfSwiglu, bf16_t>(out, ldo, A, lda, W, W2, ldw, nullptr, M, N, K, stream);
   }
   ALOFA_REQUIRE(false, "gemm_mfma: unsupported epilogue %d with out dtype %d", epilogue, o_dtype);
+}
+
+// out[m] = the column n with the highest sum_k A[m, k] * W[n, k] (the lowest n among equals), for M <= 64 rows
+// against a long matrix: the product's blocks leave candidates instead of the M x N outputs (scratch: at least
+// 4 * M * ceil(N / 128) floats), a second kernel takes the best of them; store and store_index as for
+// alofa_argmax_to_store (both null: no store).
+extern "C" int alofa_gemm_argmax(int32_t* out, int32_t* store, const int32_t* store_index, float* scratch, int64_t scratch_floats,
+                                 const void* A, int64_t lda, const void* W, int64_t ldw, int M, int N, int K, hipStream_t stream) {
+  ALOFA_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_argmax: M=%d (1..64) N=%d K=%d", M, N, K);
+  ALOFA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K, "gemm_argmax: K=%d, lda=%lld, ldw=%lld must be multiples of 8 and cover K", K,
+                static_cast<long long>(lda), static_cast<long long>(ldw));
+  ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0, "gemm_argmax: operands must be 16-byte aligned");
+  const int tiles_n = (N + 127) / 128, parts = 2 * tiles_n;
+  ALOFA_REQUIRE(out != nullptr && scratch != nullptr && scratch_floats >= 2ll * M * parts, "gemm_argmax: the scratch holds %lld floats, %lld are needed",
+                static_cast<long long>(scratch_floats), 2ll * M * parts);
+  if (launch_tile<kMfArgmax, float, 1, 2, 2, false>(tiles_n, 1, 1, scratch, parts, A, lda, W, nullptr, ldw, nullptr, M, N, K, stream)) return 1;
+  if (check_launch("gemm_argmax")) return 1;
+  return alofa_argmax_parts(out, store, store_index, scratch, reinterpret_cast<const int32_t*>(scratch + static_cast<int64_t>(M) * parts), M, parts, N, stream);
 }

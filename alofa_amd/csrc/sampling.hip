@@ -102,6 +102,35 @@ __global__ void __launch_bounds__(kWave) argmax_final_kernel(Choice choice, cons
   if (threadIdx.x == 0) choice.put(r, bi < vocab ? bi : 0);
 }
 
+// The same last stage over any number of candidates per row (value and index each, indices ascending with the
+// candidate's number or not): the highest value, the lowest index among equals. For candidates that the
+// vocabulary product leaves instead of logits.
+__global__ void __launch_bounds__(256) argmax_parts_kernel(Choice choice, const float* __restrict__ part_v,
+                                                           const int32_t* __restrict__ part_i, int n_parts, int vocab) {
+  __shared__ float best_v[4];
+  __shared__ int best_i[4];
+  const int r = blockIdx.x;
+  float bv = -FLT_MAX;
+  int bi = vocab;
+  for (int p = threadIdx.x; p < n_parts; p += 256) {
+    const float v = part_v[static_cast<int64_t>(r) * n_parts + p];
+    const int i = part_i[static_cast<int64_t>(r) * n_parts + p];
+    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+  }
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, kWave);
+    const int oi = __shfl_xor(bi, off, kWave);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  if (threadIdx.x % kWave == 0) { best_v[threadIdx.x / kWave] = bv; best_i[threadIdx.x / kWave] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w)
+      if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
+    choice.put(r, bi < vocab ? bi : 0);
+  }
+}
+
 __global__ void __launch_bounds__(kPickThreads) sample_kernel(Choice choice, const float* __restrict__ logits,
                                                               int64_t stride, int vocab,
                                                               const double* __restrict__ temperature,
@@ -233,6 +262,18 @@ extern "C" int alofa_argmax_no_alloc(int32_t* out, const float* logits, int64_t 
   if (check_launch("argmax_chunk")) return 1;
   argmax_final_kernel<<<rows, kWave, 0, stream>>>(Choice{out, nullptr, nullptr}, part_v, part_i, vocab);
   return check_launch("argmax_final");
+}
+
+// out[r] = the index of the highest of row r's n_parts candidates (part_v, part_i: [rows, n_parts]; an index of
+// `vocab` or more stands for "none"), the lowest index among equal values; store and store_index both null or
+// as for alofa_argmax_to_store.
+extern "C" int alofa_argmax_parts(int32_t* out, int32_t* store, const int32_t* store_index, const float* part_v,
+                                  const int32_t* part_i, int rows, int n_parts, int vocab, hipStream_t stream) {
+  ALOFA_REQUIRE(out != nullptr && part_v != nullptr && part_i != nullptr && rows > 0 && n_parts > 0 && vocab > 0,
+                "argmax_parts: rows=%d parts=%d vocab=%d", rows, n_parts, vocab);
+  ALOFA_REQUIRE((store == nullptr) == (store_index == nullptr), "argmax_parts: a store goes with its index");
+  argmax_parts_kernel<<<rows, 256, 0, stream>>>(Choice{out, store, store_index}, part_v, part_i, n_parts, vocab);
+  return check_launch("argmax_parts");
 }
 
 // store and store_index: both null, or as for alofa_argmax_to_store

@@ -258,14 +258,27 @@ class EngineCore:
                              **views(mirror, False)}
         return self._staging
 
-    def choose(self, logits: torch.Tensor, owes: list) -> Optional[list]:
-        """One token per row of ``logits``, for the requests in ``owes`` (in order). Requests that
+    def choose(self, logits: Optional[torch.Tensor], owes: list, by_step: Optional[torch.Tensor] = None) -> Optional[list]:
+        """One token per row of ``logits``, for the requests in ``owes`` (in order); or, with
+        ``by_step`` (int32 on the device, what a step that chose greedily by itself returned, the
+        token store already written), only their way to the host. Requests that
         sample plainly (greedy, or temperature alone) choose on the device; the tokens go to the
         token store and set out for the host, and None is returned: ``collect`` reads them later.
         With a request that needs the host's chain the whole tick is synchronous and the tokens
         are returned."""
         reqs = [self.requests[o] for o in owes]
         n = len(reqs)
+        if by_step is not None:
+            st = self._stage()
+            turn = st["turns"][st["turn"]]
+            st["turn"] = (st["turn"] + 1) % len(st["turns"])
+            turn["event"].synchronize()                          # this block's last use (three ticks ago) is over
+            turn["down"][:n].copy_(by_step[:n], non_blocking=True)
+            turn["event"].record()
+            for r in reqs:
+                r.on_device = True
+            self._inflight.append(([(r.id, r.preemptions) for r in reqs], turn["tokens"], n, turn["event"]))
+            return None
         host = [i for i, r in enumerate(reqs) if not r.params.plain]
         greedy = [i for i, r in enumerate(reqs) if r.params.plain and r_is_greedy(r)]
         drawn = [i for i, r in enumerate(reqs) if r.params.plain and not r_is_greedy(r)]
@@ -367,9 +380,12 @@ class EngineCore:
         self.ticks += 1
         self.last_rows = sum(len(e.tokens) for e in entries)
         if entries:
-            logits = self.fn.run(entries)
             wanted = [o for o in owes if o is not None]
-            chosen = self.choose(logits, wanted) if wanted else []
+            # where every request that is owed a token takes the first maximum, the step chooses by itself
+            # (the vocabulary product leaves no logits then)
+            by_step = bool(wanted) and all(self.requests[o].params.plain and r_is_greedy(self.requests[o]) for o in wanted)
+            result = self.fn.run(entries, greedy=by_step)
+            chosen = (self.choose(None, wanted, result) if by_step else self.choose(result, wanted)) if wanted else []
             self.settle(owes, chosen)
             self.collect(keep=1 if self.run_ahead else 0)
         else:

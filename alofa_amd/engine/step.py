@@ -89,6 +89,7 @@ class StepContext:
         self._memo: dict = {}
         self.token_store = fn.token_store
         self.request_slots: Optional[torch.Tensor] = None   # int32 [entries] on the device, where the step keeps them there (decode graphs)
+        self.want_slots: Optional[torch.Tensor] = None      # int32 [wanted rows] on the device: the request slot behind every wanted row
 
     @property
     def device(self):
@@ -162,6 +163,7 @@ class StepFunction:
         self._identity: dict = {}
         # the last token chosen for the request in each slot, for choices that stay on the device
         self.token_store = torch.zeros(cache.max_requests, dtype=torch.int32, device=self.device)
+        self._chosen = torch.empty(cache.max_requests, dtype=torch.int32, device=self.device)   # what a step that chooses greedily returns
         self.cache_owner = model.cache_owners()      # (entry, k) -> the key of the cache that mixer uses
         self.steps_run = 0
         self.rows_run = 0
@@ -253,20 +255,21 @@ class StepFunction:
         want = [(i, int(w)) for i, e in enumerate(entries) for w in e.want]
         width = cache.step_width(slots, n_tokens)
         # one pinned block, laid out in place, and one copy that the host does not wait for:
-        # ids, positions, request of every token, wanted rows, block tables (int32); cache slots (int64)
-        n32 = 3 * T + len(want) + G * n * width
+        # ids, positions, request of every token, wanted rows and their requests' slots, block tables (int32); cache slots (int64)
+        n32 = 3 * T + 2 * len(want) + G * n * width
         n32 += n32 % 2
         nbytes = 4 * n32 + 8 * G * T
         host = self._eager_host(nbytes)
         h32, h64 = host["block"][:4 * n32].view(torch.int32).numpy(), host["block"][4 * n32:nbytes].view(torch.int64).numpy()
-        at_rows, at_tables = 3 * T, 3 * T + len(want)
+        at_rows, at_tables = 3 * T, 3 * T + 2 * len(want)
         pos0 = np.empty(n, dtype=np.int64)
         cache.plan_step_into(slots, n_tokens, self.n_positions, pos0, h32[T:2 * T], h32[2 * T:3 * T],
                              h32[at_tables:at_tables + G * n * width].reshape(G, n, width), h64.reshape(G, T))
         h32[:T] = ids
         spans = self._spans(entries, slots, n_tokens, pos0)
         if want:
-            h32[at_rows:at_tables] = [spans[i].row0 + w for i, w in want]
+            h32[at_rows:at_rows + len(want)] = [spans[i].row0 + w for i, w in want]
+            h32[at_rows + len(want):at_tables] = [slots[i] for i, _ in want]      # the requests' places in the token store
         ctx = StepContext(self, spans, h32[T:2 * T].copy())
         ctx.entry_slots, ctx.entry_tokens = slots, n_tokens
         block = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
@@ -277,7 +280,8 @@ class StepFunction:
         tables_d, slots_d = d32[at_tables:at_tables + G * n * width].view(G, n, width), d64.view(G, T)
         ctx._tables = [tables_d[g] for g in range(G)]
         ctx._slots = [slots_d[g] for g in range(G)]
-        rows = d32[at_rows:at_tables] if want else None
+        rows = d32[at_rows:at_rows + len(want)] if want else None
+        ctx.want_slots = d32[at_rows + len(want):at_tables] if want else None
         return ctx, ids_d, rows
 
     def _eager_host(self, nbytes: int) -> dict:
@@ -329,7 +333,7 @@ class StepFunction:
             self._graph_buffers[B] = buf
         return self._graph_buffers[B]
 
-    def _run_decode_graph(self, entries: list) -> torch.Tensor:
+    def _run_decode_graph(self, entries: list, greedy: bool = False) -> torch.Tensor:
         slots, n_tokens, ids = self.plan(entries)
         cache = self.cache
         B = len(entries)
@@ -351,14 +355,22 @@ class StepFunction:
         ctx._slots = [buf["slots"][g] for g in range(len(cache.groups))]
         buf["dev"].copy_(host["block"], non_blocking=True)
         host["copied"].record()
-        key = (B, ctx.max_context)
+        ctx.want_slots = buf["request_slots"]
+        key = (B, ctx.max_context, greedy)
         saved, self._scratch = self._scratch, buf["scratch"]   # graphs of one batch size share their own buffers
+        chosen = self._chosen[:B]
+
+        def outcome(hidden):      # logits of every row, or (greedy) only each row's first maximum, which also goes to the token store
+            if greedy:
+                self.model.greedy(ctx, hidden, buf["rows"], chosen, self.token_store, buf["request_slots"])
+                return chosen
+            return self.model.logits(ctx, hidden, buf["rows"])
         try:
             if key not in self._graphs:
                 # once eagerly, so that every buffer exists before the capture and the
                 # step's result does not depend on the capture itself
                 hidden = self.model.forward(ctx, buf["ids"])
-                logits = self.model.logits(ctx, hidden, buf["rows"])
+                logits = outcome(hidden)
                 torch.cuda.current_stream().synchronize()
                 graph = torch.cuda.CUDAGraph()
                 # No garbage collection while the stream is capturing: a collected object that owns device
@@ -372,7 +384,7 @@ class StepFunction:
                 try:
                     with torch.cuda.graph(graph), ops.stream_scope():
                         hidden = self.model.forward(ctx, buf["ids"])
-                        captured = self.model.logits(ctx, hidden, buf["rows"])
+                        captured = outcome(hidden)
                 finally:
                     if collecting:
                         gc.enable()
@@ -390,16 +402,24 @@ class StepFunction:
         self.last_context = ctx
         return logits
 
-    def run(self, entries: list) -> Optional[torch.Tensor]:
+    def run(self, entries: list, greedy: bool = False) -> Optional[torch.Tensor]:
         """Run the step. Returns float32 logits [wanted, vocab] on the device in
         the order of the entries and of their ``want`` lists, or None when nothing
-        is wanted. The buffer is re-used by the next step."""
+        is wanted. With ``greedy`` the step chooses by itself: it returns, instead of
+        the logits, int32 [wanted] with the first index of every wanted row's highest
+        logit, and leaves the same in the token store at the row's request's slot.
+        The buffer is re-used by the next step."""
         with ops.stream_scope():
             if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
-                return self._run_decode_graph(entries)
+                return self._run_decode_graph(entries, greedy)
             ctx, ids, rows = self.begin(entries)
             hidden = self.model.forward(ctx, ids)
-            logits = self.model.logits(ctx, hidden, rows) if rows is not None else None
+            out = None
+            if rows is not None and greedy:
+                out = self._chosen[:rows.shape[0]]
+                self.model.greedy(ctx, hidden, rows, out, self.token_store, ctx.want_slots)
+            elif rows is not None:
+                out = self.model.logits(ctx, hidden, rows)
             self.finish(ctx)
             self.last_context = ctx
-            return logits
+            return out

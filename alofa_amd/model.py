@@ -7,6 +7,8 @@ from pathlib import Path
 
 import torch
 
+from . import ops
+
 from . import models as _models  # noqa: F401  (registers the architectures)
 from .config.base import ModelSpec
 from .config.registry import load_config
@@ -110,6 +112,17 @@ class Model:
         y = ctx.scratch("final_normed", (rows.shape[0], self.spec.hidden_size), self.rt.dtype)
         self.final_norm.forward(y, hidden, rows)
         return self.head.forward(ctx, y)
+
+    def greedy(self, ctx, hidden: torch.Tensor, rows: torch.Tensor, out: torch.Tensor, store=None, store_index=None) -> None:
+        """Final norm and head on the wanted rows, and of every row only the first index of its
+        highest logit: out[r] int32, and store[store_index[r]] when a store is given. A head that
+        cannot choose by itself gives logits, and the argmax kernels choose."""
+        y = ctx.scratch("final_normed", (rows.shape[0], self.spec.hidden_size), self.rt.dtype)
+        self.final_norm.forward(y, hidden, rows)
+        if hasattr(self.head, "greedy"):
+            self.head.greedy(ctx, y, out, store, store_index)
+        else:
+            ops.argmax(out, self.head.forward(ctx, y), store=store, store_index=store_index)
 
 
 def runtime(dtype="bfloat16", device="cuda:0") -> Runtime:

@@ -599,6 +599,39 @@ def argmax(out: torch.Tensor, logits: torch.Tensor, store: Optional[torch.Tensor
               _ptr(store), _ptr(store_index), _stream())
 
 
+def can_gemm_argmax(M: int, w: torch.Tensor) -> bool:
+    """Whether ``gemm_argmax`` takes M rows against ``w``: the few-rows form of the tiled product
+    against a matrix as long as a vocabulary (bfloat16; what ``few_rows_kernel`` sends there)."""
+    return (w.dtype is torch.bfloat16 and w.dim() == 2 and 0 < M <= SKINNY_MAX_ROWS and (w.shape[0] + 127) // 128 >= 256
+            and w.shape[1] % 8 == 0 and os.environ.get("ALOFA_FUSE_ARGMAX", "1") != "0")
+
+
+_gemm_argmax_scratch: dict = {}
+_gemm_argmax_retired: list = []
+
+
+def gemm_argmax(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, store: Optional[torch.Tensor] = None,
+                store_index: Optional[torch.Tensor] = None) -> None:
+    """out[m] = the first index of the maximum of a[m] @ w.T (lowest index on ties) without the
+    products ever being written: the blocks of the vocabulary product leave the best of their
+    columns per row, and the argmax's last stage takes the best of those. ``store`` as for ``argmax``."""
+    _gpu("out", out, torch.int32, 1), _contig("out", out)
+    _gpu("a", a, torch.bfloat16, 2), _gpu("w", w, torch.bfloat16, 2)
+    M, K = a.shape
+    if not can_gemm_argmax(M, w) or w.shape[1] != K or out.shape[0] != M:
+        raise AlofaError("unsupported", "the product with the argmax on it takes at most 64 bfloat16 rows against a long bfloat16 matrix",
+                         f"a={tuple(a.shape)} w={tuple(w.shape)} out={tuple(out.shape)}")
+    _store_operands(store, store_index, M)
+    need = 4 * SKINNY_MAX_ROWS * ((w.shape[0] + 127) // 128)
+    scratch = _gemm_argmax_scratch.get(a.device)
+    if scratch is None or scratch.numel() < need:      # (kept: a captured step addresses it)
+        if scratch is not None:
+            _gemm_argmax_retired.append(scratch)
+        scratch = _gemm_argmax_scratch[a.device] = torch.empty(need, dtype=torch.float32, device=a.device)
+    _call("alofa_gemm_argmax", _ptr(out), _ptr(store), _ptr(store_index), _ptr(scratch), _L(scratch.numel()), _ptr(a), _L(_rows("a", a)),
+          _ptr(w), _L(_rows("w", w)), _I(M), _I(w.shape[0]), _I(K), _stream())
+
+
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor,
            store: Optional[torch.Tensor] = None, store_index: Optional[torch.Tensor] = None) -> None:
     """out[r] = inverse-CDF draw from softmax(logits[r] / temperature[r]) at uniform[r] in [0, 1); ``store`` as for ``argmax``."""

@@ -57,6 +57,14 @@ class LMHead(Part):
         ops.gemm(logits, y, self.weight, exact=self.rt.exact)
         return logits
 
+    def greedy(self, ctx, y, out, store=None, store_index=None):
+        """out[r] = the first index of row r's highest logit (and store[store_index[r]], when
+        given), without the logits where the product can take the argmax with it."""
+        if not self.rt.exact and ops.can_gemm_argmax(y.shape[0], self.weight):
+            ops.gemm_argmax(out, y, self.weight, store=store, store_index=store_index)
+        else:
+            ops.argmax(out, self.forward(ctx, y), store=store, store_index=store_index)
+
 
 register_part("embedding", "token_embedding", TokenEmbedding)
 register_part("head", "lm_head", LMHead)

@@ -316,6 +316,42 @@ def test_a_model_of_windows_only_is_admitted_by_what_it_holds(tmp_path):
     held_nothing(eng)
 
 
+def test_greedy_choice_inside_the_step_changes_no_token(tmp_path, monkeypatch):
+    """With a vocabulary long enough for it (40,011 rows here), a step whose requests all take the
+    first maximum chooses by itself: the vocabulary product leaves candidates instead of logits.
+    Same tokens as with the logits written and searched (the product is the same, value for value),
+    in prefill steps, in captured decode steps and in their replays; a request that samples in the
+    batch sends the step back to logits."""
+    from alofa_amd import Engine, ops
+    from alofa_amd.weights import write_random_model
+    cfg = dict(TINY["A"], vocab_size=40011, tie_word_embeddings=False)
+    d = tmp_path / "long_vocabulary"
+    write_random_model(cfg, d, seed=91)
+    prompts = [random_ids(400 + i, 9 + 14 * i, cfg["vocab_size"]) for i in range(5)]
+    calls = []
+    real = ops.gemm_argmax
+    monkeypatch.setattr(ops, "gemm_argmax", lambda *a, **k: (calls.append(a[1].shape[0]), real(*a, **k))[1])
+    eng = Engine(d, dtype="bfloat16", max_tokens=128, max_batch=8)
+    by_step = eng.generate(prompts, max_new=20)
+    assert calls and eng.step_fn.graph_replays > 0
+    n_fused = len(calls)
+    monkeypatch.setenv("ALOFA_FUSE_ARGMAX", "0")
+    searched = Engine(d, dtype="bfloat16", max_tokens=128, max_batch=8).generate(prompts, max_new=20)
+    assert len(calls) == n_fused and by_step == searched
+    monkeypatch.delenv("ALOFA_FUSE_ARGMAX")
+    want = [plain_greedy(d, p, 20) for p in prompts]
+    assert Engine(d, dtype="float32", max_tokens=128, max_batch=8).generate(prompts, max_new=20) == want
+    assert [g[0] for g in by_step] == [w_[0] for w_ in want]      # (later tokens follow the engine's own earlier ones)
+    # one request that samples: the others still get the tokens they get alone
+    from alofa_amd.sampling.sampler import SampleParams
+    mixed = Engine(d, dtype="bfloat16", max_tokens=128, max_batch=8)
+    mixed.core.submit(1, prompts[0], 20)
+    mixed.core.submit(2, prompts[0], 20, SampleParams(temperature=0.8, top_k=5), seed=3)      # as long as the first: they run side by side to the end
+    before = len(calls)
+    mixed.core.run()
+    assert mixed.core.output(1) == by_step[0] and len(mixed.core.output(2)) == 20 and len(calls) == before
+
+
 def test_cancel_and_request_verbs(tiny_dirs):
     from alofa_amd import Engine
     from alofa_amd.errors import AlofaError

@@ -586,6 +586,43 @@ def test_kernels_refuse_what_they_cannot_take():
         assert e.value.name == "unsupported"
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 32768, 72), (8, 40011, 200), (37, 33000, 896), (64, 151936, 64)])
+def test_product_with_the_argmax_on_it(M, N, K):
+    """The vocabulary product that leaves, instead of its outputs, the best column per row: the
+    same choice as the product followed by the argmax kernels, value for value, also where whole
+    rows are full of equal values (small integers as operands: the lowest index must win, within a
+    wave's two tiles, between waves, between blocks), past the matrix's end (N no multiple of 128),
+    and with the choice going to a token store."""
+    o = ops()
+    rng = np.random.default_rng(53)
+    for kind in ("integers", "normal"):
+        if kind == "integers":
+            a = rng.integers(-1, 2, (M, K)).astype(np.float32)
+            w = rng.integers(-1, 2, (N, K)).astype(np.float32)
+        else:
+            a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
+        at, wt = t(a, torch.bfloat16), t(w, torch.bfloat16)
+        assert o.can_gemm_argmax(M, wt)
+        logits = torch.empty(M, N, device=DEV)
+        o.gemm(logits, at, wt)
+        two_steps = torch.empty(M, dtype=torch.int32, device=DEV)
+        o.argmax(two_steps, logits)
+        fused = torch.full((M,), -1, dtype=torch.int32, device=DEV)
+        o.gemm_argmax(fused, at, wt)
+        assert torch.equal(fused, two_steps), kind
+        ref = pm.linear(a, w)
+        assert np.array_equal(ref[np.arange(M), fused.cpu().numpy()], ref.max(1)) or kind == "normal"
+        if kind == "integers":     # exact sums: the plain product's first maximum is the answer
+            assert np.array_equal(fused.cpu().numpy(), ref.argmax(1))
+    store = torch.full((100,), -7, dtype=torch.int32, device=DEV)
+    index = t(rng.permutation(100)[:M].astype(np.int32), torch.int32)
+    again = torch.empty(M, dtype=torch.int32, device=DEV)
+    o.gemm_argmax(again, at, wt, store=store, store_index=index)
+    assert torch.equal(again, fused) and torch.equal(store[index.long()], fused) and int((store != -7).sum()) == M
+    with pytest.raises(AlofaError):
+        o.gemm_argmax(torch.empty(65, dtype=torch.int32, device=DEV), torch.zeros(65, K, device=DEV, dtype=torch.bfloat16), wt)
+
+
 def test_product_kernel_choice():
     """The choice between the two bfloat16 products: few rows and small weights stream, many
     rows or big weights are tiled; a kernel that cannot take the rows is an error, not a guess."""
