@@ -147,3 +147,65 @@ def test_state_slots_without_a_device_are_counted_only():
     assert s == 0 and m.slot("a") == 0 and m.admit("b") == 1
     m.free("a")
     assert m.admit("c") == 0                                      # the slot is used again
+
+
+def _replay_step_layouts(path):
+    """The reference's batch-executor traces (tests/fixtures/batchexec/ there; written by an
+    independent model, scripts/dump_batch_executor_reference.py, checked by
+    tests/unit/test_batch_executor.mojo): requests are added, fed and dropped, and every PLAN is
+    followed by its rows (row, owner, token, position, last visible key). The owners' runs, in the
+    trace's order, go through this cache manager's layout of a step; the positions it gives must
+    be the trace's, and a row sees the keys up to its own position and no further."""
+    from conftest import FIXTURES
+    import numpy as np
+    cm = CacheManager([CacheNeed.keys_and_values(1, 16)], [None], n_blocks=64, block_size=4, max_requests=8)
+    lines = [l.split() for l in (FIXTURES / "batchexec" / path).read_text().splitlines() if l and not l.startswith("#")]
+    rows, steps = [], 0
+
+    def flush():
+        nonlocal rows, steps
+        if not rows:
+            return
+        runs = []                                   # consecutive rows of one owner are one entry of the step
+        for r in rows:
+            if runs and runs[-1][0] == r["r"]:
+                runs[-1][1].append(r)
+            else:
+                runs.append((r["r"], [r]))
+        assert len({owner for owner, _ in runs}) == len(runs), "an owner's rows are one run"
+        slots = np.array([cm.slot(owner) for owner, _ in runs], dtype=np.int32)
+        n_tokens = np.array([len(run) for _, run in runs], dtype=np.int32)
+        pos0, positions, req_of_token, tables, row_slots = cm.plan_step(slots, n_tokens, 64)
+        assert [r["i"] for r in rows] == list(range(len(rows)))
+        assert positions.tolist() == [r["p"] for r in rows], path
+        assert [runs[e][0] for e in req_of_token.tolist()] == [r["r"] for r in rows]
+        assert all(r["v"] == p for r, p in zip(rows, positions.tolist())), "a row sees the keys up to its own position"
+        assert len(set(row_slots[0].tolist())) == len(rows) and (tables[0] >= -1).all()
+        cm.commit_step(slots, n_tokens)
+        cm.check()
+        rows, steps = [], steps + 1
+
+    for op, *fields in lines:
+        kv = dict(f.split("=", 1) for f in fields if "=" in f and not f.startswith("R="))
+        if op != "ROW":
+            flush()
+        if op == "ADD" and "ERR" not in " ".join(fields):
+            cm.admit(int(kv["r"]))
+        elif op == "DROP" and "ERR" not in " ".join(fields):
+            cm.free(int(kv["r"]))
+        elif op == "ROW":
+            rows.append({k: int(v) for k, v in kv.items()})
+    flush()
+    return steps
+
+
+@pytest.mark.parametrize("name", ["e01_two_requests", "e02_hole_after_drop", "e03_more_than_one_step", "e04_batch_full",
+                                  "e05_prompt_longer_than_a_step", "e06_history_outgrows_its_region"])
+def test_reference_step_layouts(name):
+    assert _replay_step_layouts(name + ".trace") >= 1
+
+
+def test_reference_step_layout_control_fails():
+    """bad.trace lets a row see one key past its own position: the replay must refuse it."""
+    with pytest.raises(AssertionError, match="own position"):
+        _replay_step_layouts("bad.trace")
