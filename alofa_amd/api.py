@@ -25,13 +25,17 @@ class Engine:
     written for the same first tokens (src/alofa/runtime/kv/space.mojo:166-243, block by block)."""
 
     def __init__(self, model_dir, dtype: str = "bfloat16", max_tokens: int = 256, max_batch: int = 8,
-                 kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 2048, max_chunk: int = 512,
+                 kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 2048, max_chunk: Optional[int] = None,
                  watermark_permille: int = 900, max_wait_ticks: int = 8, seed: int = 1234, device: str = "cuda:0",
                  trace_path=None, share_prefixes: bool = False, model=None, report=None, run_ahead: bool = True):
         """``model``: a (config, Model) pair already on the device, instead of a folder to load.
         ``report``: a callable that receives one line about device memory at start (default:
         standard error when ALOFA_REPORT_MEMORY is set). ``run_ahead``: a tick reads the tokens of the
-        tick before only after its own step is launched (``EngineCore``); off, every tick is synchronous."""
+        tick before only after its own step is launched (``EngineCore``); off, every tick is synchronous.
+        ``max_chunk``: the most prompt tokens of one request in a tick; by default the whole ``token_budget``,
+        so that a lone long prompt takes one step (requests are served in order of arrival either way, and the
+        budget alone bounds a tick's length)."""
+        max_chunk = token_budget if max_chunk is None else max_chunk
         from .csrc.build import load
         load()
         self.config, self.model = model if model is not None else load_model(Path(model_dir), dtype, device)

@@ -108,10 +108,11 @@ def main(argv=None) -> int:
     block = env_int("ALOFA_BLOCK_SIZE", 16, 1, 1024)
     kv_blocks = env_int("ALOFA_KV_BLOCKS", 0, 0, 1 << 30)
 
+    budget = env_int("ALOFA_TOKEN_BUDGET", 2048, 1, 1 << 20)
     from .api import Engine
     engine = Engine(weights, dtype=dtype, max_tokens=max_tokens, max_batch=batch, kv_blocks=kv_blocks or None,
-                    block_size=block, token_budget=env_int("ALOFA_TOKEN_BUDGET", 2048, 1, 1 << 20),
-                    max_chunk=env_int("ALOFA_MAX_CHUNK", 512, 1, 1 << 20),
+                    block_size=block, token_budget=budget,
+                    max_chunk=env_int("ALOFA_MAX_CHUNK", budget, 1, 1 << 20),
                     watermark_permille=env_int("ALOFA_WATERMARK_PERMILLE", 900, 1, 1000),
                     max_wait_ticks=env_int("ALOFA_MAX_WAIT_TICKS", 8, 0, 1 << 20), seed=seed,
                     trace_path=env_str("ALOFA_TRACE", "") or None,

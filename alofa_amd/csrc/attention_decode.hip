@@ -22,10 +22,14 @@
 // The pages of a wave's share are read from the block table once, 64 at a time,
 // one per lane; keys and values of the next two steps are on their way while a
 // step is computed. At the end the waves' states meet in LDS and are combined in
-// wave order. With several parts (long contexts) the blocks' states go to a
-// scratch buffer and a second kernel combines them in part order. The order of
-// additions depends only on the key range, the wave count and the part count,
-// never on timing.
+// wave order. A block reads its keys at the rate of one compute unit, so where
+// the (token, key head) pairs are far fewer than the compute units their keys
+// are cut into parts, one block each: the blocks' states go to a scratch buffer
+// and a second kernel combines them in part order. (Handing the states to the
+// block that arrives last, through uncached memory and a counter, was measured:
+// it costs as much as the second kernel with a few parts and more with many.)
+// The order of additions depends only on the key range, the wave count and the
+// part count, never on timing.
 // Cache layout: keys [block, kv_head, slot_in_block, d], values transposed [block, kv_head, d, slot_in_block].
 #include "common.h"
 
@@ -122,7 +126,10 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   // the new token's key (this lane's channel slices, rotated) and value (channels 16 nt + c16), kRope only
   uint4 new_k[DS];
   uint32_t new_v[DT];
+  float4 cs[kRope ? DS / 2 : 1][2], sn[kRope ? DS / 2 : 1][2];
+  int64_t new_slot = 0;
   if constexpr (kRope) {
+    new_slot = rope.slots[t];
     const bf16_t* row = q + static_cast<int64_t>(t) * q_stride;
     const bf16_t* k_row = row + static_cast<int64_t>(heads + hk) * d;
     const bf16_t* v_row = row + static_cast<int64_t>(heads + kv_heads + hk) * d;
@@ -130,33 +137,12 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     for (int ds = 0; ds < DS; ++ds) new_k[ds] = *reinterpret_cast<const uint4*>(k_row + ds * 32 + g * 8);
 #pragma unroll
     for (int nt = 0; nt < DT; ++nt) new_v[nt] = v_row[nt * 16 + c16];
-    // pairs (c, c + d / 2): slices ds and ds + DS / 2 of this lane
+    // (cos and sin of the pairs (c, c + d / 2): slices ds and ds + DS / 2 of this lane)
 #pragma unroll
     for (int ds = 0; ds < DS / 2; ++ds) {
       const int64_t at = static_cast<int64_t>(p) * (d / 2) + ds * 32 + g * 8;
-      const float4 c_lo = *reinterpret_cast<const float4*>(rope.cos_t + at), c_hi = *reinterpret_cast<const float4*>(rope.cos_t + at + 4);
-      const float4 s_lo = *reinterpret_cast<const float4*>(rope.sin_t + at), s_hi = *reinterpret_cast<const float4*>(rope.sin_t + at + 4);
-      const Pair8 rq = rotate8(__builtin_bit_cast(uint4, qf[ds]), __builtin_bit_cast(uint4, qf[ds + DS / 2]), c_lo, c_hi, s_lo, s_hi);
-      qf[ds] = __builtin_bit_cast(bf16x8, rq.lo);
-      qf[ds + DS / 2] = __builtin_bit_cast(bf16x8, rq.hi);
-      const Pair8 rk = rotate8(new_k[ds], new_k[ds + DS / 2], c_lo, c_hi, s_lo, s_hi);
-      new_k[ds] = rk.lo;
-      new_k[ds + DS / 2] = rk.hi;
-    }
-    // the wave that owns the last tile of keys (in the first chunk of heads) writes the token's cache slot
-    if (h0 == 0 && tile_begin <= last && last < tile_end) {
-      const int64_t slot = rope.slots[t];
-      const int64_t blk = slot >> bs_shift, off = slot & bs_mask;
-      if (c16 == 0) {
-#pragma unroll
-        for (int ds = 0; ds < DS; ++ds)
-          *reinterpret_cast<uint4*>(k_cache + ((((blk * kv_heads + hk) << bs_shift) + off) * d) + ds * 32 + g * 8) = new_k[ds];
-      }
-      if (g == 0) {
-#pragma unroll
-        for (int nt = 0; nt < DT; ++nt)
-          v_cache[(((blk * kv_heads + hk) * d + nt * 16 + c16) << bs_shift) + off] = static_cast<bf16_t>(new_v[nt]);
-      }
+      cs[ds][0] = *reinterpret_cast<const float4*>(rope.cos_t + at), cs[ds][1] = *reinterpret_cast<const float4*>(rope.cos_t + at + 4);
+      sn[ds][0] = *reinterpret_cast<const float4*>(rope.sin_t + at), sn[ds][1] = *reinterpret_cast<const float4*>(rope.sin_t + at + 4);
     }
   }
 
@@ -167,7 +153,8 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   const float scale2 = scale * 1.44269504088896340736f;   // scores in units of log2(e)
 
   // lane x holds the page of logical block page_base + x; a step's keys lie within 64 pages of its first
-  int page_base = (tile_begin << 4) >> bs_shift;
+  // (a share whose first step lies within the first 64 pages uses the pages that set out at the start)
+  int page_base = ((((tile_begin + 2) << 4) - 1) >> bs_shift) < 64 ? 0 : (tile_begin << 4) >> bs_shift;
   const int last_page = p >> bs_shift;
   // (pages that a window has passed read -1: they are never used, and 0 keeps every address inside the cache)
   if (page_base != 0) {     // uniform over the wave: a share that starts past the pages already on their way
@@ -295,6 +282,36 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   if (tile < tile_end) fetch(tile, s0);
   if (tile + 2 < tile_end) fetch(tile + 2, s1);
   if (kThree && tile + 4 < tile_end) fetch(tile + 4, s2);
+  // The rotation comes after the first keys and values have set out: it needs cos and sin only, which were
+  // asked for before them.
+  if constexpr (kRope) {
+    // pairs (c, c + d / 2): slices ds and ds + DS / 2 of this lane
+#pragma unroll
+    for (int ds = 0; ds < DS / 2; ++ds) {
+      const float4 c_lo = cs[ds][0], c_hi = cs[ds][1], s_lo = sn[ds][0], s_hi = sn[ds][1];
+      const Pair8 rq = rotate8(__builtin_bit_cast(uint4, qf[ds]), __builtin_bit_cast(uint4, qf[ds + DS / 2]), c_lo, c_hi, s_lo, s_hi);
+      qf[ds] = __builtin_bit_cast(bf16x8, rq.lo);
+      qf[ds + DS / 2] = __builtin_bit_cast(bf16x8, rq.hi);
+      const Pair8 rk = rotate8(new_k[ds], new_k[ds + DS / 2], c_lo, c_hi, s_lo, s_hi);
+      new_k[ds] = rk.lo;
+      new_k[ds + DS / 2] = rk.hi;
+    }
+    // the wave that owns the last tile of keys (in the first chunk of heads) writes the token's cache slot
+    if (h0 == 0 && tile_begin <= last && last < tile_end) {
+      const int64_t blk = new_slot >> bs_shift, off = new_slot & bs_mask;
+      if (c16 == 0) {
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds)
+          *reinterpret_cast<uint4*>(k_cache + ((((blk * kv_heads + hk) << bs_shift) + off) * d) + ds * 32 + g * 8) = new_k[ds];
+      }
+      if (g == 0) {
+#pragma unroll
+        for (int nt = 0; nt < DT; ++nt)
+          v_cache[(((blk * kv_heads + hk) * d + nt * 16 + c16) << bs_shift) + off] = static_cast<bf16_t>(new_v[nt]);
+      }
+    }
+  }
+
   // while every set has a further step to fetch: no branches, so that the waits are counted exactly
   for (; tile + 2 * kStride - 2 < tile_end; tile += kStride) {
     compute(tile, s0);

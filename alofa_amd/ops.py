@@ -136,11 +136,30 @@ SKINNY_MAX_ROWS = 64
 SWIGLU = 2
 
 
-def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
+ROWS_MAX_M, ROWS_MAX_K = 8, 6144      # what the vector-unit kernel for very few rows takes
+USE_ROWS_KERNEL = os.environ.get("ALOFA_ROWS_KERNEL", "1") != "0"
+
+
+def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: bool = False) -> str:
     """Which bfloat16 product takes ``M`` rows against ``w_rows`` rows of weights
-    (gate and up together for the fused feed-forward entry): ``"stream"``, every
-    wave reading its own operands straight from memory (M <= 64 only), or
-    ``"tiled"``, blocks that share both operands through LDS.
+    (gate and up together for the fused feed-forward entry): ``"rows"``, the
+    vector-unit kernel for at most eight rows, whose blocks own four or eight
+    columns each and read every row of ``a`` (float32 rows that take a norm on
+    their way if ``normed``); ``"stream"``, every wave reading its own operands
+    straight from memory into matrix-core tiles (M <= 64 only); or ``"tiled"``,
+    blocks that share both operands through LDS.
+
+    The vector-unit kernel has the most and the smallest blocks and no hand-over
+    between them, which is what a small matrix's time is made of; but it reads the
+    rows once per four columns and its arithmetic grows with M. Measured at the
+    projection sizes of 0.5B, 7B and 32B models against the streaming kernel
+    (w_rows * K in elements): it wins at one and two rows everywhere (0.5B down
+    projection 3.6 against 8.3 us, 7B gate/up 47 against 59); at three and four
+    rows except with float32 rows against 24 M elements or more (32B QKV: 28.9
+    against 26.8); at five to eight rows for plain rows up to 32 M (0.5B down 5.2
+    against 8.6, 32B output projection 18.3 against 23.2), for float32 rows only up
+    to 4 M (0.5B QKV 4.8 against 5.5, 7B QKV 20.5 against 17.1), and never for gate
+    and up together (0.5B: 10.8 against 9.9).
 
     The streaming kernel reads the rows of ``a`` once per 16 or 32 weight rows, so
     its time grows with M; the tiled kernel's hardly does, but it needs more work
@@ -156,6 +175,11 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
     if not swiglu and (w_rows + 127) // 128 >= 256:
         return "tiled"
     elements = w_rows * K
+    if USE_ROWS_KERNEL and M <= ROWS_MAX_M and K <= ROWS_MAX_K and K % 8 == 0:
+        if M <= 2 or (M <= 4 and (swiglu or not normed or elements < 24 << 20)):
+            return "rows"
+        if M > 4 and not swiglu and elements <= ((4 << 20) if normed else (32 << 20)):
+            return "rows"
     if M <= 4:
         return "stream"
     if M <= 8:
@@ -165,10 +189,12 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
     return "tiled" if elements >= 8 << 20 else "stream"
 
 
-def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int, swiglu: bool = False) -> str:
-    kernel = kernel or few_rows_kernel(M, w_rows, K, swiglu)
+def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int, swiglu: bool = False, normed: bool = False) -> str:
+    kernel = kernel or few_rows_kernel(M, w_rows, K, swiglu, normed)
     if kernel == "stream" and M <= SKINNY_MAX_ROWS:
         return "alofa_gemm_skinny"
+    if kernel == "rows" and M <= ROWS_MAX_M and K <= ROWS_MAX_K and K % 8 == 0:
+        return "alofa_gemm_rows"
     if kernel == "tiled":
         return "alofa_gemm_mfma"
     raise AlofaError("invalid_argument", "no such product kernel for these rows", f"kernel={kernel} M={M}")
@@ -201,15 +227,20 @@ NORM_MAX_ROWS, NORM_MAX_COLUMNS = 16, 8192     # what the streaming kernel's nor
 FUSE_NORMS = os.environ.get("ALOFA_FUSE_NORMS", "1") != "0"   # 0: every norm runs as a kernel of its own
 
 
-def can_fuse_norm(M: int, w: torch.Tensor, out_dtype, swiglu: bool = False) -> bool:
+def can_fuse_norm(M: int, w: torch.Tensor, out_dtype, swiglu: bool = False, kernel: Optional[str] = None) -> bool:
     """Whether the product of ``M`` float32 rows with the bfloat16 matrix ``w`` can take an RMSNorm
-    of those rows on its way (``gemm(..., norm=)``, ``gemm_swiglu(..., norm=)``): the streaming
-    kernel does, where it is the kernel of choice and does not share K out over blocks."""
+    of those rows on its way (``gemm(..., norm=)``, ``gemm_swiglu(..., norm=)``): the vector-unit
+    kernel for very few rows does, and the streaming kernel where it does not share K out over
+    blocks; whichever is the kernel of choice (or ``kernel``)."""
     N, K = w.shape
     if not FUSE_NORMS:
         return False
-    if (w.dtype is not torch.bfloat16 or out_dtype is not torch.bfloat16 or M > NORM_MAX_ROWS or K > NORM_MAX_COLUMNS or K % 8 or w.stride(0) % 8
-            or w.data_ptr() % 16 or few_rows_kernel(M, 2 * N if swiglu else N, K, swiglu) != "stream"):
+    if w.dtype is not torch.bfloat16 or out_dtype is not torch.bfloat16 or K % 8 or w.stride(0) % 8 or w.data_ptr() % 16:
+        return False
+    chosen = kernel or few_rows_kernel(M, 2 * N if swiglu else N, K, swiglu, normed=True)
+    if chosen == "rows":
+        return M <= ROWS_MAX_M and K <= ROWS_MAX_K
+    if M > NORM_MAX_ROWS or K > NORM_MAX_COLUMNS or chosen != "stream":
         return False
     if swiglu:
         return True
@@ -230,20 +261,20 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
          add_to_out: bool = False, exact: bool = False, kernel: Optional[str] = None, norm: Optional[tuple] = None) -> None:
     """out = a @ w.T (+ bias), or out += a @ w.T when ``add_to_out`` (out is then
     the float32 residual stream). w is [out_features, in_features]. ``kernel``
-    names the bfloat16 kernel ("stream" or "tiled") instead of ``few_rows_kernel``.
+    names the bfloat16 kernel ("rows", "stream" or "tiled") instead of ``few_rows_kernel``.
     ``norm`` = (weight, eps): ``a`` holds float32 rows that take an RMSNorm on their way
     into the product (only where ``can_fuse_norm`` says so)."""
     _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w", w, None, 2)
     M, K = a.shape
     N = w.shape[0]
     if norm is not None:
-        if add_to_out or exact or not can_fuse_norm(M, w, out.dtype) or tuple(out.shape) != (M, N) or w.shape[1] != K:
+        if add_to_out or exact or not can_fuse_norm(M, w, out.dtype, kernel=kernel) or tuple(out.shape) != (M, N) or w.shape[1] != K:
             raise AlofaError("unsupported", "no kernel takes a norm with this product", f"a={tuple(a.shape)} w={tuple(w.shape)} out={out.dtype}")
         if bias is not None:
             _gpu("bias", bias, torch.float32, 1), _contig("bias", bias)
             if bias.shape[0] != N:
                 raise AlofaError("shape_mismatch", "bias length does not fit", f"bias={tuple(bias.shape)} N={N}")
-        _call("alofa_gemm_skinny", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)),
+        _call(_product_entry(kernel, M, N, K, normed=True), _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)),
               _ptr(bias), _I(M), _I(N), _I(K), _I(STORE), *_norm_operands(a, norm, K), _stream())
         return
     if w.shape[1] != K or tuple(out.shape) != (M, N):
@@ -260,7 +291,7 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
     if not exact and _mfma_operands(a, w):
         _ensure_workspace(a.device)
         entry = _product_entry(kernel, M, N, K)
-        no_norm = (_ptr(None), _F(0.0)) if entry == "alofa_gemm_skinny" else ()
+        no_norm = (_ptr(None), _F(0.0)) if entry != "alofa_gemm_mfma" else ()
         _call(entry, _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
               _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
               _I(ADD_TO_RESIDUAL if add_to_out else STORE), *no_norm, _stream())
@@ -281,15 +312,15 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: 
     if w_gate.dtype is not w_up.dtype or _rows("w_gate", w_gate) != _rows("w_up", w_up):
         raise AlofaError("invalid_argument", "gate and up matrices must share dtype and layout")
     if norm is not None:
-        if exact or not can_fuse_norm(M, w_gate, out.dtype, swiglu=True) or w_up.data_ptr() % 16:
+        if exact or not can_fuse_norm(M, w_gate, out.dtype, swiglu=True, kernel=kernel) or w_up.data_ptr() % 16:
             raise AlofaError("unsupported", "no kernel takes a norm with this product", f"a={tuple(a.shape)} gate={tuple(w_gate.shape)} out={out.dtype}")
-        _call("alofa_gemm_skinny", _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
+        _call(_product_entry(kernel, M, 2 * N, K, True, normed=True), _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
               _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), *_norm_operands(a, norm, K), _stream())
         return
     if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up):
         _ensure_workspace(a.device)
         entry = _product_entry(kernel, M, 2 * N, K, True)
-        no_norm = (_ptr(None), _F(0.0)) if entry == "alofa_gemm_skinny" else ()
+        no_norm = (_ptr(None), _F(0.0)) if entry != "alofa_gemm_mfma" else ()
         _call(entry, _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
               _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), *no_norm, _stream())
         return
@@ -370,16 +401,23 @@ def decode_waves(d: int) -> int:
 
 
 def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
-    """Parts the keys of a (token, key head) are cut into beyond the waves of a block. None while a
-    wave has at most eight steps of 32 keys (a second kernel that merges the parts costs as much as
-    it saves there). Longer contexts: down to about two steps a wave, but only until the blocks fill
-    the chip (a block's fixed cost is paid once per part)."""
+    """Parts the keys of a (token, key head) are cut into beyond the waves of a block; a second
+    kernel merges the parts' states. A block reads its keys at the rate of one compute unit, so
+    while the blocks are far fewer than the compute units more of them are faster: none up to
+    four steps of 32 keys a wave (the second kernel costs in a step what the parts save there,
+    more than it does run alone), then a part per step of all the waves, at most eight (the
+    merge grows with them), from there on a part per two steps; never more parts than fill the
+    chip. (Measured at 14:2 heads of 64 and 28:4 of 128, batches of 1 to 64, contexts of 200 to
+    4,000: at 2,000 keys and batch 8, 9.6 us with eight parts against 17.6 with one.)"""
     waves = decode_waves(d)
-    if max_context <= 32 * waves * 8:
+    step = 32 * waves
+    if max_context <= 4 * step:
         return 1
     blocks = tokens * kv_heads * -(-(heads // kv_heads) // 16)
-    by_length = -(-max_context // (32 * waves * 2))
     by_chip = max(1, 256 // max(1, blocks))
+    by_length = -(-max_context // step)
+    if by_length > 8:
+        by_length = max(8, -(-max_context // (2 * step)))
     return max(1, min(64, by_length, by_chip))
 
 
@@ -443,7 +481,7 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
 
 def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
                      max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
-                     rope: Optional[tuple] = None) -> None:
+                     rope: Optional[tuple] = None, n_splits: Optional[int] = None) -> None:
     """bfloat16 attention for tokens of requests that bring few tokens: every
     token of the batch, or the tokens ``rows`` (int32 indices into the batch).
     ``req_of_token`` None: every request brings one token and token i is request
@@ -451,7 +489,9 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     With ``rope`` = (cos, sin, slots) the rows of ``q`` are the fused projection's
     [queries | keys | values] of ONE new token per request, not yet rotated: the
     kernel rotates queries and the new key itself, uses the new key and value from
-    registers and writes them to the token's cache slot (``can_fuse_rope_into_decode``)."""
+    registers and writes them to the token's cache slot (``can_fuse_rope_into_decode``).
+    ``n_splits`` (default ``decode_splits``): blocks that share the keys of a (token, key head);
+    their states go to ``scratch`` and a second kernel combines them."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     for n, t in (("req_of_token", req_of_token), ("positions", positions)):
         if t is None and n == "req_of_token":
@@ -479,7 +519,8 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
         _gpu("slots", slots, torch.int64, 1), _contig("slots", slots)
         if slots.shape[0] != T:
             raise AlofaError("shape_mismatch", "one cache slot per token", f"slots={tuple(slots.shape)} T={T}")
-    n_splits = decode_splits(n_tok, heads, kv_heads, d, min(max_context, window or max_context))
+    if n_splits is None:
+        n_splits = decode_splits(n_tok, heads, kv_heads, d, min(max_context, window or max_context))
     floats = n_tok * heads * n_splits * (d + 2) if n_splits > 1 else 0
     if floats and (scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous()):
         raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")

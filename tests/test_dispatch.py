@@ -9,11 +9,22 @@ from alofa_amd.errors import AlofaError
 def test_product_kernel_by_shape():
     assert ops.few_rows_kernel(65, 8, 8) == "tiled"                               # beyond the streaming kernel's rows
     assert ops.few_rows_kernel(1, 151936, 896) == "tiled"                         # a vocabulary-long matrix, from the first row on
-    assert ops.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "stream"       # (not so for the fused gate/up form)
-    for rows in (1, 8, 16, 64):
-        assert ops.few_rows_kernel(rows, 1152, 896) == "stream"                   # 0.5B-sized projections stream at every batch
+    assert ops.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "rows"         # (not so for the fused gate/up form)
+    for rows in (9, 16, 64):
+        assert ops.few_rows_kernel(rows, 1152, 896) == "stream"                   # 0.5B-sized projections stream from nine rows on
+    # at most eight rows: the vector-unit kernel, while the rows it reads once per four columns and its arithmetic stay light
+    for rows in (1, 2, 4, 8):
+        assert ops.few_rows_kernel(rows, 1152, 896) == "rows" and ops.few_rows_kernel(rows, 896, 4864) == "rows"
+        assert ops.few_rows_kernel(rows, 1152, 896, normed=True) == "rows"
+    assert ops.few_rows_kernel(4, 2 * 4864, 896, swiglu=True, normed=True) == "rows" and ops.few_rows_kernel(5, 2 * 4864, 896, swiglu=True, normed=True) == "stream"
+    assert ops.few_rows_kernel(4, 4608, 3584, normed=True) == "rows" and ops.few_rows_kernel(4, 7168, 5120, normed=True) == "stream"
+    assert ops.few_rows_kernel(8, 4608, 3584, normed=True) == "stream" and ops.few_rows_kernel(8, 5120, 5120) == "rows"
+    assert ops.few_rows_kernel(2, 3584, 18944) == "stream"                        # longer rows than its waves cover
     assert ops.few_rows_kernel(8, 3584, 18944) == "tiled" and ops.few_rows_kernel(4, 3584, 18944) == "stream"
     assert ops.few_rows_kernel(16, 4608, 3584) == "stream" and ops.few_rows_kernel(17, 4608, 3584) == "tiled"
+    assert ops._product_entry(None, 8, 896, 4864) == "alofa_gemm_rows" and ops._product_entry("stream", 8, 896, 4864) == "alofa_gemm_skinny"
+    with pytest.raises(AlofaError):
+        ops._product_entry("rows", 9, 64, 64)
     with pytest.raises(AlofaError):
         ops._product_entry("stream", 65, 64, 64)
     with pytest.raises(AlofaError):
@@ -21,11 +32,13 @@ def test_product_kernel_by_shape():
 
 
 def test_decode_splits_follow_the_context():
-    short = ops.decode_splits(8, 14, 2, 64, 1024)
-    assert short == 1                                                             # the waves of one block cover a short context
-    assert ops.decode_splits(8, 14, 2, 64, 1 << 13) > ops.decode_splits(8, 14, 2, 64, 1 << 12) > 1   # about two steps of 32 keys a wave
+    assert ops.decode_splits(8, 14, 2, 64, 512) == 1 and ops.decode_splits(8, 14, 2, 64, 1024) == 1    # the waves of one block cover four steps each
+    assert ops.decode_splits(8, 14, 2, 64, 2048) == 8                             # a part per step of all the waves
+    assert ops.decode_splits(8, 14, 2, 64, 1 << 12) == 8 and ops.decode_splits(8, 14, 2, 64, 1 << 13) == 16    # at most eight, then a part per two steps
     assert ops.decode_splits(8, 14, 2, 64, 1 << 16) == 256 // 16                   # until the blocks fill the chip
-    assert ops.decode_splits(64, 14, 2, 64, 1 << 13) <= ops.decode_splits(8, 14, 2, 64, 1 << 13)    # many blocks already: fewer parts
+    assert ops.decode_splits(64, 14, 2, 64, 2048) == 2 and ops.decode_splits(32, 14, 2, 64, 2048) == 4    # many blocks already: fewer parts
+    assert ops.decode_splits(8, 28, 4, 128, 512) == 1 and ops.decode_splits(8, 28, 4, 128, 1024) == 8 and ops.decode_splits(8, 28, 4, 128, 4096) == 8
+    assert ops.decode_splits(32, 28, 4, 128, 1024) == 2 and ops.decode_splits(64, 28, 4, 128, 4096) == 1
     assert ops.decode_waves(64) == 8 and ops.decode_waves(128) == 4 and ops.decode_waves(256) == 4
 
 

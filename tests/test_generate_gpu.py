@@ -392,3 +392,15 @@ def test_generate_command(tiny_dirs, tmp_path):
     env2 = dict(os.environ, ALOFA_WEIGHTS=str(tmp_path / "made"), ALOFA_RANDOM_CONFIG=str(cfgp), ALOFA_SEED="5", ALOFA_MAX_NEW="3", ALOFA_MAX_TOKENS="64")
     p = subprocess.run([str(ROOT / "bin" / "generate"), "5,6,7"], env=env2, capture_output=True, text=True, timeout=300)
     assert p.returncode == 0 and (tmp_path / "made" / "model.safetensors").exists() and len(p.stdout.strip().split(",")) == 3
+
+
+def test_a_lone_prompt_is_one_step_by_default(tiny_dirs):
+    """Without max_chunk a request may take the whole budget of a tick: a prompt below it is one step."""
+    from alofa_amd import Engine
+    eng = Engine(tiny_dirs["A"], dtype="float32", max_tokens=64, token_budget=48)
+    assert eng.sched_cfg.max_chunk == 48
+    eng.core.submit(1, random_ids(1, 40, 256), 2)
+    eng.core.tick()
+    assert eng.core.last_action.prefill == [(1, 0, 40)]
+    eng.core.run()
+    assert Engine(tiny_dirs["A"], dtype="float32", max_tokens=64, token_budget=48, max_chunk=16).sched_cfg.max_chunk == 16

@@ -149,14 +149,70 @@ def test_product_that_takes_the_norm_with_it(M, N, K):
     two = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
     o.gemm(two, y, t(w, torch.bfloat16), t(b), kernel="stream")
     assert (out.float() - two.float()).abs().max().item() <= 2e-2 * max(1.0, two.float().abs().max().item())
-    # rows do not depend on their neighbours: the first row alone gives the same bits
+    # rows do not depend on their neighbours: the first row alone gives the same bits (where the same kernel takes one row)
     one = torch.empty(1, N, device=DEV, dtype=torch.bfloat16)
-    o.gemm(one, t(x[:1]), t(w, torch.bfloat16), t(b), norm=(t(nw), eps))
+    o.gemm(one, t(x[:1]), t(w, torch.bfloat16), t(b), norm=(t(nw), eps), kernel=o.few_rows_kernel(M, N, K, normed=True))
     assert torch.equal(one[0], out[0])
     assert o.can_fuse_norm(M, t(w, torch.bfloat16), torch.bfloat16, swiglu=True)
     act = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
     o.gemm_swiglu(act, t(x), t(w, torch.bfloat16), t(w2, torch.bfloat16), norm=(t(nw), eps))
     close(act, pm.swiglu(pm.linear(normed, w), pm.linear(normed, w2)), BF16, "norm + gate/up + swiglu")
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1152, 896), (8, 896, 4864), (3, 97, 80), (7, 1000, 1544), (5, 130, 6144), (2, 64, 8), (4, 4864, 896), (6, 35, 520)])
+def test_product_for_very_few_rows(M, N, K):
+    """The vector-unit product for at most eight rows, every form of it (store with bias, float32 store,
+    residual, gate/up, and the norm on the way in), at sizes that end inside a run of 512 along K and
+    inside a block's columns; a row's bits do not depend on the rows beside it."""
+    o = ops()
+    rng = np.random.default_rng(44)
+    a, w, w2 = (bf(rng.standard_normal(shape).astype(np.float32) * scale) for shape, scale in (((M, K), 1.0), ((N, K), 0.1), ((N, K), 0.1)))
+    b = rng.standard_normal(N).astype(np.float32)
+    at, wt, w2t = t(a, torch.bfloat16), t(w, torch.bfloat16), t(w2, torch.bfloat16)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm(out, at, wt, t(b), kernel="rows")
+    close(out, pm.linear(a, w, b), BF16, "store + bias")
+    outf = torch.empty(M, N, device=DEV)
+    o.gemm(outf, at, wt, kernel="rows")
+    close(outf, pm.linear(a, w), 1e-4, "float32 store")
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    acc = t(res)
+    o.gemm(acc, at, wt, add_to_out=True, kernel="rows")
+    close(acc, pm.add(res, pm.linear(a, w)), 1e-4, "residual")
+    act = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm_swiglu(act, at, wt, w2t, kernel="rows")
+    close(act, pm.swiglu(pm.linear(a, w), pm.linear(a, w2)), BF16, "gate/up")
+    # float32 rows that take a norm on their way
+    x = (rng.standard_normal((M, K)) * rng.uniform(0.05, 30.0, (M, 1))).astype(np.float32)
+    nw = (1.0 + 0.3 * rng.standard_normal(K)).astype(np.float32)
+    normed = pm.rmsnorm(x, nw, 1e-5)
+    outn, actn = torch.empty(M, N, device=DEV, dtype=torch.bfloat16), torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm(outn, t(x), wt, t(b), norm=(t(nw), 1e-5), kernel="rows")
+    close(outn, pm.linear(normed, w, b), BF16, "norm + store + bias")
+    o.gemm_swiglu(actn, t(x), wt, w2t, norm=(t(nw), 1e-5), kernel="rows")
+    close(actn, pm.swiglu(pm.linear(normed, w), pm.linear(normed, w2)), BF16, "norm + gate/up")
+    # the last row alone: the same bits in every form
+    r = M - 1
+    one, onef, one_acc, one_act, one_n = (torch.empty(1, N, device=DEV, dtype=d) for d in (torch.bfloat16, torch.float32, torch.float32, torch.bfloat16, torch.bfloat16))
+    o.gemm(one, at[r:], wt, t(b), kernel="rows")
+    o.gemm(onef, at[r:], wt, kernel="rows")
+    one_acc.copy_(t(res[r:]))
+    o.gemm(one_acc, at[r:], wt, add_to_out=True, kernel="rows")
+    o.gemm_swiglu(one_act, at[r:], wt, w2t, kernel="rows")
+    o.gemm(one_n, t(x[r:]), wt, t(b), norm=(t(nw), 1e-5), kernel="rows")
+    for alone, batch, what in ((one, out, "store"), (onef, outf, "float32 store"), (one_acc, acc, "residual"), (one_act, act, "gate/up"), (one_n, outn, "norm + store")):
+        assert torch.equal(alone[0], batch[r]), what
+
+
+def test_product_for_very_few_rows_refuses_what_it_cannot_take():
+    o = ops()
+    w = torch.zeros(16, 6152, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(AlofaError):          # more rows than eight
+        o.gemm(torch.empty(9, 16, device=DEV), torch.zeros(9, 64, device=DEV, dtype=torch.bfloat16), w[:, :64].contiguous(), kernel="rows")
+    with pytest.raises(AlofaError):          # longer rows than its waves cover
+        o.gemm(torch.empty(2, 16, device=DEV), torch.zeros(2, 6152, device=DEV, dtype=torch.bfloat16), w, kernel="rows")
+    from alofa_amd.csrc.build import load
+    assert load().alofa_gemm_rows_fits(8, 16, 6144) == 1 and load().alofa_gemm_rows_fits(8, 16, 6152) == 0 and load().alofa_gemm_rows_fits(9, 16, 64) == 0
 
 
 def test_gemm_split_over_blocks_is_repeatable():
@@ -362,13 +418,13 @@ def test_paged_attention(heads, kv_heads, d, bs, dtype, exact, window):
 
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 80, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (18, 2, 32, 64), (20, 1, 32, 16)])
 @pytest.mark.parametrize("window", [None, 21, 300])
-@pytest.mark.parametrize("bucket", [700, 8192])
+@pytest.mark.parametrize("bucket", [700, 2048, 8192])
 def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
     """The kernel for few query tokens per request: single tokens and short
     portions, contexts from one key to many pages, groups of 1 to 9 heads per
     key head, head sizes whose lanes-per-key is no power of two. ``bucket`` is the
     context bound the launch is shaped for: the waves of one block share the keys
-    out, and for the larger bound several blocks do, whose states a second kernel combines."""
+    out, and for the larger bounds several blocks do, whose states a second kernel combines."""
     rng = np.random.default_rng(17)
     lens, q_lens = [1, 37, 700, 64, 333], [1, 2, 1, 4, 3]
     c = paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16)
@@ -381,7 +437,7 @@ def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(5)])
     close(out, ref, BF16, "decode attention")
     if (heads, d, window) == (14, 64, None):
-        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == (1 if bucket == 700 else 11)   # several parts are really in play (256 // 22 blocks)
+        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == {700: 1, 2048: 8, 8192: 11}[bucket]   # several parts are really in play (256 // 22 blocks)
     one = torch.empty(1, heads * d, device=DEV, dtype=torch.bfloat16)        # one token that sees one key
     o.paged_attention(one, c["qcat"][:1], c["kc"], c["vc"], c["table"], c["req"][:1], c["pos"][:1], heads, kv_heads, d, window, scale, False,
                       max_q_len=1, max_context=1)
@@ -627,8 +683,8 @@ def test_product_kernel_choice():
     """The choice between the two bfloat16 products: few rows and small weights stream, many
     rows or big weights are tiled; a kernel that cannot take the rows is an error, not a guess."""
     o = ops()
-    assert o.few_rows_kernel(1, 151936, 896) == "tiled" and o.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "stream"
-    assert o.few_rows_kernel(4, 4608, 3584) == "stream" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
+    assert o.few_rows_kernel(1, 151936, 896) == "tiled" and o.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "rows"
+    assert o.few_rows_kernel(4, 4608, 3584) == "rows" and o.few_rows_kernel(4, 3584, 18944) == "stream" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
     assert o.few_rows_kernel(64, 2 * 4864, 896, swiglu=True) == "tiled" and o.few_rows_kernel(16, 2 * 4864, 896, swiglu=True) == "stream"
     assert o.few_rows_kernel(64, 896, 4864) == "stream" and o.few_rows_kernel(32, 3584, 3584) == "tiled"
     assert o.few_rows_kernel(65, 8, 8) == "tiled"
