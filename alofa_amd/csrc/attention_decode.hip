@@ -24,10 +24,11 @@
 // step is computed. At the end the waves' states meet in LDS and are combined in
 // wave order. A block reads its keys at the rate of one compute unit, so where
 // the (token, key head) pairs are far fewer than the compute units their keys
-// are cut into parts, one block each: the blocks' states go to a scratch buffer
-// and a second kernel combines them in part order. (Handing the states to the
-// block that arrives last, through uncached memory and a counter, was measured:
-// it costs as much as the second kernel with a few parts and more with many.)
+// are cut into parts, one block each. Few parts hand their states over in the
+// library's workspace (uncached memory and a counter): the block that arrives
+// last combines them in part order. Many parts leave them in a scratch buffer
+// and a second kernel combines them (the last block's work grows with the parts,
+// the second kernel's does not).
 // The order of additions depends only on the key range, the wave count and the
 // part count, never on timing.
 // Cache layout: keys [block, kv_head, slot_in_block, d], values transposed [block, kv_head, d, slot_in_block].
@@ -83,12 +84,13 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     int64_t q_stride, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ rows, int heads, int kv_heads,
-    int bs_shift, int window, float scale, RopeArgs rope) {
+    int bs_shift, int window, float scale, RopeArgs rope, int* __restrict__ counters) {
   static_assert(!kRope || DT % 4 == 0, "the rotation needs a channel and its partner in the same lane: d a multiple of 64");
   constexpr int d = DT * 16;
   constexpr int DS = (d + 31) / 32;            // steps of 32 along d in the first product
   // per wave and head: maximum, sum of weights, (two unused,) weighted value sums of the wave's share
   __shared__ __attribute__((aligned(16))) float state[NW][kHeadsPerBlock][d + 4];
+  __shared__ int last_block;
   const int group = heads / kv_heads;
   const int chunks = (group + kHeadsPerBlock - 1) / kHeadsPerBlock;
   // the tokens served are rows[0..gridDim.x) of the packed batch, or all of it
@@ -364,9 +366,51 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
       store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
     } else {
       float* dst = partial + ((static_cast<int64_t>(blockIdx.x) * heads + h) * n_parts + blockIdx.z) * (d + 2);
-      dst[2 + c] = acc;
-      if (c == 0) { dst[0] = big; dst[1] = total; }
+      if (counters) {   // (device scope: written through to memory, where blocks on every die find it)
+        __hip_atomic_store(dst + 2 + c, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (c == 0) {
+          __hip_atomic_store(dst, big, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(dst + 1, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      } else {
+        dst[2 + c] = acc;
+        if (c == 0) { dst[0] = big; dst[1] = total; }
+      }
     }
+  }
+  if (n_parts == 1 || !counters) return;
+
+  // The parts of a (token, key head) hand their states over in the library's workspace: every wave waits
+  // until its stores have been performed in memory, then the block is counted; the block that arrives last
+  // combines all parts in part order (the same sum on every run) and puts the counter back to zero.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int* counter = counters + blockIdx.x * gridDim.y + blockIdx.y;
+    const int arrived = atomicAdd(counter, 1);
+    last_block = arrived == n_parts - 1;
+    if (last_block) atomicExch(counter, 0);
+  }
+  __syncthreads();
+  if (!last_block) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  for (int x = threadIdx.x; x < kHeadsPerBlock * d; x += 64 * NW) {
+    const int i = x / d, c = x % d;
+    if (h0 + i >= group) break;
+    const int h = hk * group + h0 + i;
+    const float* src = partial + (static_cast<int64_t>(blockIdx.x) * heads + h) * n_parts * (d + 2);
+    float big = -FLT_MAX;
+    for (int sp = 0; sp < n_parts; ++sp) big = fmaxf(big, __hip_atomic_load(src + sp * (d + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    float total = 0.f, acc = 0.f;
+#pragma unroll 4
+    for (int sp = 0; sp < n_parts; ++sp) {
+      const float* part = src + sp * (d + 2);
+      const float e = __builtin_amdgcn_exp2f(__hip_atomic_load(part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - big);
+      total += __hip_atomic_load(part + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * e;
+      acc += __hip_atomic_load(part + 2 + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * e;
+    }
+    store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
   }
 }
 
@@ -409,15 +453,25 @@ extern "C" int64_t alofa_attention_decode_scratch(int tokens, int heads, int d, 
   return n_splits > 1 ? static_cast<int64_t>(tokens) * heads * n_splits * (d + 2) : 0;
 }
 
+// Whether the parts of these sizes fit the library's workspace (their states and a counter per (token, key head,
+// chunk of heads)), so that the last block of a (token, key head) can combine them and no second kernel is needed.
+extern "C" int alofa_attention_decode_can_hand_over(int tokens, int heads, int kv_heads, int d, int n_splits) {
+  if (tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || n_splits <= 1) return 0;
+  const Workspace& ws = workspace();
+  const int64_t counters = static_cast<int64_t>(tokens) * kv_heads * ((heads / kv_heads + kHeadsPerBlock - 1) / kHeadsPerBlock);
+  return ws.tiles != nullptr && counters <= ws.n_counters && alofa_attention_decode_scratch(tokens, heads, d, n_splits) <= ws.tile_floats;
+}
+
 // cos_t, sin_t, slots: null for queries that are rotated and a cache that is written already; else (see RopeArgs)
 // q holds rows [queries | keys | values] of one new token per request. req_of_token may be null when every
-// request brings one token: token i then belongs to row i of block_table.
+// request brings one token: token i then belongs to row i of block_table. hand_over: the parts meet in the
+// workspace (alofa_attention_decode_can_hand_over must hold; `partial` is not used), not in `partial` and a second kernel.
 extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
                                       void* k_cache, void* v_cache, const int32_t* block_table,
                                       int max_blocks, const int32_t* req_of_token, const int32_t* positions,
                                       const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
                                       float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
-                                      hipStream_t stream) {
+                                      int hand_over, hipStream_t stream) {
   ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
   ALOFA_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention_decode: head size %d must be 16..256 in steps of 16", d);
@@ -425,7 +479,14 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
                 "attention_decode: block_size=%d must be a power of two, at least 4; max_blocks=%d window=%d", block_size, max_blocks, window);
   int bs_shift = 0;
   while ((1 << bs_shift) < block_size) ++bs_shift;
-  ALOFA_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || partial), "attention_decode: n_splits=%d (1..%d) needs scratch when above 1", n_splits, kMaxSplits);
+  ALOFA_REQUIRE(n_splits >= 1 && n_splits <= kMaxSplits && (n_splits == 1 || partial || hand_over), "attention_decode: n_splits=%d (1..%d) needs scratch when above 1", n_splits, kMaxSplits);
+  int* counters = nullptr;
+  if (hand_over && n_splits > 1) {
+    ALOFA_REQUIRE(alofa_attention_decode_can_hand_over(tokens, heads, kv_heads, d, n_splits),
+                  "attention_decode: the states of %d parts of %d tokens do not fit the workspace", n_splits, tokens);
+    partial = workspace().tiles;
+    counters = workspace().counters;
+  }
   ALOFA_REQUIRE(q_stride % 8 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_decode: q rows must be 16-byte aligned");
   ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(v_cache) % 8 == 0, "attention_decode: caches must be 16-byte aligned");
   const bool fused = cos_t != nullptr;
@@ -439,7 +500,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   attention_decode_kernel<DT, NW, ROPE><<<grid, 64 * NW, 0, stream>>>(                                                    \
       static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                            \
       static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), block_table, max_blocks, req_of_token,                \
-      positions, rows, heads, kv_heads, bs_shift, window, scale, rope)
+      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters)
   if (fused) {
     switch (d / 64) {
       case 1: ALOFA_DECODE(4, 8, true); break;
@@ -469,7 +530,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   }
 #undef ALOFA_DECODE
   if (check_launch("attention_decode")) return 1;
-  if (n_splits > 1) {
+  if (n_splits > 1 && !counters) {
     attention_merge_kernel<<<dim3(tokens, heads), 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits);
     return check_launch("attention_merge");
   }

@@ -401,30 +401,46 @@ def decode_waves(d: int) -> int:
 
 
 def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
-    """Parts the keys of a (token, key head) are cut into beyond the waves of a block; a second
-    kernel merges the parts' states. A block reads its keys at the rate of one compute unit, so
-    while the blocks are far fewer than the compute units more of them are faster: none up to
-    four steps of 32 keys a wave (the second kernel costs in a step what the parts save there,
-    more than it does run alone), then a part per step of all the waves, at most eight (the
-    merge grows with them), from there on a part per two steps; never more parts than fill the
-    chip. (Measured at 14:2 heads of 64 and 28:4 of 128, batches of 1 to 64, contexts of 200 to
-    4,000: at 2,000 keys and batch 8, 9.6 us with eight parts against 17.6 with one.)"""
+    """Parts the keys of a (token, key head) are cut into beyond the waves of a block. A block reads
+    its keys at the rate of one compute unit, so while the blocks are far fewer than the compute
+    units more of them are faster: none up to two steps of 32 keys a wave; up to four steps four
+    parts, which the last block to arrive combines (``decode_hand_over``), if the chip has room for
+    eight; then a part per step of all the waves, at most eight (the merge grows with them), and
+    from there on a part per two steps, combined by a second kernel; never more parts than fill
+    the chip. (Measured at 14:2 heads of 64 and 28:4 of 128, batches of 1 to 64, contexts of 200
+    to 4,000: at 2,000 keys and batch 8, 9.6 us with eight parts against 17.6 with one; at 1,000
+    keys 9.2 with four against 11.9.)"""
     waves = decode_waves(d)
     step = 32 * waves
-    if max_context <= 4 * step:
+    if max_context <= 2 * step:
         return 1
     blocks = tokens * kv_heads * -(-(heads // kv_heads) // 16)
     by_chip = max(1, 256 // max(1, blocks))
+    if max_context <= 4 * step:
+        return 4 if by_chip >= 8 else 1
     by_length = -(-max_context // step)
     if by_length > 8:
         by_length = max(8, -(-max_context // (2 * step)))
     return max(1, min(64, by_length, by_chip))
 
 
+HAND_OVER_MAX_PARTS = 4    # up to so many parts the last block combines them; a second kernel combines more
+
+
+def decode_hand_over(tokens: int, heads: int, kv_heads: int, d: int, n_splits: int) -> bool:
+    """Whether ``n_splits`` parts of a (token, key head) hand their states over in the library's workspace, where
+    the block that arrives last combines them (few parts that fit it); else they go to the caller's scratch and a
+    second kernel."""
+    if n_splits <= 1 or n_splits > HAND_OVER_MAX_PARTS:
+        return False
+    _ensure_workspace(None)
+    return bool(load().alofa_attention_decode_can_hand_over(_I(tokens), _I(heads), _I(kv_heads), _I(d), _I(n_splits)))
+
+
 def decode_scratch_floats(tokens: int, heads: int, kv_heads: int, d: int, max_context: int, window: Optional[int]) -> int:
     """Floats of scratch the decode kernel needs for these sizes (0: none)."""
     n = decode_splits(tokens, heads, kv_heads, d, min(max_context, window or max_context))
-    return tokens * heads * n * (d + 2) if n > 1 else 0
+    return tokens * heads * n * (d + 2) if n > 1 and not decode_hand_over(tokens, heads, kv_heads, d, n) else 0
 
 
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -481,7 +497,7 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
 
 def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
                      max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
-                     rope: Optional[tuple] = None, n_splits: Optional[int] = None) -> None:
+                     rope: Optional[tuple] = None, n_splits: Optional[int] = None, hand_over: Optional[bool] = None) -> None:
     """bfloat16 attention for tokens of requests that bring few tokens: every
     token of the batch, or the tokens ``rows`` (int32 indices into the batch).
     ``req_of_token`` None: every request brings one token and token i is request
@@ -491,7 +507,8 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     kernel rotates queries and the new key itself, uses the new key and value from
     registers and writes them to the token's cache slot (``can_fuse_rope_into_decode``).
     ``n_splits`` (default ``decode_splits``): blocks that share the keys of a (token, key head);
-    their states go to ``scratch`` and a second kernel combines them."""
+    ``hand_over`` (default ``decode_hand_over``): the last of them to arrive combines their states,
+    else the states go to ``scratch`` and a second kernel combines them."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     for n, t in (("req_of_token", req_of_token), ("positions", positions)):
         if t is None and n == "req_of_token":
@@ -521,13 +538,18 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
             raise AlofaError("shape_mismatch", "one cache slot per token", f"slots={tuple(slots.shape)} T={T}")
     if n_splits is None:
         n_splits = decode_splits(n_tok, heads, kv_heads, d, min(max_context, window or max_context))
-    floats = n_tok * heads * n_splits * (d + 2) if n_splits > 1 else 0
+    if hand_over is None:
+        hand_over = decode_hand_over(n_tok, heads, kv_heads, d, n_splits)
+    elif hand_over and not (n_splits > 1 and _ensure_workspace(None) is None
+                            and load().alofa_attention_decode_can_hand_over(_I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(n_splits))):
+        raise AlofaError("out_of_range", "the parts' states do not fit the library's workspace (or there is one part only)", f"tokens={n_tok} heads={heads} d={d} n_splits={n_splits}")
+    floats = n_tok * heads * n_splits * (d + 2) if n_splits > 1 and not hand_over else 0
     if floats and (scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous()):
         raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")
     _call("alofa_attention_decode", _ptr(out), _L(_rows("out", out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
           _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(rows),
           _I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits),
-          _ptr(cos), _ptr(sin), _ptr(slots), _stream())
+          _ptr(cos), _ptr(sin), _ptr(slots), _I(int(hand_over)), _stream())
 
 
 def can_fuse_rope_into_decode(d: int) -> bool:

@@ -437,7 +437,7 @@ def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
     ref = np.concatenate([pm.attention(c["q"][r], c["k"][r], c["v"][r], heads, kv_heads, d, window) for r in range(5)])
     close(out, ref, BF16, "decode attention")
     if (heads, d, window) == (14, 64, None):
-        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == {700: 1, 2048: 8, 8192: 11}[bucket]   # several parts are really in play (256 // 22 blocks)
+        assert o.decode_splits(sum(q_lens), heads, kv_heads, d, bucket) == {700: 4, 2048: 8, 8192: 11}[bucket]   # several parts are really in play (256 // 22 blocks)
     one = torch.empty(1, heads * d, device=DEV, dtype=torch.bfloat16)        # one token that sees one key
     o.paged_attention(one, c["qcat"][:1], c["kc"], c["vc"], c["table"], c["req"][:1], c["pos"][:1], heads, kv_heads, d, window, scale, False,
                       max_q_len=1, max_context=1)
@@ -447,6 +447,13 @@ def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
         with pytest.raises(AlofaError):                                          # needed scratch is demanded, not allocated behind the back
             o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, False,
                               max_q_len=4, max_context=bucket)
+    # both ways in which parts meet, whatever the launch would choose: the last block combines them, or a second kernel does
+    for parts in (2, 4):
+        for hand_over in (True, False):
+            again = torch.zeros_like(out)
+            o.attention_decode(again, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, bucket,
+                               torch.empty(sum(q_lens) * heads * parts * (d + 2), device=DEV), n_splits=parts, hand_over=hand_over)
+            close(again, ref, BF16, f"decode attention, {parts} parts, hand-over {hand_over}")
 
 
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(14, 2, 64, 16), (8, 2, 128, 32), (20, 1, 64, 8), (3, 3, 256, 16)])
