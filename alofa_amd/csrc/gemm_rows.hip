@@ -34,9 +34,12 @@ __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
 }
 
-// v of lane l ^ 4 (within a row of 16), by the LDS crossbar (no LDS memory is touched)
+// v of lane l ^ 4 (within a row of 16): the lanes of banks 0 and 2 (four lanes each) read four lanes up,
+// those of banks 1 and 3 four lanes down
 __device__ __forceinline__ float lane_xor4(float v) {
-  return __uint_as_float(__builtin_amdgcn_ds_swizzle(__float_as_uint(v), 0x101F));   // and 0x1f, or 0, xor 4
+  const uint32_t x = __float_as_uint(v);
+  const uint32_t up = __builtin_amdgcn_update_dpp(0u, x, 0x104, 0xf, 0x5, false);     // row_shl:4 into banks 0, 2
+  return __uint_as_float(__builtin_amdgcn_update_dpp(up, x, 0x114, 0xf, 0xa, false));   // row_shr:4 into banks 1, 3
 }
 
 // The sums over all 64 lanes of n values per lane (n a power of two, at most 64), by halving: after the
@@ -103,39 +106,35 @@ __global__ void __launch_bounds__(64 * kMaxWaves) gemm_rows_kernel(
   const int k0 = (wave * 64 + lane) * 8;
   const bool k_ok = k0 < K;
 
-  // every load of this lane sets out: the weights (from memory), then the rows (which every block reads: from L2)
+  // Every load of this lane sets out, the weights (from memory) first, then the rows (which every block reads:
+  // from L2). No load is conditional: a lane past the end of K reads where lane 0 does, rows beyond M and columns
+  // beyond N read the last row and column (what they give is cleared below, or never stored), so that the loads are
+  // one straight run of instructions with nothing to wait for between them.
+  const int k_at = k_ok ? k0 : 0;
   uint4 wv[kMats][C];
 #pragma unroll
   for (int mat = 0; mat < kMats; ++mat)
 #pragma unroll
     for (int c = 0; c < C; ++c) {
-      wv[mat][c] = make_uint4(0, 0, 0, 0);
       const bf16_t* base = mat == 0 ? W : W2;
-      if (k_ok && n0 + c < N) wv[mat][c] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(n0 + c) * ldw + k0);
+      const int n = n0 + c < N ? n0 + c : N - 1;
+      wv[mat][c] = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(n) * ldw + k_at);
     }
   uint4 av[MR];               // the rows' values as pairs of bfloat16
   float4 xlo[kNorm ? MR : 1], xhi[kNorm ? MR : 1], nlo, nhi;
   if constexpr (kNorm) {
-    nlo = nhi = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (k_ok) {
-      nlo = *reinterpret_cast<const float4*>(norm_w + k0);
-      nhi = *reinterpret_cast<const float4*>(norm_w + k0 + 4);
-    }
+    nlo = *reinterpret_cast<const float4*>(norm_w + k_at);
+    nhi = *reinterpret_cast<const float4*>(norm_w + k_at + 4);
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
-      xlo[m] = xhi[m] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (k_ok && m < M) {
-        const float* row = static_cast<const float*>(A) + static_cast<int64_t>(m) * lda + k0;
-        xlo[m] = *reinterpret_cast<const float4*>(row);
-        xhi[m] = *reinterpret_cast<const float4*>(row + 4);
-      }
+      const float* row = static_cast<const float*>(A) + static_cast<int64_t>(m < M ? m : M - 1) * lda + k_at;
+      xlo[m] = *reinterpret_cast<const float4*>(row);
+      xhi[m] = *reinterpret_cast<const float4*>(row + 4);
     }
   } else {
 #pragma unroll
-    for (int m = 0; m < MR; ++m) {
-      av[m] = make_uint4(0, 0, 0, 0);
-      if (k_ok && m < M) av[m] = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(A) + static_cast<int64_t>(m) * lda + k0);
-    }
+    for (int m = 0; m < MR; ++m)
+      av[m] = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(A) + static_cast<int64_t>(m < M ? m : M - 1) * lda + k_at);
   }
   // what the epilogue adds sets out too: thread c * MR + m finishes out[m, n0 + c]
   const int my_c = threadIdx.x / MR, my_m = threadIdx.x % MR;
@@ -144,6 +143,20 @@ __global__ void __launch_bounds__(64 * kMaxWaves) gemm_rows_kernel(
   if (finisher) {
     if (kEpilogue == kRwStore && bias) add = bias[n0 + my_c];
     if (kEpilogue == kRwResidual) add = load_f32(out + static_cast<int64_t>(my_m) * ldo + n0 + my_c);
+  }
+  // a lane past the end of K adds nothing: its weights and its rows' values are cleared
+  if (!k_ok) {
+#pragma unroll
+    for (int mat = 0; mat < kMats; ++mat)
+#pragma unroll
+      for (int c = 0; c < C; ++c) wv[mat][c] = make_uint4(0, 0, 0, 0);
+    if constexpr (kNorm) {
+#pragma unroll
+      for (int m = 0; m < MR; ++m) xlo[m] = xhi[m] = make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+#pragma unroll
+      for (int m = 0; m < MR; ++m) av[m] = make_uint4(0, 0, 0, 0);
+    }
   }
 
   float ss[MR];

@@ -36,8 +36,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 enum SkinnyEpilogue : int { kSkStore = 0, kSkResidual = 1, kSkSwiglu = 2 };
 
-constexpr int kMaxNormK = 8192;    // columns of a product that takes a norm (the norm's weights lie in LDS)
-
 
 // A partial sum leaves for the workspace at device scope: written through to memory, past this
 // die's L2, where blocks on every die find it.
@@ -208,22 +206,10 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     };
     constexpr int kStride = kUnroll * kWaves;
     int s = first_step + wave;
-    // (the norm's weights set out first: loads come back in order, so the wait for them, before the barrier,
-    // is then no wait for the weights and rows that follow)
-    constexpr int kNormLoads = kMaxNormK / (kWaves * 64 * 4);
-    float4 nw_stage[kNormLoads];
-#pragma unroll
-    for (int j = 0; j < kNormLoads; ++j) {
-      const int i = (j * kWaves * 64 + threadIdx.x) * 4;
-      nw_stage[j] = i < K ? *reinterpret_cast<const float4*>(norm_w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
     issue(ra0, w0, s);
     issue(ra1, w1, s + kStride);
-#pragma unroll
-    for (int j = 0; j < kNormLoads; ++j) {
-      const int i = (j * kWaves * 64 + threadIdx.x) * 4;
-      if (i < K) *reinterpret_cast<float4*>(norm_lds + i) = nw_stage[j];
-    }
+    for (int i = threadIdx.x * 4; i < K; i += kWaves * 64 * 4)
+      *reinterpret_cast<float4*>(norm_lds + i) = *reinterpret_cast<const float4*>(norm_w + i);
     __syncthreads();
     for (; s < n_steps; s += 2 * kStride) {
       multiply(ra0, w0, s);
@@ -327,6 +313,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   }
 }
 
+constexpr int kMaxNormK = 8192;    // columns of a product that takes a norm (the norm's weights lie in LDS)
 
 struct NormArgs {
   const float* weight;   // null: A is bfloat16 and no norm is applied
