@@ -1,5 +1,5 @@
 // Matrix products for at most eight rows (the decode steps of few requests), bfloat16, on the
-// vector units: out[m, n] = sum_k A[m, k] * W[n, k] with M <= 8 and K <= 6144.
+// vector units: out[m, n] = sum_k A[m, k] * W[n, k] with M <= 8.
 //
 // The work is streaming W once from memory, and the time is what a compute unit needs to pull
 // its share, so the shares are made small and even: a block owns C output columns (rows of W,
@@ -15,6 +15,10 @@
 // of their values and add, so that each keeps half as many, then the last pair is added; the
 // waves' sums meet in LDS and are added in wave order. The order of additions is fixed and the
 // same for every row whatever else is in the batch (M only selects how many rows are computed).
+//
+// Up to twelve runs of 512 a wave takes one run (no loop at all); a longer K (the down projection of
+// a wide feed-forward) goes to a second kernel whose eight waves take every eighth run in turn, the loads
+// of the next run on their way while this one is multiplied.
 //
 // With a norm (kNorm) the rows of A are the float residual stream: a value is x * w_norm rounded
 // to bfloat16, the squares of x are summed beside the products, and the row's factor
@@ -223,11 +227,101 @@ __global__ void __launch_bounds__(64 * kMaxWaves) gemm_rows_kernel(
   }
 }
 
+// K beyond kRowsMaxK: the block's eight waves (eight rows' operands leave no registers for more, and the number
+// must not depend on the rows: it sets the order of the additions) take the runs wave, wave + 8, ... in turn, two
+// sets of operands
+// in flight (each is loaded again as soon as it has been multiplied: no copies between sets, a copy would wait
+// for its load). Store and residual epilogues, bfloat16 rows.
+constexpr int rows_long_waves(int) { return 8; }
+
+template <int MR, int C, int kEpilogue, typename TO>
+__global__ void __launch_bounds__(64 * rows_long_waves(MR)) gemm_rows_long_kernel(
+    TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W, int64_t ldw,
+    const float* __restrict__ bias, int M, int N, int K) {
+  constexpr int V = C * MR, kWaves = rows_long_waves(MR);
+  __shared__ float red[kWaves][V];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int n0 = blockIdx.x * C;
+  const bf16_t* w_row[C];
+  const bf16_t* a_row[MR];
+#pragma unroll
+  for (int c = 0; c < C; ++c) w_row[c] = W + static_cast<int64_t>(n0 + c < N ? n0 + c : N - 1) * ldw;
+#pragma unroll
+  for (int m = 0; m < MR; ++m) a_row[m] = A + static_cast<int64_t>(m < M ? m : M - 1) * lda;
+  struct Set {
+    uint4 w[C], a[MR];
+  };
+  // run `run` of K sets out (a lane past the end of K reads where lane 0 of the first run does; cleared at use)
+  auto fetch = [&](Set& s, int run) __attribute__((always_inline)) {
+    const int k0 = (run * 64 + lane) * 8;
+    const int k_at = k0 < K ? k0 : 0;
+#pragma unroll
+    for (int c = 0; c < C; ++c) s.w[c] = *reinterpret_cast<const uint4*>(w_row[c] + k_at);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) s.a[m] = *reinterpret_cast<const uint4*>(a_row[m] + k_at);
+  };
+  float acc[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) acc[i] = 0.f;
+  auto multiply = [&](const Set& s, int run) __attribute__((always_inline)) {
+    const bool k_ok = (run * 64 + lane) * 8 < K;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const uint4 w = k_ok ? s.w[c] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int m = 0; m < MR; ++m) {
+        float t = dot2(s.a[m].x, w.x, acc[c * MR + m]);
+        t = dot2(s.a[m].y, w.y, t);
+        t = dot2(s.a[m].z, w.z, t);
+        acc[c * MR + m] = dot2(s.a[m].w, w.w, t);
+      }
+    }
+  };
+  const int my_c = threadIdx.x / MR, my_m = threadIdx.x % MR;
+  const bool finisher = threadIdx.x < V && my_m < M && n0 + my_c < N;
+  float add = 0.f;
+  if (finisher) {
+    if (kEpilogue == kRwStore && bias) add = bias[n0 + my_c];
+    if (kEpilogue == kRwResidual) add = load_f32(out + static_cast<int64_t>(my_m) * ldo + n0 + my_c);
+  }
+  const int runs = (K + 511) / 512;
+  Set s0, s1;
+  int run = wave;
+  fetch(s0, run);
+  fetch(s1, run + kWaves);
+  // (whole rounds: every fetch is issued, a run past the end reads run 0's place and adds nothing)
+  for (; run < runs; run += 2 * kWaves) {
+    multiply(s0, run);
+    fetch(s0, run + 2 * kWaves);
+    multiply(s1, run + kWaves);
+    fetch(s1, run + 3 * kWaves);
+  }
+  constexpr int kShift = 6 - log2_of(V);
+  lanes_sum<V>(acc, lane);
+  if ((lane & ((1 << kShift) - 1)) == 0) red[wave][lane >> kShift] = acc[0];
+  __syncthreads();
+  if (!finisher) return;
+  float sum = red[0][threadIdx.x];
+#pragma unroll
+  for (int w = 1; w < kWaves; ++w) sum += red[w][threadIdx.x];
+  TO* dst = out + static_cast<int64_t>(my_m) * ldo + n0 + my_c;
+  store_f32(dst, kEpilogue == kRwStore ? sum + add : add + sum);
+}
+
 template <int MR, int C, int kEpilogue, typename TO, bool kNorm>
 static int launch_rows(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                        const float* bias, int M, int N, int K, const float* norm_w, float eps, hipStream_t stream) {
   const int waves = (K + 511) / 512;
   const dim3 grid((N + C - 1) / C);
+  if (waves > kRowsMaxWaves) {
+    if constexpr (!kNorm && kEpilogue != kRwSwiglu) {
+      gemm_rows_long_kernel<MR, C, kEpilogue, TO><<<grid, 64 * rows_long_waves(MR), 0, stream>>>(
+          static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), ldw, bias, M, N, K);
+      return check_launch("gemm_rows (long K)");
+    }
+    ALOFA_REQUIRE(false, "gemm_rows: K=%d beyond %d goes with the store and residual epilogues of bfloat16 rows only", K, kRowsMaxK);
+    return 1;
+  }
 #define ALOFA_ROWS(MAXW)                                                                                               \
   gemm_rows_kernel<MR, C, kEpilogue, TO, kNorm, MAXW><<<grid, 64 * waves, 0, stream>>>(                                \
       static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, \
@@ -258,15 +352,20 @@ static int dispatch_rows(void* out, int64_t ldo, const void* A, int64_t lda, con
 using namespace alofa;
 
 // Whether alofa_gemm_rows takes these sizes.
-extern "C" int alofa_gemm_rows_fits(int M, int N, int K) { return M >= 1 && M <= 8 && N >= 1 && K >= 8 && K % 8 == 0 && K <= kRowsMaxK; }
+// (K beyond 6,144: the store and residual epilogues of bfloat16 rows only, `plain` then says that this is such a product)
+extern "C" int alofa_gemm_rows_fits(int M, int N, int K, int plain) {
+  return M >= 1 && M <= 8 && N >= 1 && K >= 8 && K % 8 == 0 && (K <= kRowsMaxK || plain);
+}
 
 // The same operands and epilogues as alofa_gemm_skinny (bfloat16 A [M, K] and W [N, K]; W2 for the swiglu epilogue;
 // 0 store (+ bias) as o_dtype, 1 add to the float residual, 2 swiglu; norm_w not null: A is float [M, K] and takes
-// an RMSNorm with these weights and eps on its way, bfloat16 store and swiglu epilogues), for M <= 8 and K <= 6144.
+// an RMSNorm with these weights and eps on its way, bfloat16 store and swiglu epilogues), for M <= 8; K beyond 6,144
+// with the store and residual epilogues of bfloat16 rows only.
 extern "C" int alofa_gemm_rows(void* out, int o_dtype, int64_t ldo, const void* A, int64_t lda, const void* W,
                                const void* W2, int64_t ldw, const float* bias, int M, int N, int K, int epilogue,
                                const float* norm_w, float eps, hipStream_t stream) {
-  ALOFA_REQUIRE(alofa_gemm_rows_fits(M, N, K), "gemm_rows: M=%d (1..8) N=%d K=%d (a multiple of 8, at most %d)", M, N, K, kRowsMaxK);
+  ALOFA_REQUIRE(alofa_gemm_rows_fits(M, N, K, norm_w == nullptr && epilogue != kRwSwiglu),
+                "gemm_rows: M=%d (1..8) N=%d K=%d (a multiple of 8; beyond %d with the store and residual epilogues of bfloat16 rows only)", M, N, K, kRowsMaxK);
   ALOFA_REQUIRE(ldw % 8 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 && (W2 == nullptr || reinterpret_cast<uintptr_t>(W2) % 16 == 0),
                 "gemm_rows: rows of W must be 16-byte aligned");
   ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && lda % (norm_w ? 4 : 8) == 0, "gemm_rows: rows of A must be 16-byte aligned");

@@ -136,7 +136,13 @@ SKINNY_MAX_ROWS = 64
 SWIGLU = 2
 
 
-ROWS_MAX_M, ROWS_MAX_K = 8, 6144      # what the vector-unit kernel for very few rows takes
+ROWS_MAX_M, ROWS_MAX_K = 8, 6144      # what the vector-unit kernel for very few rows takes (longer rows: plain products only)
+
+
+def rows_kernel_takes(M: int, K: int, swiglu: bool = False, normed: bool = False) -> bool:
+    """Sizes the vector-unit kernel takes: at most eight rows, K a multiple of 8; K beyond 6,144 only for a plain
+    product (bfloat16 rows, store or residual epilogue), which a second kernel loops over."""
+    return 1 <= M <= ROWS_MAX_M and K % 8 == 0 and (K <= ROWS_MAX_K or not (swiglu or normed))
 USE_ROWS_KERNEL = os.environ.get("ALOFA_ROWS_KERNEL", "1") != "0"
 
 
@@ -175,7 +181,7 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: b
     if not swiglu and (w_rows + 127) // 128 >= 256:
         return "tiled"
     elements = w_rows * K
-    if USE_ROWS_KERNEL and M <= ROWS_MAX_M and K <= ROWS_MAX_K and K % 8 == 0:
+    if USE_ROWS_KERNEL and rows_kernel_takes(M, K, swiglu, normed):
         if M <= 2 or (M <= 4 and (swiglu or not normed or elements < 24 << 20)):
             return "rows"
         if M > 4 and not swiglu and elements <= ((4 << 20) if normed else (32 << 20)):
@@ -193,7 +199,7 @@ def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int, swiglu: b
     kernel = kernel or few_rows_kernel(M, w_rows, K, swiglu, normed)
     if kernel == "stream" and M <= SKINNY_MAX_ROWS:
         return "alofa_gemm_skinny"
-    if kernel == "rows" and M <= ROWS_MAX_M and K <= ROWS_MAX_K and K % 8 == 0:
+    if kernel == "rows" and rows_kernel_takes(M, K, swiglu, normed):
         return "alofa_gemm_rows"
     if kernel == "tiled":
         return "alofa_gemm_mfma"
@@ -239,7 +245,7 @@ def can_fuse_norm(M: int, w: torch.Tensor, out_dtype, swiglu: bool = False, kern
         return False
     chosen = kernel or few_rows_kernel(M, 2 * N if swiglu else N, K, swiglu, normed=True)
     if chosen == "rows":
-        return M <= ROWS_MAX_M and K <= ROWS_MAX_K
+        return rows_kernel_takes(M, K, swiglu, True)
     if M > NORM_MAX_ROWS or K > NORM_MAX_COLUMNS or chosen != "stream":
         return False
     if swiglu:

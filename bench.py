@@ -434,19 +434,22 @@ def long_prompts(args):
 
 
 def sweep(args):
-    """Decode steps over batch sizes (at a context of about 550) or over contexts (batch 1, 8, 32) at the
-    0.5B sizes: one line per point with ms per step, tokens a second and the bytes the step has to read / time."""
-    cfg = dict(CONFIGS["0.5b"], num_hidden_layers=args.layers or CONFIGS["0.5b"]["num_hidden_layers"])
+    """Decode steps over batch sizes (at a context of about 550) or over contexts (batch 1, 8, 32): one line per
+    point with ms per step, tokens a second and the bytes the step has to read / time. At the 0.5B sizes, or with
+    --config 7b / 32b at those (batches up to 64; --layers for fewer layers than the configuration has)."""
+    name = args.config
+    cfg = dict(CONFIGS[name], num_hidden_layers=args.layers or CONFIGS[name]["num_hidden_layers"])
     model = device_model(cfg, args.dtype, 20260918)
     dbytes = 2 if args.dtype == "bfloat16" else 4
-    cases = ([(b, PROMPT) for b in (1, 2, 4, 8, 16, 17, 24, 32, 48, 64, 96, 128, 192, 256)] if args.sweep == "batch" else
+    batches = (1, 2, 4, 8, 16, 17, 24, 32, 48, 64, 96, 128, 192, 256) if name == "0.5b" else (1, 2, 4, 8, 16, 32, 64)
+    cases = ([(b, PROMPT) for b in batches] if args.sweep == "batch" else
              [(b, p) for p in (2048, 8192, 16384, 30000) for b in (1, 8, 32)])
     for batch, prompt in cases:
         pt = DecodePoint(model, cfg, args.dtype, batch, prompt, context=max(CONTEXT, prompt + 256))
         pt.run(8)
         s = pt.run(24)
         byts = decode_bytes(cfg, pt.context_lengths(), dbytes)
-        print(json.dumps({"batch": batch, "context": prompt, "ms_per_step": round(s * 1e3, 4), "tok_s": round(batch / s, 1),
+        print(json.dumps({"model": name, "layers": cfg["num_hidden_layers"], "batch": batch, "context": prompt, "ms_per_step": round(s * 1e3, 4), "tok_s": round(batch / s, 1),
                           "gb_s": round(byts / s / 1e9, 1), "frac_hbm": round(byts / s / 1e9 / PEAK_HBM_GBS, 4)}), flush=True)
         pt.close()
     return 0
@@ -464,7 +467,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points, the prefill, the repeats and the roofs")
     ap.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its line")
-    ap.add_argument("--sweep", choices=["batch", "context"], default=None, help="decode steps over batch sizes or over contexts, a line per point (0.5B sizes)")
+    ap.add_argument("--sweep", choices=["batch", "context"], default=None, help="decode steps over batch sizes or over contexts, a line per point (the sizes of --config)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (--gpus must be 1)")

@@ -209,10 +209,38 @@ def test_product_for_very_few_rows_refuses_what_it_cannot_take():
     w = torch.zeros(16, 6152, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(AlofaError):          # more rows than eight
         o.gemm(torch.empty(9, 16, device=DEV), torch.zeros(9, 64, device=DEV, dtype=torch.bfloat16), w[:, :64].contiguous(), kernel="rows")
-    with pytest.raises(AlofaError):          # longer rows than its waves cover
-        o.gemm(torch.empty(2, 16, device=DEV), torch.zeros(2, 6152, device=DEV, dtype=torch.bfloat16), w, kernel="rows")
+    with pytest.raises(AlofaError):          # rows longer than its waves cover at once: plain products only, not gate/up
+        o.gemm_swiglu(torch.empty(2, 16, device=DEV, dtype=torch.bfloat16), torch.zeros(2, 6152, device=DEV, dtype=torch.bfloat16), w, w, kernel="rows")
+    with pytest.raises(AlofaError):          # ... and not with a norm on the way
+        o.gemm(torch.empty(2, 16, device=DEV, dtype=torch.bfloat16), torch.zeros(2, 6152, device=DEV), w, norm=(torch.ones(6152, device=DEV), 1e-5), kernel="rows")
     from alofa_amd.csrc.build import load
-    assert load().alofa_gemm_rows_fits(8, 16, 6144) == 1 and load().alofa_gemm_rows_fits(8, 16, 6152) == 0 and load().alofa_gemm_rows_fits(9, 16, 64) == 0
+    fits = load().alofa_gemm_rows_fits
+    assert fits(8, 16, 6144, 0) == 1 and fits(8, 16, 6152, 0) == 0 and fits(8, 16, 6152, 1) == 1 and fits(9, 16, 64, 1) == 0
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 130, 18944), (4, 67, 6152), (8, 96, 12296), (3, 40, 27648)])
+def test_product_for_very_few_rows_against_long_rows(M, N, K):
+    """K beyond the runs that the waves of a block cover at once: the kernel that loops over them (store with
+    bias, float32 store, residual), at lengths that end inside a run and inside a round of the waves; a
+    row's bits do not depend on the rows beside it."""
+    o = ops()
+    rng = np.random.default_rng(45)
+    a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
+    b = rng.standard_normal(N).astype(np.float32)
+    at, wt = t(a, torch.bfloat16), t(w, torch.bfloat16)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm(out, at, wt, t(b), kernel="rows")
+    close(out, pm.linear(a, w, b), BF16, "store + bias")
+    outf = torch.empty(M, N, device=DEV)
+    o.gemm(outf, at, wt, kernel="rows")
+    close(outf, pm.linear(a, w), 2e-4, "float32 store")
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    acc = t(res)
+    o.gemm(acc, at, wt, add_to_out=True, kernel="rows")
+    close(acc, pm.add(res, pm.linear(a, w)), 2e-4, "residual")
+    onef = torch.empty(1, N, device=DEV)
+    o.gemm(onef, at[M - 1:], wt, kernel="rows")
+    assert torch.equal(onef[0], outf[M - 1])
 
 
 def test_gemm_split_over_blocks_is_repeatable():
