@@ -719,7 +719,7 @@ def test_product_kernel_choice():
     rows or big weights are tiled; a kernel that cannot take the rows is an error, not a guess."""
     o = ops()
     assert o.few_rows_kernel(1, 151936, 896) == "tiled" and o.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "rows"
-    assert o.few_rows_kernel(4, 4608, 3584) == "rows" and o.few_rows_kernel(4, 3584, 18944) == "stream" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
+    assert o.few_rows_kernel(4, 4608, 3584) == "rows" and o.few_rows_kernel(4, 3584, 18944) == "rows" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
     assert o.few_rows_kernel(64, 2 * 4864, 896, swiglu=True) == "tiled" and o.few_rows_kernel(16, 2 * 4864, 896, swiglu=True) == "stream"
     assert o.few_rows_kernel(64, 896, 4864) == "stream" and o.few_rows_kernel(32, 3584, 3584) == "tiled"
     assert o.few_rows_kernel(65, 8, 8) == "tiled"
