@@ -156,6 +156,7 @@ class StepFunction:
         self.n_positions = int(n_positions)
         self.device = model.rt.device
         self._scratch: dict = {}
+        self._views: dict = {}                   # per set of buffers: (name, dtype, shape) -> (buffer, its view of that shape)
         self._eager_scratch = self._scratch      # buffers of steps that run kernel by kernel
         self._retired: list = []                 # outgrown buffers that captured graphs may still use
         self._eager_hosts: list = []             # pinned blocks the eager steps are laid out in, taking turns
@@ -181,11 +182,19 @@ class StepFunction:
     def scratch(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
         """A named buffer re-used from step to step and layer to layer; it grows
         (outside the steady state) when a step is larger than any before."""
+        key = (name, dtype)
+        buf = self._scratch.get(key)
+        # (every layer asks for the same shapes: a buffer's views are kept beside it, and go when it is replaced)
+        views = self._views.setdefault(id(self._scratch), {})
+        shape = tuple(shape)
+        known = views.get(key)
+        if known is not None and known[0] is buf:
+            view = known[1].get(shape)
+            if view is not None:
+                return view
         n = 1
         for s in shape:
             n *= int(s)
-        key = (name, dtype)
-        buf = self._scratch.get(key)
         if buf is None or buf.numel() < n:
             if buf is not None and self._scratch is not self._eager_scratch:
                 # a captured graph may hold this buffer's address (graphs of one batch size share
@@ -194,7 +203,10 @@ class StepFunction:
                 self._retired.append(buf)
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._scratch[key] = buf
-        return buf[:n].view(shape)
+        if known is None or known[0] is not buf or len(known[1]) >= 64:
+            known = views[key] = (buf, {})
+        view = known[1][shape] = buf[:n].view(shape)
+        return view
 
     def scratch_bytes(self) -> int:
         """Bytes of the named buffers (eager steps' and the captured graphs'), retired ones included."""

@@ -32,20 +32,27 @@ def dtype_code(t: torch.Tensor) -> int:
 
 
 def _gpu(name: str, t: torch.Tensor, dtype=None, dims: Optional[int] = None) -> torch.Tensor:
+    # (the checks in the order that a good operand passes fastest: these run some thousand times a step)
+    try:
+        if t.is_cuda and (dtype is None or t.dtype is dtype) and (dims is None or t.dim() == dims):
+            return t
+    except AttributeError:
+        pass
     if not isinstance(t, torch.Tensor) or not t.is_cuda:
         raise AlofaError("invalid_argument", "kernel operand must be a GPU tensor", f"operand={name}")
     if dtype is not None and t.dtype is not dtype:
         raise AlofaError("invalid_argument", "kernel operand has the wrong dtype", f"operand={name} has={t.dtype} wants={dtype}")
-    if dims is not None and t.dim() != dims:
-        raise AlofaError("shape_mismatch", "kernel operand has the wrong rank", f"operand={name} shape={tuple(t.shape)} wants_rank={dims}")
-    return t
+    raise AlofaError("shape_mismatch", "kernel operand has the wrong rank", f"operand={name} shape={tuple(t.shape)} wants_rank={dims}")
 
 
 def _rows(name: str, t: torch.Tensor) -> int:
     """Leading dimension of a 2-d tensor whose rows are contiguous."""
-    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
-        raise AlofaError("shape_mismatch", "kernel operand must be 2-d with contiguous rows", f"operand={name} shape={tuple(t.shape)} strides={t.stride()}")
-    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    strides = t.stride()
+    if len(strides) == 2:
+        rows, columns = t.shape
+        if strides[1] == 1 or columns <= 1:
+            return strides[0] if rows > 1 else max(strides[0], columns)
+    raise AlofaError("shape_mismatch", "kernel operand must be 2-d with contiguous rows", f"operand={name} shape={tuple(t.shape)} strides={t.stride()}")
 
 
 def _contig(name: str, t: torch.Tensor) -> torch.Tensor:
