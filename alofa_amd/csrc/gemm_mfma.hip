@@ -485,13 +485,14 @@ static int launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t 
 
 template <int kEpilogue, typename TO, int WTM, int WTN, int S>
 static int launch_dma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
-                      hipStream_t stream) {
-  const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
+                      hipStream_t stream, const void* W2 = nullptr) {
+  constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? 32 * WTN : 64 * WTN;     // (gate and up rows of the same columns share a slab)
+  const int tiles_n = (N + kOutCols - 1) / kOutCols, tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
   // (tiles dealt out die by die at every size: with weights that come from memory it is 3 to 9 % faster here than row
   // by row also where the operands would fit the L2s: 12.4 against 13.3 us for N = 1,152, K = 896 at 2,048 rows)
   const int by_die = 1;
   gemm_dma_kernel<kEpilogue, TO, WTM, WTN, S><<<tiles_n * tiles_m, 256, 0, stream>>>(
-      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, bias, M, N, K,
+      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
       tiles_m, tiles_n, by_die);
   return 0;
 }
@@ -517,7 +518,17 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     if (M > 64 && static_cast<int64_t>((N + 63) / 64) * ((M + 127) / 128) >= 256) {
       if (launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 63) / 64, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     } else {
-      if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 63) / 64, (M + 63) / 64, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
+      // Tiles of 64 rows x (64 gate + 64 up) columns. With K a multiple of 64 the slabs go straight from memory into a
+      // ring in LDS: of four where K is short (one block per compute unit, and the tiles are fewer than those
+      // anyway; 0.5B sizes: 9.9, 10.6 and 11.4 us at 17, 32 and 64 rows against 11.8, 12.2 and 12.3 through
+      // registers), of three otherwise (7B sizes at 64 rows: 70.8 against 72.5 us).
+      if (K % TK == 0 && K < 2048) {
+        if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+      } else if (K % TK == 0) {
+        if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+      } else {
+        if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 63) / 64, (M + 63) / 64, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
+      }
     }
     return check_launch("gemm_mfma");
   } else {
