@@ -513,22 +513,36 @@ template <int kEpilogue, typename TO>
 static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                        const float* bias, int M, int N, int K, hipStream_t stream) {
   if constexpr (kEpilogue == kMfSwiglu) {
-    // Tiles of 128 rows unless they are fewer than the compute units or half empty. (A tile of 128 x 128
-    // outputs, 256 rows of W, leaves room for one block per compute unit only: slower.)
-    if (M > 64 && static_cast<int64_t>((N + 63) / 64) * ((M + 127) / 128) >= 256) {
+    // A block computes gate and up of the same 64 columns. With K a multiple of 64 and tiles that do not fill the
+    // chip twice over, the slabs go straight from memory into a ring in LDS (0.5B sizes, us against the kernel
+    // that brings them in through registers with 128-row tiles, one slab ahead):
+    //  * up to 64 rows, and further while the tiles of 64 rows are no more than the compute units: such tiles,
+    //    a ring of four where K is short (one block per compute unit), of three otherwise (9.9, 10.6, 11.4, 11.4
+    //    at 17, 32, 64, 192 rows against 11.8, 12.2, 12.3 through registers and 22.4; 7B sizes at 64 rows: 70.8
+    //    against 72.5);
+    //  * then, while the tiles of 128 rows are no more than the compute units: those, a ring of three (14.5 at
+    //    256 rows, 14.8 at 384 against 22.6 and 22.8);
+    //  * up to two such tiles per compute unit: a ring of two, two blocks per compute unit (22.5 at 512 rows,
+    //    23.6 at 768 against 24.1 and 25.4);
+    //  * more tiles: through registers (30.8 at 1,024 rows against 39.9).
+    const int64_t col_tiles = (N + 63) / 64;
+    const int64_t tiles_64 = col_tiles * ((M + 63) / 64), tiles_128 = col_tiles * ((M + 127) / 128);
+    const bool ring = K % TK == 0;
+    if (ring && (M <= 64 || tiles_64 <= 256)) {
+      if (K < 2048) {
+        if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+      } else {
+        if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+      }
+    } else if (ring && tiles_128 <= 256) {
+      if (launch_dma<kEpilogue, TO, 2, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+    } else if (ring && tiles_128 < 512) {
+      if (launch_dma<kEpilogue, TO, 2, 2, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+    } else if (M > 64 && tiles_128 >= 256) {
+      // (a tile of 128 x 128 outputs, 256 rows of W, leaves room for one block per compute unit only: slower)
       if (launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 63) / 64, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     } else {
-      // Tiles of 64 rows x (64 gate + 64 up) columns. With K a multiple of 64 the slabs go straight from memory into a
-      // ring in LDS: of four where K is short (one block per compute unit, and the tiles are fewer than those
-      // anyway; 0.5B sizes: 9.9, 10.6 and 11.4 us at 17, 32 and 64 rows against 11.8, 12.2 and 12.3 through
-      // registers), of three otherwise (7B sizes at 64 rows: 70.8 against 72.5 us).
-      if (K % TK == 0 && K < 2048) {
-        if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
-      } else if (K % TK == 0) {
-        if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
-      } else {
-        if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 63) / 64, (M + 63) / 64, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
-      }
+      if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 63) / 64, (M + 63) / 64, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
     }
     return check_launch("gemm_mfma");
   } else {

@@ -728,6 +728,22 @@ def test_product_kernel_choice():
         o.gemm(torch.empty(70, 16, device=DEV), a, w, kernel="stream")
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 4000, 128), (64, 330, 2112), (190, 1000, 64), (300, 4000, 128), (520, 4000, 192), (1030, 4000, 64), (130, 97, 3584)])
+def test_gate_up_tiled_with_slabs_straight_into_lds(M, N, K):
+    """Gate/up with K a multiple of 64 through the tiled kernel: tiles of 64 rows with a ring of four or three slabs,
+    tiles of 128 rows with a ring of three or two, or slabs through registers, by how many tiles there are; sizes
+    that end inside a tile of rows and of columns."""
+    rng = np.random.default_rng(47)
+    a = bf(rng.standard_normal((M, K)).astype(np.float32))
+    g, u = bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm_swiglu(out, t(a, torch.bfloat16), t(g, torch.bfloat16), t(u, torch.bfloat16), kernel="tiled")
+    close(out, pm.swiglu(pm.linear(a, g), pm.linear(a, u)), BF16, "gate/up")
+    one = torch.empty(1, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm_swiglu(one, t(a[M - 1:], torch.bfloat16), t(g, torch.bfloat16), t(u, torch.bfloat16), kernel="tiled")
+    assert (one[0].float() - out[M - 1].float()).abs().max().item() <= 2e-2 * max(1.0, out[M - 1].float().abs().max().item())
+
+
 def test_gemm_with_operands_beyond_the_l2():
     """Operands of more than 32 MB make the tiled kernel deal its tiles out die by die (another
     numbering of the blocks): every tile must still be computed exactly once, with K shared out
