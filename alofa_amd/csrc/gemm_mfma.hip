@@ -565,16 +565,21 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       if (launch_dma<kEpilogue, TO, 2, 2, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
     } else {
       const int tiles_n = (N + 63) / 64, tiles_m = (M + 63) / 64;
-      const int shares = k_shares(static_cast<int64_t>(tiles_n) * tiles_m, 64 * 64, K);
-      if (shares > 1) {
-        if (launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
-      } else if (K % TK == 0 && K >= 32 * TK && static_cast<int64_t>((M + 127) / 128) * tiles_n > 192 &&
-                 static_cast<int64_t>((M + 127) / 128) * tiles_n <= 256) {
-        // tiles of 128 x 64 that fill the chip just once, and a long K: one block per compute unit with a ring
-        // of four (35.8 against 38.8 us for N = 896, K = 4,864 at 2,048 rows; with a short K, or with more
-        // tiles than compute units, the small tiles below do better: 11.6 against 10.4 us for 896 x 896)
+      const bool ring = K % TK == 0, long_k = K >= 32 * TK;
+      const int64_t tiles_128x64 = static_cast<int64_t>((M + 127) / 128) * tiles_n;
+      // With a short K a share of it is too short to pay for the hand-over: small tiles unshared, slabs straight
+      // from memory (0.5B sizes, 96 to 768 rows: 8.1-8.5 us against 8.8-10.8 for N = 1,152, K = 896).
+      const int shares = (ring && !long_k) ? 1 : k_shares(static_cast<int64_t>(tiles_n) * tiles_m, 64 * 64, K);
+      if (ring && long_k && tiles_128x64 >= 144 && tiles_128x64 <= 256) {
+        // Tiles of 128 x 64 that fill most of the chip once, and a long K: one block per compute unit with a ring
+        // of four (35.8 against 38.8 us for N = 896, K = 4,864 at 2,048 rows; 28.8 against 36.1 with K shared out
+        // for N = 4,608, K = 3,584 at 256 rows, 121 against 151 for N = 3,584, K = 18,944 at 384 rows; fewer tiles
+        // do better with K shared out, 26.1 against 30.3 for 3,584 x 3,584 at 256 rows; with a short K, or with
+        // more tiles than compute units, the small tiles below do better: 11.6 against 10.4 us for 896 x 896)
         if (launch_dma<kEpilogue, TO, 2, 1, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
-      } else if (K % TK == 0) {
+      } else if (shares > 1) {
+        if (launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
+      } else if (ring) {
         // small tiles, slabs straight from memory into a ring of three (against the kernel below, same conditions:
         // 13.3 against 15.8 us for N = 1,152, K = 896; 10.4 against 12.2 for 896 x 896; 38.8 against 44.6 for
         // N = 896, K = 4,864; a ring of two is slower than either when the weights come from memory: 60 us)
