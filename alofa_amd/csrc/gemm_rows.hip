@@ -1,5 +1,6 @@
 // Matrix products for at most eight rows (the decode steps of few requests), bfloat16, on the
-// vector units: out[m, n] = sum_k A[m, k] * W[n, k] with M <= 8.
+// vector units: out[m, n] = sum_k A[m, k] * W[n, k] with M <= 8 (M <= 16 for plain products: bfloat16 rows,
+// store or residual epilogue, K <= 6144).
 //
 // The work is streaming W once from memory, and the time is what a compute unit needs to pull
 // its share, so the shares are made small and even: a block owns C output columns (rows of W,
@@ -94,7 +95,7 @@ __device__ __forceinline__ void lanes_sum(float (&v)[n], int lane) {
 }
 constexpr int log2_of(int n) { return n <= 1 ? 0 : 1 + log2_of(n / 2); }
 
-// MR: rows computed (1, 2, 4, 8; rows beyond M are zeros); C: columns per block; kRwSwiglu: W is the gate
+// MR: rows computed (1, 2, 4, 8, or 16 for plain products; rows beyond M are not stored); C: columns per block; kRwSwiglu: W is the gate
 // matrix and W2 the up matrix, same columns; TO: float or bf16_t; kMaxWaves: bound of the block's waves.
 template <int MR, int C, int kEpilogue, typename TO, bool kNorm, int kMaxWaves>
 __global__ void __launch_bounds__(64 * kMaxWaves) gemm_rows_kernel(
@@ -314,7 +315,7 @@ static int launch_rows(void* out, int64_t ldo, const void* A, int64_t lda, const
   const int waves = (K + 511) / 512;
   const dim3 grid((N + C - 1) / C);
   if (waves > kRowsMaxWaves) {
-    if constexpr (!kNorm && kEpilogue != kRwSwiglu) {
+    if constexpr (!kNorm && kEpilogue != kRwSwiglu && MR <= 8) {
       gemm_rows_long_kernel<MR, C, kEpilogue, TO><<<grid, 64 * rows_long_waves(MR), 0, stream>>>(
           static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), ldw, bias, M, N, K);
       return check_launch("gemm_rows (long K)");
@@ -344,6 +345,9 @@ static int dispatch_rows(void* out, int64_t ldo, const void* A, int64_t lda, con
   if (M <= 1) return launch_rows<1, C, kEpilogue, TO, kNorm>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm_w, eps, stream);
   if (M <= 2) return launch_rows<2, C, kEpilogue, TO, kNorm>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm_w, eps, stream);
   if (M <= 4) return launch_rows<4, C, kEpilogue, TO, kNorm>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm_w, eps, stream);
+  if constexpr (!kNorm && kEpilogue != kRwSwiglu) {
+    if (M > 8) return launch_rows<16, C, kEpilogue, TO, kNorm>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm_w, eps, stream);
+  }
   return launch_rows<8, C, kEpilogue, TO, kNorm>(out, ldo, A, lda, W, W2, ldw, bias, M, N, K, norm_w, eps, stream);
 }
 
@@ -352,9 +356,10 @@ static int dispatch_rows(void* out, int64_t ldo, const void* A, int64_t lda, con
 using namespace alofa;
 
 // Whether alofa_gemm_rows takes these sizes.
-// (K beyond 6,144: the store and residual epilogues of bfloat16 rows only, `plain` then says that this is such a product)
+// (K beyond 6,144, or nine to sixteen rows: the store and residual epilogues of bfloat16 rows only, `plain` then says
+// that this is such a product)
 extern "C" int alofa_gemm_rows_fits(int M, int N, int K, int plain) {
-  return M >= 1 && M <= 8 && N >= 1 && K >= 8 && K % 8 == 0 && (K <= kRowsMaxK || plain);
+  return M >= 1 && (M <= 8 || (plain && M <= 16 && K <= kRowsMaxK)) && N >= 1 && K >= 8 && K % 8 == 0 && (K <= kRowsMaxK || plain);
 }
 
 // The same operands and epilogues as alofa_gemm_skinny (bfloat16 A [M, K] and W [N, K]; W2 for the swiglu epilogue;
@@ -365,7 +370,7 @@ extern "C" int alofa_gemm_rows(void* out, int o_dtype, int64_t ldo, const void* 
                                const void* W2, int64_t ldw, const float* bias, int M, int N, int K, int epilogue,
                                const float* norm_w, float eps, hipStream_t stream) {
   ALOFA_REQUIRE(alofa_gemm_rows_fits(M, N, K, norm_w == nullptr && epilogue != kRwSwiglu),
-                "gemm_rows: M=%d (1..8) N=%d K=%d (a multiple of 8; beyond %d with the store and residual epilogues of bfloat16 rows only)", M, N, K, kRowsMaxK);
+                "gemm_rows: M=%d (1..8; to 16 for plain products of K up to 6,144) N=%d K=%d (a multiple of 8; beyond %d with the store and residual epilogues of bfloat16 rows only)", M, N, K, kRowsMaxK);
   ALOFA_REQUIRE(ldw % 8 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 && (W2 == nullptr || reinterpret_cast<uintptr_t>(W2) % 16 == 0),
                 "gemm_rows: rows of W must be 16-byte aligned");
   ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && lda % (norm_w ? 4 : 8) == 0, "gemm_rows: rows of A must be 16-byte aligned");

@@ -144,11 +144,15 @@ SWIGLU = 2
 
 
 ROWS_MAX_M, ROWS_MAX_K = 8, 6144      # what the vector-unit kernel for very few rows takes (longer rows: plain products only)
+ROWS_MAX_M_PLAIN = 16                 # ... and up to so many rows for plain products of rows up to ROWS_MAX_K
 
 
 def rows_kernel_takes(M: int, K: int, swiglu: bool = False, normed: bool = False) -> bool:
     """Sizes the vector-unit kernel takes: at most eight rows, K a multiple of 8; K beyond 6,144 only for a plain
-    product (bfloat16 rows, store or residual epilogue), which a second kernel loops over."""
+    product (bfloat16 rows, store or residual epilogue), which a second kernel loops over; nine to sixteen rows
+    only for a plain product with K up to 6,144."""
+    if ROWS_MAX_M < M <= ROWS_MAX_M_PLAIN:
+        return K % 8 == 0 and K <= ROWS_MAX_K and not (swiglu or normed)
     return 1 <= M <= ROWS_MAX_M and K % 8 == 0 and (K <= ROWS_MAX_K or not (swiglu or normed))
 USE_ROWS_KERNEL = os.environ.get("ALOFA_ROWS_KERNEL", "1") != "0"
 
@@ -172,7 +176,8 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: b
     against 26.8); at five to eight rows for plain rows up to 32 M (0.5B down 5.2
     against 8.6, 32B output projection 18.3 against 23.2), for float32 rows only up
     to 4 M (0.5B QKV 4.8 against 5.5, 7B QKV 20.5 against 17.1), and never for gate
-    and up together (0.5B: 10.8 against 9.9).
+    and up together (0.5B: 10.8 against 9.9); at nine to sixteen rows for plain rows
+    up to 8 M (0.5B down 6.6 against 8.8, 7B output projection 13.4 against 12.0).
 
     The streaming kernel reads the rows of ``a`` once per 16 or 32 weight rows, so
     its time grows with M; the tiled kernel's hardly does, but it needs more work
@@ -191,7 +196,9 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: b
     if USE_ROWS_KERNEL and rows_kernel_takes(M, K, swiglu, normed):
         if M <= 2 or (M <= 4 and (swiglu or not normed or elements < 24 << 20)):
             return "rows"
-        if M > 4 and not swiglu and elements <= ((4 << 20) if normed else (32 << 20)):
+        if 4 < M <= 8 and not swiglu and elements <= ((4 << 20) if normed else (32 << 20)):
+            return "rows"
+        if M > 8 and elements <= 8 << 20:
             return "rows"
     if M <= 4:
         return "stream"

@@ -10,8 +10,11 @@ def test_product_kernel_by_shape():
     assert ops.few_rows_kernel(65, 8, 8) == "tiled"                               # beyond the streaming kernel's rows
     assert ops.few_rows_kernel(1, 151936, 896) == "tiled"                         # a vocabulary-long matrix, from the first row on
     assert ops.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "rows"         # (not so for the fused gate/up form)
-    for rows in (9, 16, 64):
-        assert ops.few_rows_kernel(rows, 1152, 896) == "stream"                   # 0.5B-sized projections stream from nine rows on
+    for rows in (17, 64):
+        assert ops.few_rows_kernel(rows, 1152, 896) == "stream"                   # 0.5B-sized projections stream from 17 rows on
+    for rows in (9, 16):                                                          # nine to sixteen rows: plain products of small weights only
+        assert ops.few_rows_kernel(rows, 896, 4864) == "rows" and ops.few_rows_kernel(rows, 1152, 896, normed=True) == "stream"
+        assert ops.few_rows_kernel(rows, 2 * 4864, 896, swiglu=True) == "stream" and ops.few_rows_kernel(rows, 3584, 3584) == "stream"
     # at most eight rows: the vector-unit kernel, while the rows it reads once per four columns and its arithmetic stay light
     for rows in (1, 2, 4, 8):
         assert ops.few_rows_kernel(rows, 1152, 896) == "rows" and ops.few_rows_kernel(rows, 896, 4864) == "rows"
@@ -25,7 +28,9 @@ def test_product_kernel_by_shape():
     assert ops.few_rows_kernel(16, 4608, 3584) == "stream" and ops.few_rows_kernel(17, 4608, 3584) == "tiled"
     assert ops._product_entry(None, 8, 896, 4864) == "alofa_gemm_rows" and ops._product_entry("stream", 8, 896, 4864) == "alofa_gemm_skinny"
     with pytest.raises(AlofaError):
-        ops._product_entry("rows", 9, 64, 64)
+        ops._product_entry("rows", 17, 64, 64)
+    with pytest.raises(AlofaError):
+        ops._product_entry("rows", 9, 64, 64, normed=True)
     with pytest.raises(AlofaError):
         ops._product_entry("stream", 65, 64, 64)
     with pytest.raises(AlofaError):

@@ -207,22 +207,26 @@ def test_product_for_very_few_rows(M, N, K):
 def test_product_for_very_few_rows_refuses_what_it_cannot_take():
     o = ops()
     w = torch.zeros(16, 6152, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(AlofaError):          # more rows than eight
-        o.gemm(torch.empty(9, 16, device=DEV), torch.zeros(9, 64, device=DEV, dtype=torch.bfloat16), w[:, :64].contiguous(), kernel="rows")
+    with pytest.raises(AlofaError):          # more rows than sixteen
+        o.gemm(torch.empty(17, 16, device=DEV), torch.zeros(17, 64, device=DEV, dtype=torch.bfloat16), w[:, :64].contiguous(), kernel="rows")
+    with pytest.raises(AlofaError):          # more than eight: plain products only
+        o.gemm_swiglu(torch.empty(9, 16, device=DEV, dtype=torch.bfloat16), torch.zeros(9, 64, device=DEV, dtype=torch.bfloat16), w[:, :64].contiguous(), w[:, :64].contiguous(), kernel="rows")
+    with pytest.raises(AlofaError):          # ... of rows that its waves cover at once
+        o.gemm(torch.empty(9, 16, device=DEV), torch.zeros(9, 6152, device=DEV, dtype=torch.bfloat16), w, kernel="rows")
     with pytest.raises(AlofaError):          # rows longer than its waves cover at once: plain products only, not gate/up
         o.gemm_swiglu(torch.empty(2, 16, device=DEV, dtype=torch.bfloat16), torch.zeros(2, 6152, device=DEV, dtype=torch.bfloat16), w, w, kernel="rows")
     with pytest.raises(AlofaError):          # ... and not with a norm on the way
         o.gemm(torch.empty(2, 16, device=DEV, dtype=torch.bfloat16), torch.zeros(2, 6152, device=DEV), w, norm=(torch.ones(6152, device=DEV), 1e-5), kernel="rows")
     from alofa_amd.csrc.build import load
     fits = load().alofa_gemm_rows_fits
-    assert fits(8, 16, 6144, 0) == 1 and fits(8, 16, 6152, 0) == 0 and fits(8, 16, 6152, 1) == 1 and fits(9, 16, 64, 1) == 0
+    assert fits(8, 16, 6144, 0) == 1 and fits(8, 16, 6152, 0) == 0 and fits(8, 16, 6152, 1) == 1 and fits(9, 16, 64, 0) == 0 and fits(16, 16, 64, 1) == 1 and fits(17, 16, 64, 1) == 0 and fits(9, 16, 6152, 1) == 0
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 130, 18944), (4, 67, 6152), (8, 96, 12296), (3, 40, 27648)])
+@pytest.mark.parametrize("M,N,K", [(1, 130, 18944), (4, 67, 6152), (8, 96, 12296), (3, 40, 27648), (9, 35, 520), (12, 896, 4864), (16, 130, 1544)])
 def test_product_for_very_few_rows_against_long_rows(M, N, K):
-    """K beyond the runs that the waves of a block cover at once: the kernel that loops over them (store with
-    bias, float32 store, residual), at lengths that end inside a run and inside a round of the waves; a
-    row's bits do not depend on the rows beside it."""
+    """The plain forms (store with bias, float32 store, residual) beyond what every form takes: K beyond the runs
+    that the waves of a block cover at once (the kernel that loops over them, at lengths that end inside a run
+    and inside a round of the waves), and nine to sixteen rows; a row's bits do not depend on the rows beside it."""
     o = ops()
     rng = np.random.default_rng(45)
     a, w = bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
