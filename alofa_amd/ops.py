@@ -420,6 +420,9 @@ def decode_waves(d: int) -> int:
     return 8 if d < 128 else 4
 
 
+FORCED_DECODE_PARTS = int(os.environ.get("ALOFA_DECODE_PARTS", "0"))     # for measurements: so many parts whatever the sizes (0: the rule below)
+
+
 def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
     """Parts the keys of a (token, key head) are cut into beyond the waves of a block. A block reads
     its keys at the rate of one compute unit, so while the blocks are far fewer than the compute
@@ -427,9 +430,12 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     parts, which the last block to arrive combines (``decode_hand_over``), if the chip has room for
     eight; then a part per step of all the waves, at most eight (the merge grows with them), and
     from there on a part per two steps, combined by a second kernel; never more parts than fill
-    the chip. (Measured at 14:2 heads of 64 and 28:4 of 128, batches of 1 to 64, contexts of 200
+    the chip, and up to eight steps a wave none where the chip has room for two or three only (two
+    parts gain at the long end of such a context bound what they lose at its short end). (Measured at 14:2 heads of 64 and 28:4 of 128, batches of 1 to 64, contexts of 200
     to 4,000: at 2,000 keys and batch 8, 9.6 us with eight parts against 17.6 with one; at 1,000
     keys 9.2 with four against 11.9.)"""
+    if FORCED_DECODE_PARTS:
+        return FORCED_DECODE_PARTS
     waves = decode_waves(d)
     step = 32 * waves
     if max_context <= 2 * step:
@@ -438,6 +444,8 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     by_chip = max(1, 256 // max(1, blocks))
     if max_context <= 4 * step:
         return 4 if by_chip >= 8 else 1
+    if max_context <= 8 * step and by_chip < 4:
+        return 1
     by_length = -(-max_context // step)
     if by_length > 8:
         by_length = max(8, -(-max_context // (2 * step)))
