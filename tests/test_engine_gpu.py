@@ -126,6 +126,32 @@ def test_long_decoding(replayers, tiny_dirs, dtype):
     assert_close(got, plain_logits(tiny_dirs["C"], tuple(ids)), dtype, "C long decode")
 
 
+@pytest.mark.parametrize("name,n", [("B", 660), ("D", 430)])
+def test_decoding_where_the_parts_of_a_context_are_handed_over(tiny_dirs, name, n):
+    """Contexts of two to four steps of 32 keys a wave (bfloat16): decode attention cuts the keys of a (token, key
+    head) into four parts, and the block that arrives last combines them. Two requests decode side by side at
+    such contexts, the last 40 tokens one by one (captured graphs from the second step on)."""
+    from alofa_amd import ops
+    from alofa_amd.replay import Replayer
+    cfg = TINY[name]
+    d = cfg.get("head_dim", cfg["hidden_size"] // cfg["num_attention_heads"])
+    parts = ops.decode_splits(2, cfg["num_attention_heads"], cfg["num_key_value_heads"], d, 1 << (n - 1).bit_length())
+    assert 1 < parts <= ops.HAND_OVER_MAX_PARTS and ops.decode_hand_over(2, cfg["num_attention_heads"], cfg["num_key_value_heads"], d, parts)
+    ids, other = random_ids(31, n, cfg["vocab_size"]), random_ids(32, n - 70, cfg["vocab_size"])
+    ref, ref_other = plain_logits(tiny_dirs[name], tuple(ids)), plain_logits(tiny_dirs[name], tuple(other))
+    r = Replayer(tiny_dirs[name], "bfloat16", round64(n) + round64(n - 70))
+    tail = 40
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ids[:n - tail], "want": list(range(n - tail))},
+                                     {"id": "b", "tokens": other[:n - 70 - tail], "want": list(range(n - 70 - tail))}], "end": []}]
+    for i in range(tail):
+        steps.append({"step": 1 + i, "entries": [{"id": "a", "tokens": [ids[n - tail + i]], "want": [0]},
+                                                  {"id": "b", "tokens": [other[n - 70 - tail + i]], "want": [0]}],
+                      "end": ["a", "b"] if i == tail - 1 else []})
+    got = collect(r, steps)
+    assert_close(got["a"], ref, "bfloat16", f"{name} a")
+    assert_close(got["b"], ref_other, "bfloat16", f"{name} b")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["B", "C"])
 def test_long_context(tiny_dirs, name, dtype):
