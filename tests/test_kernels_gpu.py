@@ -748,6 +748,62 @@ def test_gate_up_tiled_with_slabs_straight_into_lds(M, N, K):
     assert (one[0].float() - out[M - 1].float()).abs().max().item() <= 2e-2 * max(1.0, out[M - 1].float().abs().max().item())
 
 
+def test_products_at_random_sizes():
+    """Every form of the bfloat16 product (store with bias, float32 store, residual, gate/up, and the norm on the
+    way in) through every kernel that takes the sizes (vector-unit, matrix-core for few rows, tiled, and the one
+    the rule picks), at sizes drawn at random around the kernels' boundaries, against a float32 product of the
+    same operands."""
+    import random
+    o = ops()
+    rnd = random.Random(11)
+    ran = {}
+    for _ in range(150):
+        M = rnd.choice([1, 2, 3, 5, 8, 9, 16, 17, 33, 64, 65, 130, 257, 520])
+        N = rnd.choice([8, 35, 97, 200, 896, 1152, 2049])
+        K = 8 * rnd.choice([1, 5, 16, 33, 64, 112, 193, 608, 770])
+        kind = rnd.choice(["store", "float32 store", "residual", "gate/up", "norm + store", "norm + gate/up"])
+        x = torch.randn(M, K, device=DEV)
+        a = x.to(torch.bfloat16)
+        w, w2 = (torch.randn(N, K, device=DEV).mul_(0.1).to(torch.bfloat16) for _ in range(2))
+        bias, nw = torch.randn(N, device=DEV), torch.rand(K, device=DEV) + 0.5
+        normed = (x * nw).to(torch.bfloat16).float() * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-5)
+        for kernel in ("rows", "stream", "tiled", None):
+            if kind.startswith("norm") and kernel == "tiled":
+                continue
+            try:
+                if kind == "store":
+                    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+                    o.gemm(out, a, w, bias, kernel=kernel)
+                    ref = a.float() @ w.float().T + bias
+                elif kind == "float32 store":
+                    out = torch.full((M, N), float("nan"), device=DEV)
+                    o.gemm(out, a, w, kernel=kernel)
+                    ref = a.float() @ w.float().T
+                elif kind == "residual":
+                    base = torch.randn(M, N, device=DEV)
+                    out = base.clone()
+                    o.gemm(out, a, w, add_to_out=True, kernel=kernel)
+                    ref = base + a.float() @ w.float().T
+                elif kind == "gate/up":
+                    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+                    o.gemm_swiglu(out, a, w, w2, kernel=kernel)
+                    ref = torch.nn.functional.silu(a.float() @ w.float().T) * (a.float() @ w2.float().T)
+                elif kind == "norm + store":
+                    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+                    o.gemm(out, x, w, bias, kernel=kernel, norm=(nw, 1e-5))
+                    ref = normed @ w.float().T + bias
+                else:
+                    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+                    o.gemm_swiglu(out, x, w, w2, kernel=kernel, norm=(nw, 1e-5))
+                    ref = torch.nn.functional.silu(normed @ w.float().T) * (normed @ w2.float().T)
+            except AlofaError:
+                continue              # a kernel that does not take these sizes says so
+            err = ((out.float() - ref).abs().max() / ref.abs().max().clamp_min(1e-6)).item()
+            assert err < (1e-2 if out.dtype is torch.bfloat16 else 1e-4), f"{kind} through {kernel}: M={M} N={N} K={K} relative error {err}"
+            ran[(kind, kernel)] = ran.get((kind, kernel), 0) + 1
+    assert all(ran.get((kind, kernel), 0) > 0 for kind in ("store", "residual", "gate/up") for kernel in ("rows", "stream", "tiled", None)), ran
+
+
 def test_gemm_with_operands_beyond_the_l2():
     """Operands of more than 32 MB make the tiled kernel deal its tiles out die by die (another
     numbering of the blocks): every tile must still be computed exactly once, with K shared out
