@@ -516,7 +516,8 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     // A block computes gate and up of the same 64 columns. With K a multiple of 64 and tiles that do not fill the
     // chip twice over, the slabs go straight from memory into a ring in LDS (0.5B sizes, us against the kernel
     // that brings them in through registers with 128-row tiles, one slab ahead):
-    //  * up to 64 rows, and further while the tiles of 64 rows are no more than the compute units: such tiles,
+    //  * up to 64 rows, and further while the tiles of 64 rows are no more than the compute units: such tiles
+    //    (64 gate + 64 up columns; 128 + 128 for a long and wide pair of matrices, see below),
     //    a ring of four where K is short (one block per compute unit), of three otherwise (9.9, 10.6, 11.4, 11.4
     //    at 17, 32, 64, 192 rows against 11.8, 12.2, 12.3 through registers and 22.4; 7B sizes at 64 rows: 70.8
     //    against 72.5);
@@ -529,7 +530,13 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     const int64_t tiles_64 = col_tiles * ((M + 63) / 64), tiles_128 = col_tiles * ((M + 127) / 128);
     const bool ring = K % TK == 0;
     if (ring && (M <= 64 || tiles_64 <= 256)) {
-      if (K < 2048) {
+      if (K >= 2048 && (N + 127) / 128 >= 192) {
+        // a long and wide pair of matrices: 128 gate + 128 up columns per block, a ring of three, one block per
+        // compute unit; the rows are read half as often (32B sizes: 105, 107, 109 us at 16, 32, 64 rows against
+        // 114, 120, 125; with fewer such tiles than three quarters of the compute units it gains nothing: 7B sizes
+        // 64.1 against 62.4 at 16 rows)
+        if (launch_dma<kEpilogue, TO, 1, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+      } else if (K < 2048) {
         if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
       } else {
         if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;

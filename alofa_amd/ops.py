@@ -173,7 +173,8 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: b
     (w_rows * K in elements): it wins at one and two rows everywhere (0.5B down
     projection 3.6 against 8.3 us, 7B gate/up 47 against 59); at three and four
     rows except with float32 rows against 24 M elements or more (32B QKV: 28.9
-    against 26.8); at five to eight rows for plain rows up to 32 M (0.5B down 5.2
+    against 26.8) and gate and up of 256 M or more (32B: 129 against 105 for the
+    tiled kernel with its wide tiles); at five to eight rows for plain rows up to 32 M (0.5B down 5.2
     against 8.6, 32B output projection 18.3 against 23.2), for float32 rows only up
     to 4 M (0.5B QKV 4.8 against 5.5, 7B QKV 20.5 against 17.1), and never for gate
     and up together (0.5B: 10.8 against 9.9); at nine to sixteen rows for plain rows
@@ -194,14 +195,14 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: b
         return "tiled"
     elements = w_rows * K
     if USE_ROWS_KERNEL and rows_kernel_takes(M, K, swiglu, normed):
-        if M <= 2 or (M <= 4 and (swiglu or not normed or elements < 24 << 20)):
+        if M <= 2 or (M <= 4 and ((swiglu and elements < 256 << 20) or (not swiglu and (not normed or elements < 24 << 20)))):
             return "rows"
         if 4 < M <= 8 and not swiglu and elements <= ((4 << 20) if normed else (32 << 20)):
             return "rows"
         if M > 8 and elements <= 8 << 20:
             return "rows"
     if M <= 4:
-        return "stream"
+        return "tiled" if swiglu and elements >= 256 << 20 else "stream"
     if M <= 8:
         return "tiled" if elements >= 64 << 20 else "stream"
     if M <= 16:

@@ -19,11 +19,13 @@ def test_product_kernel_by_shape():
     for rows in (1, 2, 4, 8):
         assert ops.few_rows_kernel(rows, 1152, 896) == "rows" and ops.few_rows_kernel(rows, 896, 4864) == "rows"
         assert ops.few_rows_kernel(rows, 1152, 896, normed=True) == "rows"
+    assert ops.few_rows_kernel(4, 2 * 27648, 5120, swiglu=True, normed=True) == "tiled" and ops.few_rows_kernel(2, 2 * 27648, 5120, swiglu=True) == "rows"
     assert ops.few_rows_kernel(4, 2 * 4864, 896, swiglu=True, normed=True) == "rows" and ops.few_rows_kernel(5, 2 * 4864, 896, swiglu=True, normed=True) == "stream"
     assert ops.few_rows_kernel(4, 4608, 3584, normed=True) == "rows" and ops.few_rows_kernel(4, 7168, 5120, normed=True) == "stream"
     assert ops.few_rows_kernel(8, 4608, 3584, normed=True) == "stream" and ops.few_rows_kernel(8, 5120, 5120) == "rows"
     assert ops.few_rows_kernel(2, 3584, 18944) == "rows" and ops.few_rows_kernel(4, 3584, 18944) == "rows"    # long rows: its looping form
-    assert ops.few_rows_kernel(2, 2 * 18944, 8192, swiglu=True) == "stream" and ops.few_rows_kernel(2, 1024, 8192, normed=True) == "stream"    # (plain products only)
+    assert ops.few_rows_kernel(2, 2 * 4864, 8192, swiglu=True) == "stream" and ops.few_rows_kernel(2, 1024, 8192, normed=True) == "stream"    # (plain products only)
+    assert ops.few_rows_kernel(2, 2 * 18944, 8192, swiglu=True) == "tiled"        # gate and up of 256 M weights or more: the tiled kernel's wide tiles
     assert ops.few_rows_kernel(8, 3584, 18944) == "tiled"
     assert ops.few_rows_kernel(16, 4608, 3584) == "stream" and ops.few_rows_kernel(17, 4608, 3584) == "tiled"
     assert ops._product_entry(None, 8, 896, 4864) == "alofa_gemm_rows" and ops._product_entry("stream", 8, 896, 4864) == "alofa_gemm_skinny"

@@ -748,6 +748,21 @@ def test_gate_up_tiled_with_slabs_straight_into_lds(M, N, K):
     assert (one[0].float() - out[M - 1].float()).abs().max().item() <= 2e-2 * max(1.0, out[M - 1].float().abs().max().item())
 
 
+def test_gate_up_of_few_rows_against_a_long_and_wide_pair_of_matrices():
+    """The tiled gate/up form with 128 + 128 columns per block (192 such tiles or more, K from 2,048): sizes that end
+    inside a tile, against a float32 product of the same operands."""
+    o = ops()
+    M, N, K = 37, 24700, 2112
+    g = torch.Generator(device="cpu").manual_seed(3)
+    a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
+    wg, wu = (torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16) for _ in range(2))
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    o.gemm_swiglu(out, a, wg, wu, kernel="tiled")
+    ref = torch.nn.functional.silu(a.float() @ wg.float().T) * (a.float() @ wu.float().T)
+    err = ((out.float() - ref).abs().max() / ref.abs().max()).item()
+    assert err < 1e-2, err
+
+
 def test_products_at_random_sizes():
     """Every form of the bfloat16 product (store with bias, float32 store, residual, gate/up, and the norm on the
     way in) through every kernel that takes the sizes (vector-unit, matrix-core for few rows, tiled, and the one
