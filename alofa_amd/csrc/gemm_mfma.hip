@@ -340,8 +340,9 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 
 // The same product with the slabs brought from memory straight into LDS (global_load_lds_dwordx4: every lane's
 // 16 bytes land at consecutive LDS addresses, 1 KB per wave and instruction, no registers and no LDS writes in
-// between) into a ring of S slabs, S - 1 of them on their way while one is multiplied. For K a multiple of 64 and
-// no K shares. Which products take it: see launch_mfma.
+// between) into a ring of S slabs, S - 1 of them on their way while one is multiplied. For K a multiple of 64; with
+// kSplitK a block takes a share of the slabs and the shares meet in the workspace as above. Which products take it:
+// see launch_mfma.
 // A slab is 64 WTM rows of A and 64 WTN rows of W, 128 bytes each, unpadded; the eight 16-byte chunks of a row are
 // permuted by the row's number (chunk c of row r lies at place c ^ swz(r)), which the lane that fetches place p
 // of row r undoes by fetching chunk p ^ swz(r), so that the 16 or 32 rows whose fragments are read together
@@ -349,11 +350,12 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 // Rows beyond M or N are fetched from the last valid row (their results are never stored).
 __device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 
-template <int kEpilogue, typename TO, int WTM, int WTN, int S>
+template <int kEpilogue, typename TO, int WTM, int WTN, int S, bool kSplitK = false>
 __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda,
                                                        const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2, int64_t ldw,
                                                        const float* __restrict__ bias, int M, int N, int K, int tiles_m,
-                                                       int tiles_n, int by_die) {
+                                                       int tiles_n, int by_die, int shares = 1, float* __restrict__ ws = nullptr,
+                                                       int* __restrict__ counters = nullptr) {
   constexpr int TM = 64 * WTM, TN = 64 * WTN;
   constexpr int kGateTiles = WTN / 2;
   static_assert(kEpilogue != kMfSwiglu || WTN % 2 == 0, "the swiglu epilogue needs an even number of column tiles per wave");
@@ -361,7 +363,8 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
   constexpr int kStageBytes = kRows * 128;
   constexpr int kLoads = kRows / 32;           // fetch instructions per wave and slab (each brings eight rows)
   __shared__ __attribute__((aligned(1024))) char ring[S * kStageBytes];
-  const TilePlace place = place_tile(blockIdx.x, tiles_m, tiles_n, 1, by_die != 0);
+  __shared__ int last_block;
+  const TilePlace place = place_tile(blockIdx.x, tiles_m, tiles_n, kSplitK ? shares : 1, by_die != 0);
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int wm = wave / 2, wn = wave % 2;
   constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
@@ -419,7 +422,10 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
     return j * 32 * 128;
   };
 
-  const int slabs = K / TK;
+  // (with K shared out this block takes the slabs first .. slabs - 1 of all)
+  const int all_slabs = K / TK, per_share = kSplitK ? (all_slabs + shares - 1) / shares : all_slabs;
+  const int first = kSplitK ? place.share * per_share : 0;
+  const int slabs = min(first + per_share, all_slabs);
   bf16x8 a[4][WTM], w[4][WTN];
   auto read = [&](int slab) {
     const char* stage = ring + (slab % S) * kStageBytes;
@@ -446,8 +452,8 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
   constexpr int kLead = S - 1;
 #pragma unroll
   for (int p = 0; p < kLead; ++p)
-    if (p < slabs) fetch(p);
-  int k = 0;
+    if (first + p < slabs) fetch(first + p);
+  int k = first;
   for (; k + kLead < slabs; ++k) {
     asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLoads * (kLead - 1)) : "memory");
     __syncthreads();
@@ -460,6 +466,46 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
     __syncthreads();
     read(k);
     multiply();
+  }
+  if constexpr (kSplitK) {
+    // the shares of K meet in the workspace, as in the kernel above
+    const int tile_id = place.bm * tiles_n + place.bn;
+    constexpr int kTileFloats = WTM * WTN * 16 * 256;
+    float* mine = ws + (static_cast<int64_t>(tile_id) * shares + place.share) * kTileFloats;
+#pragma unroll
+    for (int i = 0; i < WTM; ++i)
+#pragma unroll
+      for (int j = 0; j < WTN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          __hip_atomic_store(mine + ((i * WTN + j) * 16 + e) * 256 + tid, acc[i][j][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      const int arrived = atomicAdd(&counters[tile_id], 1);
+      last_block = arrived == shares - 1;
+      if (last_block) atomicExch(&counters[tile_id], 0);
+    }
+    __syncthreads();
+    if (!last_block) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const float* parts = ws + static_cast<int64_t>(tile_id) * shares * kTileFloats;
+#pragma unroll
+    for (int i = 0; i < WTM; ++i)
+#pragma unroll
+      for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int sp = 0; sp < shares; ++sp) {
+          float part[16];
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            part[e] = __hip_atomic_load(parts + static_cast<int64_t>(sp) * kTileFloats + ((i * WTN + j) * 16 + e) * 256 + tid,
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] += part[e];
+        }
+      }
   }
   tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out, ldo, bias, M, N, m0, n0, wm, wn, lane);
 }
@@ -480,6 +526,20 @@ static int launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t 
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W),
       static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, tiles_m, tiles_n, shares, kSplitK ? g_ws.tiles : nullptr,
       kSplitK ? g_ws.counters : nullptr, by_die);
+  return 0;
+}
+
+template <int kEpilogue, typename TO, int WTM, int WTN, int S>
+static int launch_dma_shared(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
+                             int shares, hipStream_t stream) {
+  const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
+  const Workspace& g_ws = workspace();
+  const int64_t tiles = static_cast<int64_t>(tiles_n) * tiles_m;
+  ALOFA_REQUIRE(g_ws.tiles != nullptr && tiles <= g_ws.n_counters && tiles * shares * (WTM * WTN * 16 * 256) <= g_ws.tile_floats,
+                "gemm_mfma: %lld tiles in %d shares of K do not fit the workspace", static_cast<long long>(tiles), shares);
+  gemm_dma_kernel<kEpilogue, TO, WTM, WTN, S, true><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
+      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, bias, M, N, K,
+      tiles_m, tiles_n, 1, shares, g_ws.tiles, g_ws.counters);
   return 0;
 }
 
@@ -585,6 +645,12 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
         // more tiles than compute units, the small tiles below do better: 11.6 against 10.4 us for 896 x 896)
         if (launch_dma<kEpilogue, TO, 2, 1, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
       } else if (shares > 1) {
+        // K shared out among blocks: with weights of 128 MB or more the slabs go straight into a ring of three in
+        // LDS here too (N = 5,120, K = 27,648 at 32 rows: 75 against 85 us; N = 3,584, K = 18,944 at 16 rows: 34.4
+        // against 36.1); smaller ones gain nothing by it (N = 896, K = 4,864 at 96 rows: 19.5 against 18.2)
+        if (ring && static_cast<int64_t>(N) * K * 2 >= (128ll << 20)) {
+          if (launch_dma_shared<kEpilogue, TO, 1, 1, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, shares, stream)) return 1;
+        } else
         if (launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
       } else if (ring) {
         // small tiles, slabs straight from memory into a ring of three (against the kernel below, same conditions:

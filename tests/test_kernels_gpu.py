@@ -763,6 +763,27 @@ def test_gate_up_of_few_rows_against_a_long_and_wide_pair_of_matrices():
     assert err < 1e-2, err
 
 
+def test_few_rows_against_a_big_matrix_with_k_shared_out():
+    """The tiled kernel with K shared out among blocks and the slabs straight into LDS (weights of 128 MB or more):
+    sizes that end inside a tile and a share, residual and store epilogues, against a float32 product."""
+    o = ops()
+    M, N, K = 40, 3600, 18944 + 64
+    g = torch.Generator(device="cpu").manual_seed(4)
+    a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
+    w = torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16)
+    base = torch.randn(M, N, generator=g).to(DEV)
+    acc = base.clone()
+    o.gemm(acc, a, w, add_to_out=True, kernel="tiled")
+    ref = a.float() @ w.float().T
+    assert ((acc - base - ref).abs().max() / ref.abs().max()).item() < 1e-4
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    o.gemm(out, a, w, kernel="tiled")
+    assert ((out.float() - ref).abs().max() / ref.abs().max()).item() < 1e-2
+    again = base.clone()
+    o.gemm(again, a, w, add_to_out=True, kernel="tiled")
+    assert torch.equal(again, acc)                       # the shares are added in a fixed order
+
+
 def test_products_at_random_sizes():
     """Every form of the bfloat16 product (store with bias, float32 store, residual, gate/up, and the norm on the
     way in) through every kernel that takes the sizes (vector-unit, matrix-core for few rows, tiled, and the one
