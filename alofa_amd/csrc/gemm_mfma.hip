@@ -590,11 +590,11 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     const int64_t tiles_64 = col_tiles * ((M + 63) / 64), tiles_128 = col_tiles * ((M + 127) / 128);
     const bool ring = K % TK == 0;
     if (ring && (M <= 64 || tiles_64 <= 256)) {
-      if (K >= 2048 && (N + 127) / 128 >= 192) {
+      if (K >= 2048 && ((N + 127) / 128 >= 192 || ((N + 127) / 128 >= 128 && M > 32))) {
         // a long and wide pair of matrices: 128 gate + 128 up columns per block, a ring of three, one block per
         // compute unit; the rows are read half as often (32B sizes: 105, 107, 109 us at 16, 32, 64 rows against
-        // 114, 120, 125; with fewer such tiles than three quarters of the compute units it gains nothing: 7B sizes
-        // 64.1 against 62.4 at 16 rows)
+        // 114, 120, 125; with fewer such tiles than three quarters of the compute units only from 33 rows on: 7B
+        // sizes, 148 tiles, 64.1 against 62.4 at 16 rows, 67.6 against 70.7 at 64)
         if (launch_dma<kEpilogue, TO, 1, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
       } else if (K < 2048) {
         if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
