@@ -645,10 +645,11 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
         // more tiles than compute units, the small tiles below do better: 11.6 against 10.4 us for 896 x 896)
         if (launch_dma<kEpilogue, TO, 2, 1, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
       } else if (shares > 1) {
-        // K shared out among blocks: with weights of 128 MB or more the slabs go straight into a ring of three in
+        // K shared out among blocks: with weights of 32 MB or more the slabs go straight into a ring of three in
         // LDS here too (N = 5,120, K = 27,648 at 32 rows: 75 against 85 us; N = 3,584, K = 18,944 at 16 rows: 34.4
-        // against 36.1); smaller ones gain nothing by it (N = 896, K = 4,864 at 96 rows: 19.5 against 18.2)
-        if (ring && static_cast<int64_t>(N) * K * 2 >= (128ll << 20)) {
+        // against 36.1; N = 4,608, K = 3,584 at 16 rows: 14.6 against 16.2); smaller ones gain nothing by it
+        // (3,584 x 3,584 at 16 rows: 15.7 against 15.4; N = 896, K = 4,864 at 96 rows: 19.5 against 18.2)
+        if (ring && static_cast<int64_t>(N) * K * 2 >= (32ll << 20)) {
           if (launch_dma_shared<kEpilogue, TO, 1, 1, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, shares, stream)) return 1;
         } else
         if (launch_tile<kEpilogue, TO, 1, 1, 2, true>(tiles_n, tiles_m, shares, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;

@@ -764,7 +764,7 @@ def test_gate_up_of_few_rows_against_a_long_and_wide_pair_of_matrices():
 
 
 def test_few_rows_against_a_big_matrix_with_k_shared_out():
-    """The tiled kernel with K shared out among blocks and the slabs straight into LDS (weights of 128 MB or more):
+    """The tiled kernel with K shared out among blocks and the slabs straight into LDS (weights of 32 MB or more):
     sizes that end inside a tile and a share, residual and store epilogues, against a float32 product."""
     o = ops()
     M, N, K = 40, 3600, 18944 + 64
