@@ -557,6 +557,13 @@ static int launch_dma(void* out, int64_t ldo, const void* A, int64_t lda, const 
   return 0;
 }
 
+// Whether `tiles` blocks that run one per compute unit come out in nearly full rounds of the chip (the last
+// round at least seven eighths full on average over the rounds).
+static bool fills_rounds(int64_t tiles) {
+  const int64_t rounds = (tiles + 255) / 256;
+  return tiles * 8 >= rounds * 256 * 7;
+}
+
 // How many shares of K make `tiles` output tiles (of tile_floats each) fill the chip: doubled while the blocks
 // stay within two per compute unit, every share keeps at least four slabs and the partial tiles fit the workspace.
 static int k_shares(int64_t tiles, int64_t tile_floats, int K) {
@@ -605,6 +612,12 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       if (launch_dma<kEpilogue, TO, 2, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
     } else if (ring && tiles_128 < 512) {
       if (launch_dma<kEpilogue, TO, 2, 2, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+    } else if (ring && K >= 2048 && fills_rounds(static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128))) {
+      // many rows against a long and wide pair of matrices: tiles of 128 rows x (128 gate + 128 up) columns, a ring of
+      // three, one block per compute unit, where such tiles come out in nearly full rounds of the chip (2,048 rows,
+      // 7B sizes: 705 against 738 us; 32B sizes: 1,322 against 1,418; with a short K the tiles below stay ahead:
+      // 0.5B sizes 65.8 against 60.1)
+      if (launch_dma<kEpilogue, TO, 2, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
     } else if (M > 64 && tiles_128 >= 256) {
       // (a tile of 128 x 128 outputs, 256 rows of W, leaves room for one block per compute unit only: slower)
       if (launch_tile<kEpilogue, TO, 2, 2, 1, false>((N + 63) / 64, (M + 127) / 128, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;
@@ -618,6 +631,12 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     // unit, were slower here even with four slabs ahead. Where even the small tiles are too few, K is
     // shared out among blocks as well.
     const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
+    if (M > 64 && K % TK == 0 && K >= 2048 && big_blocks >= 256 && fills_rounds(static_cast<int64_t>((N + 255) / 256) * ((M + 127) / 128))) {
+      // tiles of 128 x 256, a ring of three, one block per compute unit, where such tiles come out in nearly full
+      // rounds of the chip (2,048 rows: 343 against 368 us for N = 3,584, K = 18,944, 198 against 234 for N = 7,168,
+      // K = 5,120; where the last round is half empty they lose: 138 against 121 for N = 4,608, K = 3,584)
+      if (launch_dma<kEpilogue, TO, 2, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
+    } else
     if (M <= 64 && (N + 127) / 128 >= 256) {
       // one tile of rows against a long matrix (the vocabulary): tiles of 64 rows, so that no empty rows are staged
       if (launch_tile<kEpilogue, TO, 1, 2, 2, false>((N + 127) / 128, 1, 1, out, ldo, A, lda, W, W2, ldw, bias, M, N, K, stream)) return 1;

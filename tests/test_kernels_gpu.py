@@ -784,6 +784,32 @@ def test_few_rows_against_a_big_matrix_with_k_shared_out():
     assert torch.equal(again, acc)                       # the shares are added in a fixed order
 
 
+def test_many_rows_in_tiles_of_128_x_256():
+    """The tiled kernel's widest tiles (store, residual and gate/up; K from 2,048 and tile counts that fill rounds of
+    the chip): sizes that end inside a tile, against a float32 product."""
+    o = ops()
+    g = torch.Generator(device="cpu").manual_seed(6)
+    M, N, K = 1990, 3600, 2112                 # 15 x 16 tiles of 128 x 256: 240 of 256
+    a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
+    w = torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16)
+    ref = a.float() @ w.float().T
+    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    bias = torch.randn(N, generator=g).to(DEV)
+    o.gemm(out, a, w, bias, kernel="tiled")
+    assert ((out.float() - ref - bias).abs().max() / ref.abs().max()).item() < 1e-2
+    base = torch.randn(M, N, generator=g).to(DEV)
+    acc = base.clone()
+    o.gemm(acc, a, w, add_to_out=True, kernel="tiled")
+    assert ((acc - base - ref).abs().max() / ref.abs().max()).item() < 1e-4
+    M, N = 1990, 3800                          # gate/up: 16 x 30 tiles of 128 x (128 + 128): 480 of 512
+    a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
+    wg, wu = (torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16) for _ in range(2))
+    act = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    o.gemm_swiglu(act, a, wg, wu, kernel="tiled")
+    ref = torch.nn.functional.silu(a.float() @ wg.float().T) * (a.float() @ wu.float().T)
+    assert ((act.float() - ref).abs().max() / ref.abs().max()).item() < 1e-2
+
+
 def test_products_at_random_sizes():
     """Every form of the bfloat16 product (store with bias, float32 store, residual, gate/up, and the norm on the
     way in) through every kernel that takes the sizes (vector-unit, matrix-core for few rows, tiled, and the one
