@@ -631,7 +631,19 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     // unit, were slower here even with four slabs ahead. Where even the small tiles are too few, K is
     // shared out among blocks as well.
     const int64_t big_blocks = static_cast<int64_t>((N + 127) / 128) * ((M + 127) / 128);
-    if (M > 64 && K % TK == 0 && K >= 2048 && big_blocks >= 256 && fills_rounds(static_cast<int64_t>((N + 255) / 256) * ((M + 127) / 128))) {
+    const int64_t tiles_192 = static_cast<int64_t>((N + 191) / 192) * ((M + 127) / 128);
+    const int64_t tiles_256 = static_cast<int64_t>((N + 255) / 256) * ((M + 127) / 128);
+    const int64_t rounds_192 = (tiles_192 + 255) / 256, rounds_256 = (tiles_256 + 255) / 256;
+    if (M > 64 && K % TK == 0 && K >= 2048 && rounds_192 * 192 < rounds_256 * 256 &&
+        (rounds_192 == 1 ? tiles_192 >= 128 : tiles_192 * 16 >= rounds_192 * 256 * 13)) {
+      // tiles of 128 x 192, a ring of three, one block per compute unit, where their rounds of the chip cover
+      // fewer columns than those of the 256-wide tiles below and are full enough: a single round on half of the
+      // compute units or more (1,024 rows: 235 against 307 us for N = 3,584, K = 18,944, 390 against 500 for
+      // N = 5,120, K = 27,648, 61 against 75 for N = 4,608, K = 3,584), or several at least 13/16 full (2,048 rows:
+      // 762 against 825 for N = 5,120, K = 27,648; 4,096 rows: 189 against 203 for N = 4,608, K = 3,584)
+      if (launch_dma<kEpilogue, TO, 2, 3, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream)) return 1;
+    } else
+    if (M > 64 && K % TK == 0 && K >= 2048 && big_blocks >= 256 && fills_rounds(tiles_256)) {
       // tiles of 128 x 256, a ring of three, one block per compute unit, where such tiles come out in nearly full
       // rounds of the chip (2,048 rows: 343 against 368 us for N = 3,584, K = 18,944, 198 against 234 for N = 7,168,
       // K = 5,120; where the last round is half empty they lose: 138 against 121 for N = 4,608, K = 3,584)

@@ -785,8 +785,9 @@ def test_few_rows_against_a_big_matrix_with_k_shared_out():
 
 
 def test_many_rows_in_tiles_of_128_x_256():
-    """The tiled kernel's widest tiles (store, residual and gate/up; K from 2,048 and tile counts that fill rounds of
-    the chip): sizes that end inside a tile, against a float32 product."""
+    """The tiled kernel's widest tiles (128 x 256 and 128 x 192 for store and residual, 128 x (128 + 128) for gate/up;
+    K from 2,048 and tile counts that fill rounds of the chip): sizes that end inside a tile, against a float32
+    product."""
     o = ops()
     g = torch.Generator(device="cpu").manual_seed(6)
     M, N, K = 1990, 3600, 2112                 # 15 x 16 tiles of 128 x 256: 240 of 256
@@ -801,6 +802,18 @@ def test_many_rows_in_tiles_of_128_x_256():
     acc = base.clone()
     o.gemm(acc, a, w, add_to_out=True, kernel="tiled")
     assert ((acc - base - ref).abs().max() / ref.abs().max()).item() < 1e-4
+    for M, N in ((1000, 3700), (1990, 5100)):  # tiles of 128 x 192: 8 x 20 in one round; 16 x 27 = 432 of 512
+        a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
+        w = torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16)
+        ref = a.float() @ w.float().T
+        out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+        bias = torch.randn(N, generator=g).to(DEV)
+        o.gemm(out, a, w, bias, kernel="tiled")
+        assert ((out.float() - ref - bias).abs().max() / ref.abs().max()).item() < 1e-2
+        base = torch.randn(M, N, generator=g).to(DEV)
+        acc = base.clone()
+        o.gemm(acc, a, w, add_to_out=True, kernel="tiled")
+        assert ((acc - base - ref).abs().max() / ref.abs().max()).item() < 1e-4
     M, N = 1990, 3800                          # gate/up: 16 x 30 tiles of 128 x (128 + 128): 480 of 512
     a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
     wg, wu = (torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16) for _ in range(2))
