@@ -607,11 +607,25 @@ def prefill_share(heads: int, kv_heads: int, d: int, runs: int) -> int:
     return int(load().alofa_attention_prefill_share(_I(heads), _I(kv_heads), _I(d), _I(runs), _I(compute_units())))
 
 
-def prefill_blocks_per_run(heads: int, kv_heads: int, share: int) -> int:
+PREFILL_ROWS_16_ONLY = os.environ.get("ALOFA_PREFILL_ROWS") == "16"   # the prefill kernel's 16-row form everywhere
+
+
+def prefill_rows(heads: int, kv_heads: int, d: int, share: int, runs: int) -> int:
+    """Query rows a wave of the prefill attention kernel owns when it serves ``runs`` runs: 32 where
+    ``share`` heads share their tiles, the head size is 32, 64 or 96 and the blocks of 32 rows are
+    at least one and a half per compute unit (the kernel's own rule), else 16."""
+    if PREFILL_ROWS_16_ONLY:
+        return 16
+    return int(load().alofa_attention_prefill_rows(_I(heads), _I(kv_heads), _I(d), _I(share), _I(runs), _I(compute_units())))
+
+
+def prefill_blocks_per_run(heads: int, kv_heads: int, share: int, rows: int = 16) -> int:
     """Blocks of the prefill attention kernel that serve one run of up to 64 rows: one per query
-    head, or, where ``share`` heads of a group share their tiles, four blocks of 16 rows per chunk
-    of that many heads."""
-    return kv_heads * -(-(heads // kv_heads) // share) * 4 if share else heads
+    head, or, where ``share`` heads of a group share their tiles, per chunk of that many heads
+    four blocks of 16 rows or two of 32 (``rows`` from ``prefill_rows``)."""
+    if not share:
+        return heads
+    return kv_heads * -(-(heads // kv_heads) // share) * (64 // rows)
 
 
 def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = None) -> list:
@@ -637,12 +651,14 @@ def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = 
     return out
 
 
-def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale, share: int = 0) -> None:
+def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale, share: int = 0,
+                      rows: int = 16) -> None:
     """bfloat16 attention for portions of prompts. ``tiles`` is int32 [n, 2, 4]
     from ``pair_tiles``: per block up to two runs of rows, each (request index,
     first row, rows <= 64 or 0 for none, position of the first row). ``share``
     (from ``prefill_share``; the tiles were paired for its count of blocks):
-    that many heads of a group are served from one staged tile."""
+    that many heads of a group are served from one staged tile. ``rows``: query rows a wave owns
+    (from ``prefill_rows``; the tiles were paired for it too)."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     if d not in PREFILL_HEAD_DIMS:
         raise AlofaError("unsupported", "the prefill attention kernel is not built for this head size", f"head_dim={d} built={PREFILL_HEAD_DIMS}")
@@ -651,7 +667,7 @@ def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_he
         raise AlofaError("shape_mismatch", "tiles must be [n, 2, 4]", f"tiles={tuple(tiles.shape)}")
     _call("alofa_attention_prefill", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
           _ptr(block_table), _I(block_table.shape[1]), _ptr(tiles), _I(tiles.shape[0]), _I(heads), _I(kv_heads), _I(d), _I(bs),
-          _I(int(window or 0)), _F(scale), _I(share), _stream())
+          _I(int(window or 0)), _F(scale), _I(share), _I(rows), _stream())
 
 
 # ------------------------------------------------------------------ sampling

@@ -45,13 +45,15 @@ class RowPlan:
                                                dtype=torch.int32, device=self.device)
 
     def tiles(self, heads: int, kv_heads: int, d: int, window):
-        """The runs as blocks of the prefill kernel for a mixer with these head counts, and how many
-        heads of a group share a block's tiles (both depend on how many blocks there are)."""
+        """The runs as blocks of the prefill kernel for a mixer with these head counts, how many heads
+        of a group share a block's tiles and how many rows a wave owns (all three depend on how many
+        blocks there are)."""
         key = (heads, kv_heads, d, window)
         if key not in self._tiles:
             share = ops.prefill_share(heads, kv_heads, d, len(self.long_runs))
-            per_run = ops.prefill_blocks_per_run(heads, kv_heads, share)
-            self._tiles[key] = (torch.tensor(ops.pair_tiles(self.long_runs, window, per_run), dtype=torch.int32, device=self.device), share)
+            rows = ops.prefill_rows(heads, kv_heads, d, share, len(self.long_runs))
+            per_run = ops.prefill_blocks_per_run(heads, kv_heads, share, rows)
+            self._tiles[key] = (torch.tensor(ops.pair_tiles(self.long_runs, window, per_run), dtype=torch.int32, device=self.device), share, rows)
         return self._tiles[key]
 
 
@@ -144,8 +146,8 @@ class GQAAttention(Mixer):
             ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
         else:
             if plan.long_runs is not None:      # portions of prompts
-                tiles, share = plan.tiles(self.heads, self.kv_heads, self.d, self.window)
-                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, tiles, *common, share=share)
+                tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window)
+                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, tiles, *common, share=share, rows=rows)
             if plan.n_short:                    # single tokens and very short portions, all query heads of a key head together
                 floats = ops.decode_scratch_floats(plan.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
                 partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
