@@ -81,11 +81,13 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
   constexpr int kStageBytes = (BKV * KROW + (RW == 32 ? 32 * OT : d) * VROW) * 2, kStateBytes = kTeamThreads * (OV * OT + 2) * 4;
   constexpr int kTeamBytes = (((TEAMS > 1 && kStateBytes > kStageBytes) ? kStateBytes : kStageBytes) + 15) / 16 * 16;   // (one team hands no state over)
   __shared__ __attribute__((aligned(16))) char team_room[TEAMS * kTeamBytes];
-  const int team = threadIdx.x / kTeamThreads;
+  // (the wave's number as a scalar: what depends on it alone, the team's tile and whether it is whole, then stays out of the vector unit)
+  const int wave_of_block = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  const int team = wave_of_block / WPT;
   bf16_t* Ks = reinterpret_cast<bf16_t*>(team_room + team * kTeamBytes);
   bf16_t* Vt = Ks + BKV * KROW;
 
-  const int tid = threadIdx.x % kTeamThreads, wave = tid / 64, lane = tid % 64;
+  const int wave = wave_of_block % WPT, lane = threadIdx.x % 64, tid = wave * 64 + lane;
   const int c16 = lane % 16, g = lane / 16;
   const int r32 = lane % 32, h = lane / 32;
   const int group = heads / kv_heads, chunks = (group + WPT - 1) / WPT;
