@@ -54,20 +54,21 @@ __device__ __forceinline__ float halves_sum(float v) {
 }
 
 constexpr int BQ = 64;    // query rows per block
-constexpr int BKV = 64;   // keys per tile
 constexpr int KPAD = 8, VPAD = 8;
 
 // tiles: int32 [n_blocks, 2, 4]: a block serves up to two runs of rows, one after the other, each
 // (request index, first row in the packed batch, rows (<= 64; 0: none), position of the first row). The caller
 // pairs long runs with short ones so that blocks carry about the same number of key tiles.
 // kShare: blockIdx.y = key head * chunks + chunk of up to WPT query heads of its group; blockIdx.z = which RW rows of the run.
-template <int DT, int TEAMS, int WPT, bool kShare, int RW = 16>  // DT = d / 16; RW: query rows per wave (16 or 32)
+template <int DT, int TEAMS, int WPT, bool kShare, int RW = 16, int KT = 64>  // DT = d / 16; RW: query rows per wave (16 or 32); KT: keys per tile (64; 32 with RW = 32)
 __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAMS <= 256) ? 2 : 1) attention_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
     int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int bs_shift, int window,
     float scale) {
   constexpr int d = DT * 16;
+  constexpr int BKV = KT;
+  static_assert(KT == 64 || (KT == 32 && RW == 32), "tiles of 64 keys, or of 32 with 32 rows a wave");
   constexpr int DS = RW == 32 ? DT : (d + 31) / 32;   // steps of 32 (RW = 32: of 16) along d in the first product
   constexpr int OT = RW == 32 ? (d + 31) / 32 : DT;   // output tiles of 16 (RW = 32: of 32) channels
   constexpr int OV = RW == 32 ? 16 : 4;               // ... each this many values per lane
@@ -147,7 +148,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
   int k_page[kPerThread], v_page[kPerThread];
   auto chunk_of = [&](int j) { const int c = tid + kTeamThreads * j; return c < kChunks ? c : kChunks - 1; };
   auto k_key = [&](int t, int j) { return t * BKV + chunk_of(j) / (d / 8); };
-  auto v_key0 = [&](int t, int j) { return t * BKV + (chunk_of(j) % 8) * 8; };
+  auto v_key0 = [&](int t, int j) { return t * BKV + (chunk_of(j) % (BKV / 8)) * 8; };
   auto clamp = [](int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); };
   auto lookup = [&](int t) {
 #pragma unroll
@@ -169,7 +170,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) {
       const int c = chunk_of(j);
-      const int key0 = clamp(v_key0(t, j), v_first, v_last), channel = c / 8;
+      const int key0 = clamp(v_key0(t, j), v_first, v_last), channel = c / (BKV / 8);
       v_reg[j] = *reinterpret_cast<const uint4*>(
           v_cache + (((static_cast<int64_t>(v_page[j]) * kv_heads + hk) * d + channel) << bs_shift) + (key0 & page_mask));
     }
@@ -201,12 +202,12 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
           vv = make_uint4(w[0], w[1], w[2], w[3]);
         }
         *reinterpret_cast<uint4*>(&Ks[(c / (d / 8)) * KROW + (c % (d / 8)) * 8]) = kv;
-        // row c / 8 of V^T, keys 8 (c % 8) .. + 7. Groups of four keys are permuted within a row by the row's
+        // row c / 8 of V^T, keys 8 (c % 8) .. + 7 (with tiles of 64 keys). Groups of four keys are permuted within a row by the row's
         // number / 8, so that lanes reading rows r and r + 8 hit different banks: the two groups of this chunk
         // stay in their 16 bytes and change places when that number is odd.
-        const int sw = ((c / 8) >> 3) & 7;
+        const int row = c / (BKV / 8), sw = (row >> 3) & 7;
         if (sw & 1) vv = make_uint4(vv.z, vv.w, vv.x, vv.y);
-        *reinterpret_cast<uint4*>(&Vt[(c / 8) * VROW + ((((c % 8) * 2) ^ (sw & 6)) << 2)]) = vv;
+        *reinterpret_cast<uint4*>(&Vt[row * VROW + ((((c % (BKV / 8)) * 2) ^ (sw & 6)) << 2)]) = vv;
       }
     }
   };
@@ -230,10 +231,11 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
     if (!head_ok) continue;     // (a wave without a head of its own has done its share of the staging)
 
     if constexpr (RW == 32) {
-    // S^T for the two 32-key halves of the tile
-    f32x16 s[2];
+    // S^T for the 32-key halves of the tile
+    constexpr int KH = BKV / 32;
+    f32x16 s[KH];
 #pragma unroll
-    for (int kh = 0; kh < 2; ++kh) {
+    for (int kh = 0; kh < KH; ++kh) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[kh][e] = 0.f;
 #pragma unroll
@@ -243,25 +245,25 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
       }
     }
     // scale, mask, running maximum, as below; element i of this lane: key 32 (i / 16) + 8 ((i % 16) / 4) + 4 h + i % 4 of the tile
-    float p[32];
+    float p[16 * KH];
     float tile_max = -FLT_MAX;
     const bool whole = t * BKV + BKV - 1 <= pos0 && (window <= 0 || t * BKV > last_pos - window);
     float corr, sum = 0.f;
     if (whole) {
 #pragma unroll
-      for (int i = 0; i < 32; ++i) tile_max = fmaxf(tile_max, s[i / 16][i % 16]);
+      for (int i = 0; i < 16 * KH; ++i) tile_max = fmaxf(tile_max, s[i / 16][i % 16]);
       tile_max = halves_max(tile_max);   // over the two lanes that share the query row
       const float m_new = fmaxf(m, tile_max * scale2);
       corr = __builtin_amdgcn_exp2f(m - m_new);
       m = m_new;
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
+      for (int i = 0; i < 16 * KH; ++i) {
         p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[i / 16][i % 16], scale2, -m_new));
         sum += p[i];
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
+      for (int i = 0; i < 16 * KH; ++i) {
         const int key = t * BKV + (i / 16) * 32 + ((i % 16) / 4) * 8 + h * 4 + i % 4;
         const bool seen = key <= my_pos && (window <= 0 || key > my_pos - window);
         p[i] = seen ? s[i / 16][i % 16] * scale2 : -FLT_MAX;
@@ -272,7 +274,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
       corr = __builtin_amdgcn_exp2f(m - m_new);
       m = m_new;
 #pragma unroll
-      for (int i = 0; i < 32; ++i) {
+      for (int i = 0; i < 16 * KH; ++i) {
         p[i] = (p[i] > -FLT_MAX) ? __builtin_amdgcn_exp2f(p[i] - m_new) : 0.f;
         sum += p[i];
       }
@@ -282,21 +284,23 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
       fetch_values(t + TEAMS);
       lookup(t + 2 * TEAMS);
     }
-    bf16x8 pf[4];         // the weights of keys 16 x .. 16 x + 15 of the tile, in this lane's order
+    bf16x8 pf[2 * KH];    // the weights of keys 16 x .. 16 x + 15 of the tile, in this lane's order
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
+    for (int x = 0; x < 2 * KH; ++x) {
       const uint4 w = make_uint4(pack_bf16x2(p[8 * x], p[8 * x + 1]), pack_bf16x2(p[8 * x + 2], p[8 * x + 3]),
                                  pack_bf16x2(p[8 * x + 4], p[8 * x + 5]), pack_bf16x2(p[8 * x + 6], p[8 * x + 7]));
       pf[x] = __builtin_bit_cast(bf16x8, w);
     }
     // O^T += V^T P^T, one MFMA per 16 keys: this lane's slots are keys 16 x + 4 h .. + 3 and 16 x + 8 + 4 h .. + 3
+    // (leaving the outputs alone where no row's maximum moved, a branch of the wave, is slower: 1.76 against 1.56 ms
+    // for 40/8 heads of size 128 and 16k keys)
 #pragma unroll
     for (int nt = 0; nt < OT; ++nt) {
       o[nt] *= corr;
       const bf16_t* vrow = &Vt[(nt * 32 + r32) * VROW];
       const int sw = ((nt * 4 + (r32 >> 3)) & 7) << 2;   // this row's permutation of its four-key groups
 #pragma unroll
-      for (int x = 0; x < 4; ++x) {
+      for (int x = 0; x < 2 * KH; ++x) {
         const uint2 lo = *reinterpret_cast<const uint2*>(vrow + ((x * 16 + h * 4) ^ sw));
         const uint2 hi = *reinterpret_cast<const uint2*>(vrow + ((x * 16 + 8 + h * 4) ^ sw));
         const uint4 vv = make_uint4(lo.x, lo.y, hi.x, hi.y);
@@ -474,9 +478,18 @@ extern "C" int alofa_attention_prefill_share(int heads, int kv_heads, int d, int
 // (14/2 heads of size 64, 2,048 tokens: 32.9 against 32.1 us). Blocks of 32 rows are half as many and a compute
 // unit holds one of them: below one and a half blocks per compute unit the 16-row form's smaller blocks spread
 // prompts' unequal runs better (two prompts of 2,048 tokens: 64 against 56 us; one of 4,096: 117 against 100).
-extern "C" int alofa_attention_prefill_rows_fit(int d, int share) { return share > 0 && d % 32 == 0 && d <= 96; }
+// At head size 128 the state of 32 rows fits beside a tile of 32 keys on its way (tiles of 64: spills, 4.3 against
+// 1.6 ms for 40/8 heads and 16k keys): where every head has blocks of its own, a block of two teams of two waves,
+// in launches of at least two blocks per compute unit (40/8 heads, 2,048 rows: 133 against 146 us at 2,048 keys,
+// 1.56 against 1.67 ms at 16k; 4,096 rows at 16k: 2.33 against 2.60 ms; with fewer blocks the four-wave blocks
+// leave compute units idle, 16/16 heads and 2,048 rows: 65 against 56 us); with shared tiles it gains 1 to 3 %
+// and is left out.
+extern "C" int alofa_attention_prefill_rows_fit(int d, int share) {
+  return share > 0 ? (d % 32 == 0 && d <= 96) : d == 128;
+}
 extern "C" int alofa_attention_prefill_rows(int heads, int kv_heads, int d, int share, int runs, int compute_units) {
   if (!alofa_attention_prefill_rows_fit(d, share) || heads <= 0 || kv_heads <= 0) return 16;
+  if (share == 0) return static_cast<int64_t>(runs) * heads >= 4 * static_cast<int64_t>(compute_units) ? 32 : 16;   // (two runs a block)
   const int group = heads / kv_heads, chunks = (group + share - 1) / share;
   return static_cast<int64_t>(runs) * kv_heads * chunks * 2 * 2 >= 3 * static_cast<int64_t>(compute_units) ? 32 : 16;
 }
@@ -504,14 +517,14 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
                 width, group, d);
   const int chunks = width ? (group + width - 1) / width : 0;
   ALOFA_REQUIRE(rows_per_wave == 16 || (rows_per_wave == 32 && alofa_attention_prefill_rows_fit(d, width)),
-                "attention_prefill: %d rows a wave at head size %d with %d heads sharing their tiles (16 always; 32 with shared tiles and head sizes 32, 64, 96)",
+                "attention_prefill: %d rows a wave at head size %d with %d heads sharing their tiles (16 always; 32 with shared tiles and head sizes 32, 64, 96, and without at head size 128)",
                 rows_per_wave, d, width);
 #define ALOFA_PREFILL_AS(DT, TEAMS, WPT, SHARE, GRID)                                                                         \
   attention_prefill_kernel<DT, TEAMS, WPT, SHARE><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(                                    \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
       static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
 #define ALOFA_PREFILL_AS32(DT, TEAMS, WPT, SHARE, GRID)                                                                       \
-  attention_prefill_kernel<DT, TEAMS, WPT, SHARE, 32><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(                                \
+  attention_prefill_kernel<DT, TEAMS, WPT, SHARE, 32, (DT > 6 ? 32 : 64)><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(            \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
       static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
 #define ALOFA_PREFILL_WIDE32(DT, WPT)                                                                            \
@@ -528,6 +541,7 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
       case 2: ALOFA_PREFILL32(2); break;
       case 4: ALOFA_PREFILL32(4); break;
       case 6: ALOFA_PREFILL32(6); break;
+      case 8: ALOFA_PREFILL_AS32(8, 2, 2, false, dim3(n_tiles, heads)); break;
     }
     return check_launch("attention_prefill");
   }

@@ -613,7 +613,8 @@ PREFILL_ROWS_16_ONLY = os.environ.get("ALOFA_PREFILL_ROWS") == "16"   # the pref
 def prefill_rows(heads: int, kv_heads: int, d: int, share: int, runs: int) -> int:
     """Query rows a wave of the prefill attention kernel owns when it serves ``runs`` runs: 32 where
     ``share`` heads share their tiles, the head size is 32, 64 or 96 and the blocks of 32 rows are
-    at least one and a half per compute unit (the kernel's own rule), else 16."""
+    at least one and a half per compute unit, or where no heads share, the head size is 128 and
+    the blocks are at least two per compute unit (the kernel's own rule), else 16."""
     if PREFILL_ROWS_16_ONLY:
         return 16
     return int(load().alofa_attention_prefill_rows(_I(heads), _I(kv_heads), _I(d), _I(share), _I(runs), _I(compute_units())))

@@ -568,7 +568,8 @@ def test_prefill_attention(heads, kv_heads, d, bs, window):
     one head, or, in launches with many blocks and six or more query heads per key head (head sizes up
     to 128), 16 rows of the heads of a group, which share the staged tiles (groups of six to eight in
     teams of as many waves, eleven in chunks of six and five), or 32 rows of them where the head size is 32,
-    64 or 96: every form is run where it exists."""
+    64 or 96; at head size 128 a block of one head also comes with 32 rows a wave and tiles of 32 keys: every
+    form is run where it exists."""
     rng = np.random.default_rng(23)
     lens, q_lens = [37, 130, 700, 64, 65, 200], [37, 5, 100, 64, 65, 200]
     c = paged_case(rng, lens, q_lens, heads, kv_heads, d, bs, torch.bfloat16)
@@ -590,22 +591,24 @@ def test_prefill_attention(heads, kv_heads, d, bs, window):
     assert ops().prefill_share(heads, kv_heads, d, 1) == 0
     assert wide == {1: 0, 2: 0, 3: 0, 5: 0, 6: 6 if d <= 128 else 0, 7: 7, 8: 8, 11: 6}[group]
     rows32 = bool(wide) and d in (32, 64, 96)
-    assert ops().prefill_rows(heads, kv_heads, d, wide, 1 << 20) == (32 if rows32 else 16) and ops().prefill_rows(heads, kv_heads, d, 0, 1 << 20) == 16
+    assert ops().prefill_rows(heads, kv_heads, d, wide, 1 << 20) == (32 if rows32 or (d == 128 and not wide) else 16)
+    assert ops().prefill_rows(heads, kv_heads, d, 0, 1 << 20) == (32 if d == 128 else 16) and ops().prefill_rows(heads, kv_heads, d, 0, 1) == 16
     if rows32:     # blocks of 32 rows from one and a half per compute unit on
         per_run, cus = kv_heads * -(-group // wide) * 2, ops().compute_units()
         assert ops().prefill_rows(heads, kv_heads, d, wide, -(-3 * cus // (2 * per_run))) == 32
         assert ops().prefill_rows(heads, kv_heads, d, wide, -(-3 * cus // (2 * per_run)) - 1) == 16
     assert ops().prefill_blocks_per_run(heads, kv_heads, wide) == (kv_heads * -(-group // wide) * 4 if wide else heads)
     assert ops().prefill_blocks_per_run(heads, kv_heads, wide, 32) == (kv_heads * -(-group // wide) * 2 if wide else heads)
-    for share, rows in [(0, 16)] + ([(wide, 16)] if wide else []) + ([(wide, 32)] if rows32 else []):
+    for share, rows in [(0, 16)] + ([(0, 32)] if d == 128 else []) + ([(wide, 16)] if wide else []) + ([(wide, 32)] if rows32 else []):
         for name, blocks in (("paired", paired), ("single", single)):
             out.zero_()
             ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(blocks, np.int32), torch.int32), heads, kv_heads, d, window, scale,
                                     share=share, rows=rows)
             close(out, ref, BF16, f"prefill attention, {name}, {share} heads share, {rows} rows a wave")
-    with pytest.raises(Exception, match="rows a wave"):
-        ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(single, np.int32), torch.int32), heads, kv_heads, d, window, scale,
-                                share=0, rows=32)
+    if d != 128 or wide:
+        with pytest.raises(Exception, match="rows a wave"):
+            ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(single, np.int32), torch.int32), heads, kv_heads, d, window, scale,
+                                    share=wide if d == 128 else 0, rows=32)
     with pytest.raises(Exception, match="cannot share"):
         ops().attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(single, np.int32), torch.int32), heads, kv_heads, d, window, scale,
                                 share=5)
