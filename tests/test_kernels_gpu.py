@@ -48,7 +48,7 @@ def test_embed_gather(dtype):
     assert np.array_equal(out.cpu().numpy(), pm.embed(table, ids))
 
 
-@pytest.mark.parametrize("width", [80, 896, 1000, 1026, 2044, 3584, 5120, 8192, 9000])     # rows kept in registers (multiples of four up to 8,192) and rows read twice
+@pytest.mark.parametrize("width", [80, 896, 1000, 1024, 1026, 2044, 3584, 5120, 8192, 9000])     # rows kept in registers (multiples of four up to 8,192) and rows read twice
 def test_rmsnorm(width):
     rng = np.random.default_rng(1)
     x = (rng.standard_normal((9, width)) * 3).astype(np.float32)
@@ -63,6 +63,9 @@ def test_rmsnorm(width):
     outg = torch.empty(4, width, device=DEV)
     ops().rmsnorm(outg, t(x), t(w), 1e-5, True, t(rows, torch.int32))
     close(outg, pm.rmsnorm(x[rows], w, 1e-5), EXACT, "gather")
+    outgb = torch.empty(4, width, device=DEV, dtype=torch.bfloat16)
+    ops().rmsnorm(outgb, t(x), t(w), 1e-5, False, t(rows, torch.int32))
+    close(outgb, pm.rmsnorm(x[rows], w, 1e-5), BF16, "bf16 gather")
 
 
 SHAPES = [(1, 100, 72), (5, 130, 200), (70, 33, 264), (130, 257, 48), (3, 64, 1000), (300, 200, 136), (64, 300, 96), (65, 129, 40)]
