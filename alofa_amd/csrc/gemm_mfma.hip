@@ -350,7 +350,9 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
 // Rows beyond M or N are fetched from the last valid row (their results are never stored).
 __device__ __forceinline__ int swz(int r) { return (r & 7) ^ ((r >> 3) & 1); }
 
-template <int kEpilogue, typename TO, int WTM, int WTN, int S, bool kSplitK = false>
+// kSplitK = 2: a block leaves its share's sums as they are, tile by tile, in part `share` of `out` (float
+// [shares, M, ldo]); a second kernel (split_sum_kernel) adds the parts and runs the epilogue.
+template <int kEpilogue, typename TO, int WTM, int WTN, int S, int kSplitK = 0>
 __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda,
                                                        const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2, int64_t ldw,
                                                        const float* __restrict__ bias, int M, int N, int K, int tiles_m,
@@ -467,7 +469,12 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
     read(k);
     multiply();
   }
-  if constexpr (kSplitK) {
+  if constexpr (kSplitK == 2) {
+    static_assert(kEpilogue == kMfStore && sizeof(TO) == 4, "parts of a sum are stored as float");
+    tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out + static_cast<int64_t>(place.share) * M * ldo, ldo, nullptr, M, N, m0, n0, wm, wn, lane);
+    return;
+  }
+  if constexpr (kSplitK == 1) {
     // the shares of K meet in the workspace, as in the kernel above
     const int tile_id = place.bm * tiles_n + place.bn;
     constexpr int kTileFloats = WTM * WTN * 16 * 256;
@@ -537,9 +544,48 @@ static int launch_dma_shared(void* out, int64_t ldo, const void* A, int64_t lda,
   const int64_t tiles = static_cast<int64_t>(tiles_n) * tiles_m;
   ALOFA_REQUIRE(g_ws.tiles != nullptr && tiles <= g_ws.n_counters && tiles * shares * (WTM * WTN * 16 * 256) <= g_ws.tile_floats,
                 "gemm_mfma: %lld tiles in %d shares of K do not fit the workspace", static_cast<long long>(tiles), shares);
-  gemm_dma_kernel<kEpilogue, TO, WTM, WTN, S, true><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
+  gemm_dma_kernel<kEpilogue, TO, WTM, WTN, S, 1><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, bias, M, N, K,
       tiles_m, tiles_n, 1, shares, g_ws.tiles, g_ws.counters);
+  return 0;
+}
+
+// out = epilogue(sum over the parts, in their order) for parts [shares, M, N] of float; four columns a thread.
+template <int kEpilogue, typename TO>
+__global__ void __launch_bounds__(256) split_sum_kernel(TO* __restrict__ out, int64_t ldo, const float* __restrict__ parts, int shares,
+                                                        const float* __restrict__ bias, int M, int N) {
+  const int groups = N / 4;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= static_cast<int64_t>(M) * groups) return;
+  const int m = static_cast<int>(idx / groups), n = static_cast<int>(idx % groups) * 4;
+  const float* src = parts + static_cast<int64_t>(m) * N + n;
+  float4 sum = *reinterpret_cast<const float4*>(src);
+  for (int sp = 1; sp < shares; ++sp) {
+    const float4 v = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(sp) * M * N);
+    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+  }
+  TO* dst = out + static_cast<int64_t>(m) * ldo + n;
+  if constexpr (kEpilogue == kMfResidual) {
+    dst[0] += sum.x; dst[1] += sum.y; dst[2] += sum.z; dst[3] += sum.w;
+  } else {
+    if (bias != nullptr) { sum.x += bias[n]; sum.y += bias[n + 1]; sum.z += bias[n + 2]; sum.w += bias[n + 3]; }
+    store_f32(dst, sum.x); store_f32(dst + 1, sum.y); store_f32(dst + 2, sum.z); store_f32(dst + 3, sum.w);
+  }
+}
+
+// K shared out among the blocks of a launch (tiles of 64 rows x 64 WTN columns, a ring of S slabs), and a second
+// launch that adds the shares and runs the epilogue. The parts lie in the workspace as [shares, M, N] floats.
+template <int kEpilogue, typename TO, int WTN, int S>
+static int launch_dma_sliced(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
+                             int shares, hipStream_t stream) {
+  const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 63) / 64;
+  const Workspace& g_ws = workspace();
+  ALOFA_REQUIRE(g_ws.tiles != nullptr && N % 4 == 0 && static_cast<int64_t>(shares) * M * N <= g_ws.tile_floats,
+                "gemm_mfma: %d shares of %d x %d sums do not fit the workspace (or N is no multiple of four)", shares, M, N);
+  gemm_dma_kernel<kMfStore, float, 1, WTN, S, 2><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
+      g_ws.tiles, N, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, nullptr, M, N, K, tiles_m, tiles_n, 1, shares);
+  const int64_t threads = static_cast<int64_t>(M) * (N / 4);
+  split_sum_kernel<kEpilogue, TO><<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(static_cast<TO*>(out), ldo, g_ws.tiles, shares, bias, M, N);
   return 0;
 }
 
@@ -668,6 +714,22 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       // With a short K a share of it is too short to pay for the hand-over: small tiles unshared, slabs straight
       // from memory (0.5B sizes, 96 to 768 rows: 8.1-8.5 us against 8.8-10.8 for N = 1,152, K = 896).
       const int shares = (ring && !long_k) ? 1 : k_shares(static_cast<int64_t>(tiles_n) * tiles_m, 64 * 64, K);
+      // Up to 64 rows against a matrix of few columns and a long K: with few column tiles the blocks that arrive
+      // last, one per tile, would add all the shares of their tiles while the rest of the chip is done. Tiles of
+      // 128 columns instead, K in as many shares as fill the chip once (four slabs each at least), every block
+      // leaving its sums as they are, and a second launch of a thread per four outputs that adds the shares in
+      // their order (us against the hand-over, 64 rows: N = 4,608, K = 3,584 14.2 against 18.7; 3,584 x 3,584
+      // 13.6 against 16.5; N = 3,584, K = 18,944 35.0 against 40.6; N = 1,536, K = 8,960 16.4 against 21.3; with
+      // 40 column tiles and more the hand-over is ahead: N = 5,120, K = 5,120 at 32 rows 25.3 against 23.1,
+      // N = 7,168 29.3 against 24.1).
+      const int wide_tiles = (N + 127) / 128, all_slabs = K / TK;
+      const int per_share = max(4, (all_slabs * wide_tiles + 255) / 256), slices = (all_slabs + per_share - 1) / per_share;
+      if (kEpilogue != kMfSwiglu && ring && long_k && M <= 64 && wide_tiles <= 36 && N % 4 == 0 && slices > 1 &&
+          static_cast<int64_t>(slices) * M * N <= workspace().tile_floats) {
+        if constexpr (kEpilogue != kMfSwiglu) {
+          if (launch_dma_sliced<kEpilogue, TO, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, slices, stream)) return 1;
+        }
+      } else
       if (ring && long_k && tiles_128x64 >= 144 && tiles_128x64 <= 256) {
         // Tiles of 128 x 64 that fill most of the chip once, and a long K: one block per compute unit with a ring
         // of four (35.8 against 38.8 us for N = 896, K = 4,864 at 2,048 rows; 28.8 against 36.1 with K shared out

@@ -781,24 +781,30 @@ def test_gate_up_of_few_rows_against_a_long_and_wide_pair_of_matrices():
 
 
 def test_few_rows_against_a_big_matrix_with_k_shared_out():
-    """The tiled kernel with K shared out among blocks and the slabs straight into LDS (weights of 32 MB or more):
-    sizes that end inside a tile and a share, residual and store epilogues, against a float32 product."""
+    """The tiled kernel with K shared out among blocks and the slabs straight into LDS: with few column tiles the
+    shares are added by a second launch, with many (and weights of 32 MB or more) by the block of a tile that
+    arrives last; a width that is no multiple of four takes neither. Sizes that end inside a tile and a share,
+    residual and store epilogues, against a float32 product."""
     o = ops()
-    M, N, K = 40, 3600, 18944 + 64
     g = torch.Generator(device="cpu").manual_seed(4)
-    a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
-    w = torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16)
-    base = torch.randn(M, N, generator=g).to(DEV)
-    acc = base.clone()
-    o.gemm(acc, a, w, add_to_out=True, kernel="tiled")
-    ref = a.float() @ w.float().T
-    assert ((acc - base - ref).abs().max() / ref.abs().max()).item() < 1e-4
-    out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
-    o.gemm(out, a, w, kernel="tiled")
-    assert ((out.float() - ref).abs().max() / ref.abs().max()).item() < 1e-2
-    again = base.clone()
-    o.gemm(again, a, w, add_to_out=True, kernel="tiled")
-    assert torch.equal(again, acc)                       # the shares are added in a fixed order
+    for M, N, K in ((40, 3600, 18944 + 64), (17, 1000, 2112), (64, 4608, 3584), (40, 5000, 3392), (33, 1001, 4160)):
+        a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
+        w = torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16)
+        base = torch.randn(M, N, generator=g).to(DEV)
+        acc = base.clone()
+        o.gemm(acc, a, w, add_to_out=True, kernel="tiled")
+        ref = a.float() @ w.float().T
+        assert ((acc - base - ref).abs().max() / ref.abs().max()).item() < 1e-4, (M, N, K)
+        bias = torch.randn(N, generator=g).to(DEV)
+        out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+        o.gemm(out, a, w, bias, kernel="tiled")
+        assert ((out.float() - ref - bias).abs().max() / ref.abs().max()).item() < 1e-2, (M, N, K)
+        out32 = torch.full((M, N), float("nan"), device=DEV)
+        o.gemm(out32, a, w, kernel="tiled")
+        assert ((out32 - ref).abs().max() / ref.abs().max()).item() < 1e-4, (M, N, K)
+        again = base.clone()
+        o.gemm(again, a, w, add_to_out=True, kernel="tiled")
+        assert torch.equal(again, acc), (M, N, K)            # the shares are added in a fixed order
 
 
 def test_many_rows_in_tiles_of_128_x_256():
