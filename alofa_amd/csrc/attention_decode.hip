@@ -414,12 +414,18 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   }
 }
 
-// Combines the parts' states of one (token, head) in part order (maxima in units of log2 e).
-__global__ void __launch_bounds__(64) attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
-                                                             const float* __restrict__ partial,
-                                                             const int32_t* __restrict__ rows, int heads, int d,
-                                                             int n_splits) {
-  const int t = rows ? rows[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+// Combines the parts' states of one (token, head) (maxima in units of log2 e). The waves of the block take the
+// parts in turn (wave w parts w, w + waves, ..), sixteen at a time with all their loads on their way together:
+// the states come from memory, and one after the other 64 parts took 20 us. Every wave sums its parts in
+// ascending order and the waves' sums are added in wave order, so the result depends on nothing but the number
+// of parts and of waves.
+__global__ void __launch_bounds__(256) attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
+                                                              const float* __restrict__ partial,
+                                                              const int32_t* __restrict__ rows, int heads, int d,
+                                                              int n_splits) {
+  __shared__ float sums[4][256];
+  const int t = rows ? rows[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x % 64;
+  const int wave = threadIdx.x / 64, waves = blockDim.x / 64;
   const float* src = partial + (static_cast<int64_t>(blockIdx.x) * heads + h) * n_splits * (d + 2);
   // lane s holds part s's maximum and sum (n_splits <= 64)
   const float m = lane < n_splits ? src[lane * (d + 2)] : -FLT_MAX;
@@ -431,12 +437,28 @@ __global__ void __launch_bounds__(64) attention_merge_kernel(bf16_t* __restrict_
   for (int c0 = 0; c0 < d; c0 += 64) {
     const int c = c0 + lane;
     float acc = 0.f;
-#pragma unroll 8
-    for (int s = 0; s < n_splits; ++s) {
-      const float w = __shfl(e, s, 64);
-      if (c < d) acc += src[s * (d + 2) + 2 + c] * w;
+    for (int base = wave; base < n_splits; base += 16 * waves) {    // uniform over the wave
+      float v[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int sp = base + i * waves;
+        v[i] = (sp < n_splits && c < d) ? src[sp * (d + 2) + 2 + c] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int sp = base + i * waves;
+        acc += v[i] * __shfl(e, sp < n_splits ? sp : 0, 64);
+      }
     }
-    if (c < d) store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
+    if (waves > 1) {
+      if (c < d) sums[wave][c] = acc;
+      __syncthreads();
+      if (wave == 0) {
+        acc = sums[0][c < d ? c : 0];
+        for (int w = 1; w < waves; ++w) acc += sums[w][c < d ? c : 0];
+      }
+    }
+    if (wave == 0 && c < d) store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
   }
 }
 
@@ -531,7 +553,8 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
 #undef ALOFA_DECODE
   if (check_launch("attention_decode")) return 1;
   if (n_splits > 1 && !counters) {
-    attention_merge_kernel<<<dim3(tokens, heads), 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits);
+    // (one wave up to sixteen parts, whose loads are all on their way at once; four beyond)
+    attention_merge_kernel<<<dim3(tokens, heads), n_splits <= 16 ? 64 : 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits);
     return check_launch("attention_merge");
   }
   return 0;
