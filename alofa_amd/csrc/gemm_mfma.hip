@@ -559,10 +559,16 @@ __global__ void __launch_bounds__(256) split_sum_kernel(TO* __restrict__ out, in
   if (idx >= static_cast<int64_t>(M) * groups) return;
   const int m = static_cast<int>(idx / groups), n = static_cast<int>(idx % groups) * 4;
   const float* src = parts + static_cast<int64_t>(m) * N + n;
-  float4 sum = *reinterpret_cast<const float4*>(src);
-  for (int sp = 1; sp < shares; ++sp) {
-    const float4 v = *reinterpret_cast<const float4*>(src + static_cast<int64_t>(sp) * M * N);
-    sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+  // (eight parts' loads on their way together: the parts come from memory, one after the other they are waited for one by one)
+  float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int64_t part = static_cast<int64_t>(M) * N;
+  for (int s0 = 0; s0 < shares; s0 += 8) {
+    float4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = *reinterpret_cast<const float4*>(src + min(s0 + i, shares - 1) * part);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (s0 + i < shares) { sum.x += v[i].x; sum.y += v[i].y; sum.z += v[i].z; sum.w += v[i].w; }
   }
   TO* dst = out + static_cast<int64_t>(m) * ldo + n;
   if constexpr (kEpilogue == kMfResidual) {
