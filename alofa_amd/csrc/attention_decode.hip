@@ -400,15 +400,37 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     if (h0 + i >= group) break;
     const int h = hk * group + h0 + i;
     const float* src = partial + (static_cast<int64_t>(blockIdx.x) * heads + h) * n_parts * (d + 2);
-    float big = -FLT_MAX;
-    for (int sp = 0; sp < n_parts; ++sp) big = fmaxf(big, __hip_atomic_load(src + sp * (d + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-    float total = 0.f, acc = 0.f;
+    float big = -FLT_MAX, total = 0.f, acc = 0.f;
+    if (n_parts <= 4) {
+      // up to four parts: everything that is read is asked for at once (the states come from memory; one after
+      // the other, every load is waited for by itself); same sums in the same order as below
+      float ms[4], ls[4], vs[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float* part = src + min(u, n_parts - 1) * (d + 2);
+        ms[u] = __hip_atomic_load(part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ls[u] = __hip_atomic_load(part + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        vs[u] = __hip_atomic_load(part + 2 + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (u < n_parts) big = fmaxf(big, ms[u]);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (u < n_parts) {
+          const float e = __builtin_amdgcn_exp2f(ms[u] - big);
+          total += ls[u] * e;
+          acc += vs[u] * e;
+        }
+    } else {
+      for (int sp = 0; sp < n_parts; ++sp) big = fmaxf(big, __hip_atomic_load(src + sp * (d + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 #pragma unroll 4
-    for (int sp = 0; sp < n_parts; ++sp) {
-      const float* part = src + sp * (d + 2);
-      const float e = __builtin_amdgcn_exp2f(__hip_atomic_load(part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - big);
-      total += __hip_atomic_load(part + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * e;
-      acc += __hip_atomic_load(part + 2 + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * e;
+      for (int sp = 0; sp < n_parts; ++sp) {
+        const float* part = src + sp * (d + 2);
+        const float e = __builtin_amdgcn_exp2f(__hip_atomic_load(part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - big);
+        total += __hip_atomic_load(part + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * e;
+        acc += __hip_atomic_load(part + 2 + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * e;
+      }
     }
     store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
   }

@@ -318,14 +318,20 @@ __global__ void __launch_bounds__(256) gemm_mfma_kernel(TO* __restrict__ out, in
       for (int j = 0; j < WTN; ++j) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-        for (int sp = 0; sp < splits; ++sp) {
-          float part[16];
+        for (int sp0 = 0; sp0 < splits; sp0 += 4) {     // four shares' loads on their way together; added in the shares' order
+          float part[4][16];
 #pragma unroll
-          for (int e = 0; e < 16; ++e)
-            part[e] = __hip_atomic_load(parts + static_cast<int64_t>(sp) * kTileFloats + ((i * WTN + j) * 16 + e) * 256 + tid,
-                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int u = 0; u < 4; ++u)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) acc[i][j][e] += part[e];
+            for (int e = 0; e < 16; ++e)
+              part[u][e] = __hip_atomic_load(parts + static_cast<int64_t>(min(sp0 + u, splits - 1)) * kTileFloats + ((i * WTN + j) * 16 + e) * 256 + tid,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (sp0 + u < splits) {
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc[i][j][e] += part[u][e];
+            }
         }
       }
   }
@@ -503,14 +509,20 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
       for (int j = 0; j < WTN; ++j) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-        for (int sp = 0; sp < shares; ++sp) {
-          float part[16];
+        for (int sp0 = 0; sp0 < shares; sp0 += 4) {     // four shares' loads on their way together; added in the shares' order
+          float part[4][16];
 #pragma unroll
-          for (int e = 0; e < 16; ++e)
-            part[e] = __hip_atomic_load(parts + static_cast<int64_t>(sp) * kTileFloats + ((i * WTN + j) * 16 + e) * 256 + tid,
-                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int u = 0; u < 4; ++u)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) acc[i][j][e] += part[e];
+            for (int e = 0; e < 16; ++e)
+              part[u][e] = __hip_atomic_load(parts + static_cast<int64_t>(min(sp0 + u, shares - 1)) * kTileFloats + ((i * WTN + j) * 16 + e) * 256 + tid,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            if (sp0 + u < shares) {
+#pragma unroll
+              for (int e = 0; e < 16; ++e) acc[i][j][e] += part[u][e];
+            }
         }
       }
   }

@@ -29,6 +29,8 @@
 // the step; D holds column l % 16, rows 4 * (l / 16) .. + 3.
 #include "common.h"
 
+#include <type_traits>
+
 namespace alofa {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -268,8 +270,22 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     const int nt = (kEpilogue == kSkSwiglu) ? 0 : tile % NT;
     f32x4 sum, up = f32x4{0.f, 0.f, 0.f, 0.f};
     if (k_splits > 1) {
-      sum = parts[(mt * NT + nt) * 64 + lane];
-      for (int ks = 1; ks < k_splits; ++ks) sum += parts[(ks * MT * NT + mt * NT + nt) * 64 + lane];
+      // (all the splits' loads on their way together, two, four or eight: they come from memory, and one after
+      // the other each is waited for by itself; the order of the additions stays)
+      const f32x4* first = parts + (mt * NT + nt) * 64 + lane;
+      auto in_order = [&](auto count) {
+        constexpr int kCount = decltype(count)::value;
+        f32x4 theirs[kCount];
+#pragma unroll
+        for (int ks = 0; ks < kCount; ++ks) theirs[ks] = first[ks * MT * NT * 64];
+        f32x4 total = theirs[0];
+#pragma unroll
+        for (int ks = 1; ks < kCount; ++ks) total += theirs[ks];
+        return total;
+      };
+      if (k_splits == 2) sum = in_order(std::integral_constant<int, 2>());
+      else if (k_splits == 4) sum = in_order(std::integral_constant<int, 4>());
+      else sum = in_order(std::integral_constant<int, 8>());     // (the splits are doubled from one up to eight)
     } else {
       sum = red[0][mt * NT + nt][lane];
 #pragma unroll
