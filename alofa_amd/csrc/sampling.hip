@@ -112,10 +112,21 @@ __global__ void __launch_bounds__(256) argmax_parts_kernel(Choice choice, const 
   const int r = blockIdx.x;
   float bv = -FLT_MAX;
   int bi = vocab;
-  for (int p = threadIdx.x; p < n_parts; p += 256) {
-    const float v = part_v[static_cast<int64_t>(r) * n_parts + p];
-    const int i = part_i[static_cast<int64_t>(r) * n_parts + p];
-    if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+  // (eight candidates' loads on their way together; compared in ascending order as one by one)
+  const float* row_v = part_v + static_cast<int64_t>(r) * n_parts;
+  const int32_t* row_i = part_i + static_cast<int64_t>(r) * n_parts;
+  for (int p0 = threadIdx.x; p0 < n_parts; p0 += 8 * 256) {
+    float vs[8];
+    int is[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int p = min(p0 + 256 * u, n_parts - 1);
+      vs[u] = row_v[p];
+      is[u] = row_i[p];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (p0 + 256 * u < n_parts && (vs[u] > bv || (vs[u] == bv && is[u] < bi))) { bv = vs[u]; bi = is[u]; }
   }
   for (int off = kWave / 2; off > 0; off >>= 1) {
     const float ov = __shfl_xor(bv, off, kWave);
