@@ -34,6 +34,8 @@
 // Cache layout: keys [block, kv_head, slot_in_block, d], values transposed [block, kv_head, d, slot_in_block].
 #include "common.h"
 
+#include <type_traits>
+
 #include <float.h>
 
 namespace alofa {
@@ -401,27 +403,34 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     const int h = hk * group + h0 + i;
     const float* src = partial + (static_cast<int64_t>(blockIdx.x) * heads + h) * n_parts * (d + 2);
     float big = -FLT_MAX, total = 0.f, acc = 0.f;
-    if (n_parts <= 4) {
-      // up to four parts: everything that is read is asked for at once (the states come from memory; one after
-      // the other, every load is waited for by itself); same sums in the same order as below
-      float ms[4], ls[4], vs[4];
+    if (n_parts <= 16) {
+      // up to sixteen parts: everything that is read is asked for at once (the states come from memory; one after
+      // the other, every load is waited for by itself), in arrays of four, eight or sixteen; same sums in the same
+      // order as below
+      auto at_once = [&](auto count) {
+        constexpr int kCount = decltype(count)::value;
+        float ms[kCount], ls[kCount], vs[kCount];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float* part = src + min(u, n_parts - 1) * (d + 2);
-        ms[u] = __hip_atomic_load(part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ls[u] = __hip_atomic_load(part + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        vs[u] = __hip_atomic_load(part + 2 + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (u < n_parts) big = fmaxf(big, ms[u]);
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (u < n_parts) {
-          const float e = __builtin_amdgcn_exp2f(ms[u] - big);
-          total += ls[u] * e;
-          acc += vs[u] * e;
+        for (int u = 0; u < kCount; ++u) {
+          const float* part = src + min(u, n_parts - 1) * (d + 2);
+          ms[u] = __hip_atomic_load(part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          ls[u] = __hip_atomic_load(part + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          vs[u] = __hip_atomic_load(part + 2 + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+#pragma unroll
+        for (int u = 0; u < kCount; ++u)
+          if (u < n_parts) big = fmaxf(big, ms[u]);
+#pragma unroll
+        for (int u = 0; u < kCount; ++u)
+          if (u < n_parts) {
+            const float e = __builtin_amdgcn_exp2f(ms[u] - big);
+            total += ls[u] * e;
+            acc += vs[u] * e;
+          }
+      };
+      if (n_parts <= 4) at_once(std::integral_constant<int, 4>());
+      else if (n_parts <= 8) at_once(std::integral_constant<int, 8>());
+      else at_once(std::integral_constant<int, 16>());
     } else {
       for (int sp = 0; sp < n_parts; ++sp) big = fmaxf(big, __hip_atomic_load(src + sp * (d + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 #pragma unroll 4

@@ -428,7 +428,7 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     """Parts the keys of a (token, key head) are cut into beyond the waves of a block. A block reads
     its keys at the rate of one compute unit, so while the blocks are far fewer than the compute
     units more of them are faster: none up to two steps of 32 keys a wave; up to four steps four
-    parts, which the last block to arrive combines (``decode_hand_over``), if the chip has room for
+    parts, which the last block to arrive combines (``decode_hand_over``: up to eight parts), if the chip has room for
     eight; then a part per step of all the waves, at most eight (the merge grows with them), and
     from there on a part per two steps, combined by a second kernel; never more parts than fill
     the chip, and up to eight steps a wave none where the chip has room for two or three only (two
@@ -453,7 +453,7 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     return max(1, min(64, by_length, by_chip))
 
 
-HAND_OVER_MAX_PARTS = 4    # up to so many parts the last block combines them; a second kernel combines more
+HAND_OVER_MAX_PARTS = 8    # up to so many parts the last block combines them; a second kernel combines more
 
 
 def decode_hand_over(tokens: int, heads: int, kv_heads: int, d: int, n_splits: int) -> bool:

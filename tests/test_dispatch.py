@@ -48,7 +48,7 @@ def test_decode_splits_follow_the_context():
     assert ops.decode_splits(64, 14, 2, 64, 2048) == 1 and ops.decode_splits(64, 14, 2, 64, 4096) == 2 and ops.decode_splits(32, 14, 2, 64, 2048) == 4    # many blocks already: fewer parts
     assert ops.decode_splits(8, 28, 4, 128, 256) == 1 and ops.decode_splits(8, 28, 4, 128, 512) == 4 and ops.decode_splits(8, 28, 4, 128, 4096) == 8
     assert ops.decode_splits(32, 28, 4, 128, 512) == 1 and ops.decode_splits(32, 28, 4, 128, 1024) == 1 and ops.decode_splits(32, 28, 4, 128, 2048) == 2 and ops.decode_splits(64, 28, 4, 128, 4096) == 1
-    assert ops.HAND_OVER_MAX_PARTS == 4
+    assert ops.HAND_OVER_MAX_PARTS == 8
     assert ops.decode_waves(64) == 8 and ops.decode_waves(128) == 4 and ops.decode_waves(256) == 4
 
 

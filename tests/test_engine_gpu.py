@@ -126,10 +126,10 @@ def test_long_decoding(replayers, tiny_dirs, dtype):
     assert_close(got, plain_logits(tiny_dirs["C"], tuple(ids)), dtype, "C long decode")
 
 
-@pytest.mark.parametrize("name,n", [("B", 660), ("D", 430)])
+@pytest.mark.parametrize("name,n", [("B", 660), ("D", 430), ("B", 1300)])
 def test_decoding_where_the_parts_of_a_context_are_handed_over(tiny_dirs, name, n):
-    """Contexts of two to four steps of 32 keys a wave (bfloat16): decode attention cuts the keys of a (token, key
-    head) into four parts, and the block that arrives last combines them. Two requests decode side by side at
+    """Contexts of two to eight steps of 32 keys a wave (bfloat16): decode attention cuts the keys of a (token, key
+    head) into four or eight parts, and the block that arrives last combines them. Two requests decode side by side at
     such contexts, the last 40 tokens one by one (captured graphs from the second step on)."""
     from alofa_amd import ops
     from alofa_amd.replay import Replayer

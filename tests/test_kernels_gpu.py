@@ -483,7 +483,7 @@ def test_decode_attention(heads, kv_heads, d, bs, window, bucket):
             o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, False,
                               max_q_len=4, max_context=bucket)
     # both ways in which parts meet, whatever the launch would choose: the last block combines them, or a second kernel does
-    for parts in (2, 4):
+    for parts in (2, 4, 7, 8, 13):
         for hand_over in (True, False):
             again = torch.zeros_like(out)
             o.attention_decode(again, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, window, scale, bucket,
