@@ -429,7 +429,7 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     its keys at the rate of one compute unit, so while the blocks are far fewer than the compute
     units more of them are faster: none up to two steps of 32 keys a wave; up to four steps four
     parts, which the last block to arrive combines (``decode_hand_over``: up to eight parts), if the chip has room for
-    eight; then a part per step of all the waves, at most eight (the merge grows with them), and
+    four (batch 32 at 600 keys: 1.26 against 1.30 ms a step); then a part per step of all the waves, at most eight (the merge grows with them), and
     from there on a part per two steps, combined by a second kernel; never more parts than fill
     the chip, and up to eight steps a wave none where the chip has room for two or three only (two
     parts gain at the long end of such a context bound what they lose at its short end). (Measured at 14:2 heads of 64 and 28:4 of 128, batches of 1 to 64, contexts of 200
@@ -444,7 +444,7 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     blocks = tokens * kv_heads * -(-(heads // kv_heads) // 16)
     by_chip = max(1, 256 // max(1, blocks))
     if max_context <= 4 * step:
-        return 4 if by_chip >= 8 else 1
+        return 4 if by_chip >= 4 else 1
     if max_context <= 8 * step and by_chip < 4:
         return 1
     by_length = -(-max_context // step)

@@ -41,7 +41,7 @@ def test_product_kernel_by_shape():
 
 def test_decode_splits_follow_the_context():
     assert ops.decode_splits(8, 14, 2, 64, 512) == 1                              # the waves of one block cover two steps each
-    assert ops.decode_splits(8, 14, 2, 64, 1024) == 4 and ops.decode_splits(32, 14, 2, 64, 1024) == 1    # four parts up to four steps, with room for eight
+    assert ops.decode_splits(8, 14, 2, 64, 1024) == 4 and ops.decode_splits(32, 14, 2, 64, 1024) == 4 and ops.decode_splits(64, 14, 2, 64, 1024) == 1    # four parts up to four steps, with room for four
     assert ops.decode_splits(8, 14, 2, 64, 2048) == 8                             # a part per step of all the waves
     assert ops.decode_splits(8, 14, 2, 64, 1 << 12) == 8 and ops.decode_splits(8, 14, 2, 64, 1 << 13) == 16    # at most eight, then a part per two steps
     assert ops.decode_splits(8, 14, 2, 64, 1 << 16) == 256 // 16                   # until the blocks fill the chip
