@@ -593,14 +593,14 @@ __global__ void __launch_bounds__(256) split_sum_kernel(TO* __restrict__ out, in
 
 // K shared out among the blocks of a launch (tiles of 64 rows x 64 WTN columns, a ring of S slabs), and a second
 // launch that adds the shares and runs the epilogue. The parts lie in the workspace as [shares, M, N] floats.
-template <int kEpilogue, typename TO, int WTN, int S>
+template <int kEpilogue, typename TO, int WTN, int S, int WTM = 1>
 static int launch_dma_sliced(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
                              int shares, hipStream_t stream) {
-  const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 63) / 64;
+  const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
   const Workspace& g_ws = workspace();
   ALOFA_REQUIRE(g_ws.tiles != nullptr && N % 4 == 0 && static_cast<int64_t>(shares) * M * N <= g_ws.tile_floats,
                 "gemm_mfma: %d shares of %d x %d sums do not fit the workspace (or N is no multiple of four)", shares, M, N);
-  gemm_dma_kernel<kMfStore, float, 1, WTN, S, 2><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
+  gemm_dma_kernel<kMfStore, float, WTM, WTN, S, 2><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
       g_ws.tiles, N, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, nullptr, M, N, K, tiles_m, tiles_n, 1, shares);
   const int64_t threads = static_cast<int64_t>(M) * (N / 4);
   split_sum_kernel<kEpilogue, TO><<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(static_cast<TO*>(out), ldo, g_ws.tiles, shares, bias, M, N);
@@ -740,12 +740,29 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       // 13.6 against 16.5; N = 3,584, K = 18,944 35.0 against 40.6; N = 1,536, K = 8,960 16.4 against 21.3; with
       // 40 column tiles and more the hand-over is ahead: N = 5,120, K = 5,120 at 32 rows 25.3 against 23.1,
       // N = 7,168 29.3 against 24.1).
+      // More than 64 rows, a long K and too few tiles of 128 x 128 for the chip (a down projection in a prefill of
+      // a small model, a portion of a prompt against the projections of a large one): such tiles with K in two to
+      // eight shares, as many as fill the chip once, and the second launch that adds them (us against the rules
+      // below: N = 896, K = 4,864 at 2,048 rows 32.0 against 33.7, at 1,024 rows 21.8 against 28.7; N = 3,584,
+      // K = 18,944 at 128, 256, 384 rows 43.6, 61.1, 76.8 against 55.4, 89.7, 120.7; N = 5,120, K = 27,648 at 128
+      // and 256 rows 74 and 110 against 135 and 178; 5,120 x 5,120 at 256 rows 32.1 against 42.9).
+      const int64_t tiles_128x128 = static_cast<int64_t>((M + 127) / 128) * ((N + 127) / 128);
+      int tall_shares = static_cast<int>(256 / tiles_128x128);      // as many as fill the chip once: up to eight, of sixteen slabs or more
+      if (tall_shares > 8) tall_shares = 8;
+      if (tall_shares > K / TK / 16) tall_shares = K / TK / 16;
+      if (tiles_128x128 * tall_shares < 160) tall_shares = 0;       // (too few blocks for the chip: the rules below)
       const int wide_tiles = (N + 127) / 128, all_slabs = K / TK;
       const int per_share = max(4, (all_slabs * wide_tiles + 255) / 256), slices = (all_slabs + per_share - 1) / per_share;
       if (kEpilogue != kMfSwiglu && ring && long_k && M <= 64 && wide_tiles <= 36 && N % 4 == 0 && slices > 1 &&
           static_cast<int64_t>(slices) * M * N <= workspace().tile_floats) {
         if constexpr (kEpilogue != kMfSwiglu) {
           if (launch_dma_sliced<kEpilogue, TO, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, slices, stream)) return 1;
+        }
+      } else
+      if (tall_shares > 1 && kEpilogue != kMfSwiglu && ring && K >= 4096 && M > 64 && N % 4 == 0 &&
+          static_cast<int64_t>(tall_shares) * M * N <= workspace().tile_floats) {
+        if constexpr (kEpilogue != kMfSwiglu) {
+          if (launch_dma_sliced<kEpilogue, TO, 2, 3, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, tall_shares, stream)) return 1;
         }
       } else
       if (ring && long_k && tiles_128x64 >= 144 && tiles_128x64 <= 256) {
