@@ -745,7 +745,8 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       // eight shares, as many as fill the chip once, and the second launch that adds them (us against the rules
       // below: N = 896, K = 4,864 at 2,048 rows 32.0 against 33.7, at 1,024 rows 21.8 against 28.7; N = 3,584,
       // K = 18,944 at 128, 256, 384 rows 43.6, 61.1, 76.8 against 55.4, 89.7, 120.7; N = 5,120, K = 27,648 at 128
-      // and 256 rows 74 and 110 against 135 and 178; 5,120 x 5,120 at 256 rows 32.1 against 42.9).
+      // and 256 rows 74 and 110 against 135 and 178; 5,120 x 5,120 at 256 rows 32.1 against 42.9; 3,584 x 3,584 at 384 rows 23.9 against 30.0; with K = 2,048 it loses,
+      // N = 2,560 at 512 rows 20.0 against 16.9).
       const int64_t tiles_128x128 = static_cast<int64_t>((M + 127) / 128) * ((N + 127) / 128);
       int tall_shares = static_cast<int>(256 / tiles_128x128);      // as many as fill the chip once: up to eight, of sixteen slabs or more
       if (tall_shares > 8) tall_shares = 8;
@@ -759,7 +760,7 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
           if (launch_dma_sliced<kEpilogue, TO, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, slices, stream)) return 1;
         }
       } else
-      if (tall_shares > 1 && kEpilogue != kMfSwiglu && ring && K >= 4096 && M > 64 && N % 4 == 0 &&
+      if (tall_shares > 1 && kEpilogue != kMfSwiglu && ring && K >= 3072 && M > 64 && N % 4 == 0 &&
           static_cast<int64_t>(tall_shares) * M * N <= workspace().tile_floats) {
         if constexpr (kEpilogue != kMfSwiglu) {
           if (launch_dma_sliced<kEpilogue, TO, 2, 3, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, tall_shares, stream)) return 1;
