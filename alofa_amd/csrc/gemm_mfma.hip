@@ -752,15 +752,19 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       if (tall_shares > 8) tall_shares = 8;
       if (tall_shares > K / TK / 16) tall_shares = K / TK / 16;
       if (tiles_128x128 * tall_shares < 160) tall_shares = 0;       // (too few blocks for the chip: the rules below)
-      const int wide_tiles = (N + 127) / 128, all_slabs = K / TK;
+      const bool tall = tall_shares > 1 && K >= 3072 && M > 64;
+      // (the tiles of 64 x 128 also up to 256 rows, for K from 3,072, where those of 128 x 128 are too few even in
+      // shares: N = 896, K = 4,864 at 65, 128 and 256 rows 10.4, 12.3 and 14.0 us against 15.0, 15.1 and 16.8;
+      // N = 2,048, K = 11,008 at 128 rows 22.2 against 24.8)
+      const int wide_tiles = ((N + 127) / 128) * tiles_m, all_slabs = K / TK;
       const int per_share = max(4, (all_slabs * wide_tiles + 255) / 256), slices = (all_slabs + per_share - 1) / per_share;
-      if (kEpilogue != kMfSwiglu && ring && long_k && M <= 64 && wide_tiles <= 36 && N % 4 == 0 && slices > 1 &&
+      if (kEpilogue != kMfSwiglu && ring && long_k && (M <= 64 || (M <= 256 && !tall && K >= 3072)) && wide_tiles <= 36 && N % 4 == 0 && slices > 1 &&
           static_cast<int64_t>(slices) * M * N <= workspace().tile_floats) {
         if constexpr (kEpilogue != kMfSwiglu) {
           if (launch_dma_sliced<kEpilogue, TO, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, slices, stream)) return 1;
         }
       } else
-      if (tall_shares > 1 && kEpilogue != kMfSwiglu && ring && K >= 3072 && M > 64 && N % 4 == 0 &&
+      if (tall && kEpilogue != kMfSwiglu && ring && N % 4 == 0 &&
           static_cast<int64_t>(tall_shares) * M * N <= workspace().tile_floats) {
         if constexpr (kEpilogue != kMfSwiglu) {
           if (launch_dma_sliced<kEpilogue, TO, 2, 3, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, tall_shares, stream)) return 1;

@@ -788,7 +788,8 @@ def test_few_rows_against_a_big_matrix_with_k_shared_out():
     o = ops()
     g = torch.Generator(device="cpu").manual_seed(4)
     for M, N, K in ((40, 3600, 18944 + 64), (17, 1000, 2112), (64, 4608, 3584), (40, 5000, 3392), (33, 1001, 4160),
-                    (1100, 896, 4864), (2000, 1000, 4160)):      # many rows against a narrow matrix: tiles of 128 x 128, four and two shares
+                    (1100, 896, 4864), (2000, 1000, 4160),       # many rows against a narrow matrix: tiles of 128 x 128, four and two shares
+                    (100, 896, 4864), (250, 1000, 3136)):        # up to 256 rows: tiles of 64 x 128
         a = torch.randn(M, K, generator=g).to(DEV, torch.bfloat16)
         w = torch.randn(N, K, generator=g).mul_(0.05).to(DEV, torch.bfloat16)
         base = torch.randn(M, N, generator=g).to(DEV)
