@@ -366,7 +366,9 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
                                                        int* __restrict__ counters = nullptr) {
   constexpr int TM = 64 * WTM, TN = 64 * WTN;
   constexpr int kGateTiles = WTN / 2;
-  static_assert(kEpilogue != kMfSwiglu || WTN % 2 == 0, "the swiglu epilogue needs an even number of column tiles per wave");
+  // (swiglu with WTN = 1: the waves of column 0 take 32 gate columns, those of column 1 the up columns of the same
+  // outputs, and the two meet in LDS after the last slab)
+  static_assert(kEpilogue != kMfSwiglu || WTN % 2 == 0 || WTN == 1, "the swiglu epilogue needs an even number of column tiles per wave, or one");
   constexpr int kRows = TM + TN;               // slab rows: A's, then W's
   constexpr int kStageBytes = kRows * 128;
   constexpr int kLoads = kRows / 32;           // fetch instructions per wave and slab (each brings eight rows)
@@ -421,11 +423,12 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
   // fragments: lane l reads row l % 32 of its 32-row group, chunk 2 q + l / 32 in step q of the slab's four
   const int sw = swz(lane % 32), half = lane / 32;
   const int a_row = (wm * 32 * WTM + lane % 32) * 128;
-  const int w_row = (TM + wn * 32 * (kEpilogue == kMfSwiglu ? kGateTiles : WTN) + lane % 32) * 128;
+  const int w_row = (TM + wn * 32 * (kEpilogue == kMfSwiglu ? (WTN == 1 ? 1 : kGateTiles) : WTN) + lane % 32) * 128;
   int place_of[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) place_of[q] = ((2 * q + half) ^ sw) * 16;
   auto w_group = [&](int j) {      // byte offset of this wave's j-th 32-row group of W within the slab's W rows
+    if (kEpilogue == kMfSwiglu && WTN == 1) return 0;
     if (kEpilogue == kMfSwiglu) return (j < kGateTiles ? j * 32 : TN / 2 + (j - kGateTiles) * 32) * 128;
     return j * 32 * 128;
   };
@@ -474,6 +477,31 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
     __syncthreads();
     read(k);
     multiply();
+  }
+  if constexpr (kEpilogue == kMfSwiglu && WTN == 1) {
+    __syncthreads();      // every wave has read the last slab: the ring is free
+    float* meet = reinterpret_cast<float*>(ring);     // [wm][i][e][lane]
+    if (wn == 1) {
+#pragma unroll
+      for (int i = 0; i < WTM; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) meet[((wm * WTM + i) * 16 + e) * 64 + lane] = acc[i][0][e];
+    }
+    __syncthreads();
+    if (wn == 0) {
+      const int n = n0 + lane % 32;
+#pragma unroll
+      for (int i = 0; i < WTM; ++i) {
+        const int m_first = m0 + wm * 32 * WTM + i * 32 + (lane / 32) * 4;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int m = m_first + 8 * (e / 4) + e % 4;
+          const float g = acc[i][0][e], up = meet[((wm * WTM + i) * 16 + e) * 64 + lane];
+          if (m < M && n < N) store_f32(out + static_cast<int64_t>(m) * ldo + n, g / (1.f + __expf(-g)) * up);
+        }
+      }
+    }
+    return;
   }
   if constexpr (kSplitK == 2) {
     static_assert(kEpilogue == kMfStore && sizeof(TO) == 4, "parts of a sum are stored as float");
@@ -668,6 +696,12 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
         // sizes, 148 tiles, 64.1 against 62.4 at 16 rows, 67.6 against 70.7 at 64)
         if (launch_dma<kEpilogue, TO, 1, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
       } else if (K < 2048) {
+        // (up to 64 rows and fewer tiles than half the compute units: tiles of 32 outputs, whose gate and up halves
+        // are computed by different waves and meet in LDS; N = 4,864, K = 896 at 17 to 64 rows 8.5-9.4 us against
+        // 9.9-11.2)
+        if (M <= 64 && (N + 63) / 64 < 128) {
+          if (launch_dma<kEpilogue, TO, 1, 1, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+        } else
         if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
       } else {
         if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;

@@ -749,9 +749,10 @@ def test_product_kernel_choice():
         o.gemm(torch.empty(70, 16, device=DEV), a, w, kernel="stream")
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 4000, 128), (64, 330, 2112), (190, 1000, 64), (300, 4000, 128), (520, 4000, 192), (1030, 4000, 64), (130, 97, 3584)])
+@pytest.mark.parametrize("M,N,K", [(17, 4000, 128), (40, 3990, 192), (64, 1000, 896), (64, 330, 2112), (190, 1000, 64), (300, 4000, 128), (520, 4000, 192), (1030, 4000, 64), (130, 97, 3584)])
 def test_gate_up_tiled_with_slabs_straight_into_lds(M, N, K):
-    """Gate/up with K a multiple of 64 through the tiled kernel: tiles of 64 rows with a ring of four or three slabs,
+    """Gate/up with K a multiple of 64 through the tiled kernel: tiles of 64 rows with a ring of four or three slabs
+    (of 32 outputs where the tiles are few, the gate and up halves meeting in LDS),
     tiles of 128 rows with a ring of three or two, or slabs through registers, by how many tiles there are; sizes
     that end inside a tile of rows and of columns."""
     rng = np.random.default_rng(47)
