@@ -19,8 +19,11 @@ from .sampling.sampler import SampleParams
 class Engine:
     """``max_tokens`` is the context window of one request (prompt + generated),
     as the reference's ALOFA_MAX_TOKENS (src/alofa/srv/config.mojo:94-97).
-    ``kv_blocks`` pages of ``block_size`` tokens make the pool of each cache group;
-    by default enough for ``max_batch`` requests of ``max_tokens``. With
+    ``kv_blocks`` pages of ``block_size`` tokens make the pool of a group of layers that
+    keeps every key, by default enough for ``max_batch`` requests of ``max_tokens``; a group
+    whose layers see a window only gets what ``max_batch`` requests can hold of it (the
+    window, a step's tokens and two pages each), never more than ``kv_blocks``. A dict
+    from a group's window (None: every key) to its pages sets every pool by hand. With
     ``share_prefixes`` a new request starts on the whole pages a resident request has
     written for the same first tokens (src/alofa/runtime/kv/space.mojo:166-243, block by block)."""
 
@@ -41,17 +44,21 @@ class Engine:
         self.config, self.model = model if model is not None else load_model(Path(model_dir), dtype, device)
         if max_tokens > self.model.spec.max_positions:
             raise AlofaError("out_of_range", "max_tokens passes the model's position bound", f"max_tokens={max_tokens} max_position_embeddings={self.model.spec.max_positions}")
-        per_request = (max_tokens + block_size - 1) // block_size
-        if kv_blocks is None:
-            # enough for max_batch whole windows below the scheduler's watermark
-            kv_blocks = (per_request * max_batch * 1000 + watermark_permille - 1) // watermark_permille + 1
-        self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), kv_blocks, block_size,
+        needs = self.model.cache_needs()
+        if not isinstance(kv_blocks, dict):
+            def under_watermark(pages):      # enough for max_batch such requests below the scheduler's watermark
+                return (pages * 1000 + watermark_permille - 1) // watermark_permille + 1
+            own = {w: under_watermark(CacheManager.pages_for(w, max_batch, max_tokens, max_chunk, block_size))
+                   for w in CacheManager.windows_of(needs)}
+            kv_blocks = {w: n if kv_blocks is None else (int(kv_blocks) if w is None else min(int(kv_blocks), n)) for w, n in own.items()}
+        self.cache = CacheManager(needs, self.model.state_needs(), kv_blocks, block_size,
                                   max_requests=max(32, max_batch), device=self.model.rt.device, dtype=self.model.rt.dtype)
         self.step_fn = StepFunction(self.model, self.cache, n_positions=max_tokens)
-        # (pages are counted per request by what the group of layers that holds the most holds: everything,
-        # or, where every layer sees a window only, the window and a step's tokens)
-        self.sched_cfg = SchedConfig(token_budget, max_chunk, block_size, kv_blocks, watermark_permille, max_wait_ticks,
-                                     n_slots=max(32, max_batch), held_tokens=self.cache.held_tokens_bound(max_chunk))
+        # (the scheduler counts a request's pages in every group of layers by what that group holds of it:
+        # everything, or a window and a step's tokens; the group that binds decides)
+        self.sched_cfg = SchedConfig.for_groups(self.cache.group_rules(max_chunk), token_budget=token_budget, max_chunk=max_chunk,
+                                                block_size=block_size, watermark_permille=watermark_permille,
+                                                max_wait_ticks=max_wait_ticks, n_slots=max(32, max_batch))
         self.core = EngineCore(self.step_fn, self.sched_cfg, trace_path, share_prefixes=share_prefixes, run_ahead=run_ahead)
         self.seed = seed
         self._next_id = 1
@@ -60,7 +67,7 @@ class Engine:
         if report is not None:
             m = self.memory()
             report(f"[alofa_amd] device memory: weights {m['weights'] / 2**20:.1f} MiB + cache pool {m['cache_pool'] / 2**20:.1f} MiB "
-                   f"({kv_blocks} pages of {block_size} tokens x {len(self.cache.groups)} group(s)) + scratch {m['scratch'] / 2**20:.1f} MiB "
+                   f"({' + '.join(str(g.pool.n_blocks) for g in self.cache.groups) or 0} pages of {block_size} tokens in {len(self.cache.groups)} group(s)) + scratch {m['scratch'] / 2**20:.1f} MiB "
                    f"(grows to the largest step, then stays) = {m['total'] / 2**20:.1f} MiB")
 
     def memory(self) -> dict:

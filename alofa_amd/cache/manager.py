@@ -57,14 +57,38 @@ class CacheManager:
     [blocks, *page shape], and one state tensor per owner of state.
     ``cache_needs`` and ``state_needs`` map an owner's key (any hashable: the
     model uses (run entry, mixer index)) to its need; a list stands for the keys
-    0, 1, 2, ... with None where nothing is kept."""
+    0, 1, 2, ... with None where nothing is kept. ``n_blocks``: the pages of every
+    group's pool, or a dict from a group's window (None: the group that keeps every
+    key) to the pages of that group's pool; every owner's tensors have as many pages
+    as its group's pool, so a group that holds a window only can be given what its
+    window needs (``pages_for``)."""
 
-    def __init__(self, cache_needs, state_needs, n_blocks: int, block_size: int = 16,
+    @staticmethod
+    def windows_of(cache_needs) -> list:
+        """The groups that these needs make, as their windows in group order (None: every key is kept)."""
+        out: list = []
+        for need in _keyed(cache_needs).values():
+            if need.window not in out:
+                out.append(need.window)
+        return out
+
+    @staticmethod
+    def held_tokens_of(window: Optional[int], step_tokens: int, block_size: int) -> int:
+        """The most tokens a request holds pages for at any time in a group with this window, when a step
+        brings it at most ``step_tokens``: -1 for no bound (every key is kept), else the window plus the step
+        plus the two pages that the window's ends may lie in."""
+        return -1 if window is None else int(window) + int(step_tokens) + 2 * int(block_size)
+
+    @staticmethod
+    def pages_for(window: Optional[int], requests: int, tokens: int, step_tokens: int, block_size: int) -> int:
+        """Pages that ``requests`` requests of up to ``tokens`` tokens hold at most in a group with this window."""
+        held = CacheManager.held_tokens_of(window, step_tokens, block_size)
+        return max(1, requests * blocks_for(tokens if held < 0 else min(tokens, held), block_size))
+
+    def __init__(self, cache_needs, state_needs, n_blocks, block_size: int = 16,
                  max_requests: int = 64, device=None, dtype=torch.bfloat16):
         if block_size <= 0 or max_requests <= 0:
             raise AlofaError("invalid_argument", "block_size and max_requests must be positive", f"block_size={block_size} max_requests={max_requests}")
-        if n_blocks <= 0:
-            raise AlofaError("invalid_argument", "a pool needs at least one block", f"n_blocks={n_blocks}")
         self.block_size = block_size
         self.max_requests = max_requests
         windows: list = []
@@ -78,9 +102,20 @@ class CacheManager:
             g = windows.index(need.window)
             entries[g].append(i)
             self.group_of_entry[i] = g
+        if isinstance(n_blocks, dict):
+            missing = [w for w in windows if w not in n_blocks]
+            if missing:
+                raise AlofaError("invalid_argument", "no page count for a group of layers", f"windows={missing} given={sorted(n_blocks, key=str)}")
+            pages = [int(n_blocks[w]) for w in windows]
+        else:
+            pages = [int(n_blocks)] * len(windows)
+            if int(n_blocks) <= 0:
+                raise AlofaError("invalid_argument", "a pool needs at least one block", f"n_blocks={n_blocks}")
+        if any(n <= 0 for n in pages):
+            raise AlofaError("invalid_argument", "a pool needs at least one block", f"n_blocks={n_blocks}")
         self._lib = hostlib.lib()
         self._h = ctypes.c_void_p(self._lib.alofa_cache_new(len(windows), hostlib.long_array([-1 if w is None else w for w in windows]),
-                                                             n_blocks, block_size, max_requests))
+                                                             hostlib.long_array(pages), block_size, max_requests))
         self.groups = [Group(w, entries[g], BlockPool(0, _borrowed=self._lib.alofa_cache_pool(self._h, g))) for g, w in enumerate(windows)]
         self.requests: dict = {}      # request key -> its slot
         self.needs = cache_needs
@@ -90,7 +125,7 @@ class CacheManager:
         self.device = device
         if device is not None:
             for i, need in cache_needs.items():
-                self.tensors[i] = {t.name: torch.zeros((n_blocks, *t.page_shape(block_size)), dtype=t.dtype or dtype, device=device)
+                self.tensors[i] = {t.name: torch.zeros((pages[self.group_of_entry[i]], *t.page_shape(block_size)), dtype=t.dtype or dtype, device=device)
                                    for t in need.tensors}
             for i, need in state_needs.items():
                 self.state[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
@@ -208,16 +243,13 @@ class CacheManager:
             row_slots.ctypes.data_as(lp), ctypes.c_int64(T)))
         return pos0, positions, req_of_token, tables, row_slots
 
-    def held_tokens_bound(self, step_tokens: int) -> int:
-        """The most tokens a request holds pages for at any time, in the group that holds the most,
-        when a step brings it at most ``step_tokens``: -1 for no bound (some group keeps every key),
-        0 where no group keeps pages at all, else the longest window plus the step plus the two pages
-        that a window's ends may lie in. What the scheduler counts a request's pages by."""
+    def group_rules(self, step_tokens: int) -> list:
+        """What the scheduler counts a request's pages by, per group: (pages of the group's pool, the most
+        tokens a request holds pages for in it when a step brings it at most ``step_tokens``: ``held_tokens_of``).
+        A model none of whose layers keeps pages has one rule, (1, 0): nothing is held, nothing binds."""
         if not self.groups:
-            return 0
-        if any(g.window is None for g in self.groups):
-            return -1
-        return max(g.window for g in self.groups) + int(step_tokens) + 2 * self.block_size
+            return [(1, 0)]
+        return [(g.pool.n_blocks, self.held_tokens_of(g.window, step_tokens, self.block_size)) for g in self.groups]
 
     def step_width(self, slots: np.ndarray, n_tokens: np.ndarray) -> int:
         """How many blocks the longest request of a step will hold once the step's tokens are in:

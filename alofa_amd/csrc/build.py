@@ -107,7 +107,7 @@ def load_host() -> ctypes.CDLL:
         _host.alofa_host_last_error.restype = c.c_char_p
         for name in ("alofa_pool_new", "alofa_cache_new", "alofa_cache_pool", "alofa_sched_new"):
             getattr(_host, name).restype = c.c_void_p
-        for name in ("alofa_cache_length", "alofa_sched_scalar"):
+        for name in ("alofa_cache_length", "alofa_sched_scalar", "alofa_sched_scalar_of"):
             getattr(_host, name).restype = c.c_int64
     return _host
 

@@ -145,47 +145,69 @@ struct Cache {
 constexpr int ST_FREE = 0, ST_WAITING = 1, ST_RUNNING = 2;
 constexpr int64_t DIGEST_MOD = 2147483647, DIGEST_MUL = 1000003;
 
-struct SchedConfig {
-  int64_t token_budget, max_chunk, block_size, capacity_blocks, watermark_permille, max_wait_ticks;
-  int n_slots;
-  // The most tokens a request holds pages for at any time, in the group of layers that holds the most: below
-  // zero for no bound (a group that keeps every key, the reference's only case), a window's length plus what
-  // a step adds where every group gives back what a window has passed, 0 where no layer keeps pages at all.
-  int64_t held_tokens;
-  int64_t threshold() const { return capacity_blocks * watermark_permille / 1000; }
-  // pages a request of this many tokens holds
-  int64_t blocks(int64_t tokens) const { return blocks_for(held_tokens < 0 ? tokens : std::min(tokens, held_tokens), block_size); }
+// What the scheduler knows of one group of layers: its pool's pages, and the most tokens a request holds pages
+// for in it at any time: below zero for no bound (a group that keeps every key, the reference's only case), a
+// window's length plus what a step adds where the group gives back what its window has passed, 0 where it keeps
+// no pages at all.
+struct GroupRule {
+  int64_t capacity, held_tokens;
 };
+
+struct SchedConfig {
+  int64_t token_budget, max_chunk, block_size, watermark_permille, max_wait_ticks;
+  int n_slots;
+  std::vector<GroupRule> groups;  // at least one; the first is the one the reference's single count stands for
+  int n_groups() const { return static_cast<int>(groups.size()); }
+  int64_t threshold(int g) const { return groups[g].capacity * watermark_permille / 1000; }
+  // pages a request of this many tokens holds in group g
+  int64_t blocks(int g, int64_t tokens) const {
+    const int64_t held = groups[g].held_tokens;
+    return blocks_for(held < 0 ? tokens : std::min(tokens, held), block_size);
+  }
+};
+
+// cfg: token_budget, max_chunk, block_size, capacity_blocks, watermark_permille, max_wait_ticks, n_slots, held_tokens,
+// n_more, then (capacity_blocks, held_tokens) of every further group
+SchedConfig config_from(const int64_t* cfg) {
+  SchedConfig c{cfg[0], cfg[1], cfg[2], cfg[4], cfg[5], static_cast<int>(cfg[6]), {GroupRule{cfg[3], cfg[7]}}};
+  for (int64_t g = 0; g < cfg[8]; ++g) c.groups.push_back(GroupRule{cfg[9 + 2 * g], cfg[10 + 2 * g]});
+  return c;
+}
 
 struct Action {
   std::vector<int64_t> prefill;  // triples id, start, end
   std::vector<int64_t> decode, preempted, finished;
 };
 
+// Every count of pages is kept per group of layers, and every decision holds for all groups at once: a request
+// is admitted, a chunk runs, a decode proceeds only where no group's bound is passed; the group that binds
+// decides. With one group this is the reference's arithmetic number for number.
 struct Sched {
   SchedConfig cfg;
   std::vector<int64_t> ids, prompt_len, done, generated, max_new, state, wait_ticks, preempt_count;
-  int64_t blocks_used = 0, cached_blocks = 0, preempt_total = 0, tick_seq = 0;
+  std::vector<int64_t> blocks_used, cached_blocks;  // per group
+  int64_t preempt_total = 0, tick_seq = 0;
 
-  explicit Sched(const SchedConfig& c) : cfg(c) {
+  explicit Sched(const SchedConfig& c) : cfg(c), blocks_used(c.groups.size(), 0), cached_blocks(c.groups.size(), 0) {
     for (auto* v : {&ids, &prompt_len, &done, &generated, &max_new, &state, &wait_ticks, &preempt_count}) v->assign(c.n_slots, 0);
   }
+  int G() const { return cfg.n_groups(); }
   int find(int64_t req) const {
     for (int i = 0; i < cfg.n_slots; ++i)
       if (state[i] != ST_FREE && ids[i] == req) return i;
     return -1;
   }
   int n_live() const { return static_cast<int>(std::count_if(state.begin(), state.end(), [](int64_t s) { return s != ST_FREE; })); }
-  int64_t blocks_held() const {
+  int64_t blocks_held(int g) const {
     int64_t t = 0;
     for (int i = 0; i < cfg.n_slots; ++i)
-      if (state[i] != ST_FREE) t += cfg.blocks(done[i] + generated[i]);
+      if (state[i] != ST_FREE) t += cfg.blocks(g, done[i] + generated[i]);
     return t;
   }
-  int64_t blocks_wanted() const {
+  int64_t blocks_wanted(int g) const {
     int64_t t = 0;
     for (int i = 0; i < cfg.n_slots; ++i)
-      if (state[i] == ST_WAITING) t += std::max<int64_t>(0, cfg.blocks(prompt_len[i]) - cfg.blocks(done[i]));
+      if (state[i] == ST_WAITING) t += std::max<int64_t>(0, cfg.blocks(g, prompt_len[i]) - cfg.blocks(g, done[i]));
     return t;
   }
   int64_t digest() const {
@@ -193,22 +215,43 @@ struct Sched {
     for (int i = 0; i < cfg.n_slots; ++i)
       for (int64_t x : {state[i], ids[i], prompt_len[i], done[i], generated[i], max_new[i], wait_ticks[i], preempt_count[i]})
         h = (h * DIGEST_MUL + x) % DIGEST_MOD;
-    for (int64_t x : {blocks_used, cached_blocks, preempt_total}) h = (h * DIGEST_MUL + x) % DIGEST_MOD;
+    for (int64_t x : {blocks_used[0], cached_blocks[0], preempt_total}) h = (h * DIGEST_MUL + x) % DIGEST_MOD;
+    for (int g = 1; g < G(); ++g)  // (further groups follow; with one group the value is the reference's)
+      for (int64_t x : {blocks_used[g], cached_blocks[g]}) h = (h * DIGEST_MUL + x) % DIGEST_MOD;
     return h;
   }
-  int64_t committed() const {
+  int64_t committed(int g) const {
     int64_t t = 0;
     for (int i = 0; i < cfg.n_slots; ++i)
-      if (state[i] != ST_FREE) t += cfg.blocks(prompt_len[i] + max_new[i]);
+      if (state[i] != ST_FREE) t += cfg.blocks(g, prompt_len[i] + max_new[i]);
     return t;
+  }
+  // pages the growth from `from` to `to` tokens takes, per group, and whether they fit under every group's capacity
+  // (a group that is asked for nothing is looked at only with `also_idle`: the reference's decode phase does not, its
+  // prefill phase does)
+  bool growth_fits(int64_t from, int64_t to, std::vector<int64_t>& need, bool also_idle) const {
+    bool fits = true;
+    need.resize(G());
+    for (int g = 0; g < G(); ++g) {
+      need[g] = cfg.blocks(g, to) - cfg.blocks(g, from);
+      fits &= (need[g] <= 0 && !also_idle) || blocks_used[g] + need[g] <= cfg.groups[g].capacity;
+    }
+    return fits;
+  }
+  bool over_watermark() const {
+    for (int g = 0; g < G(); ++g)
+      if (blocks_used[g] > cfg.threshold(g)) return true;
+    return false;
   }
   int admit(int64_t req, int64_t p_len, int64_t m_new) {
     if (p_len <= 0) return fail(kInvalidArgument, "prompt_len must be positive [request=%lld]", (long long)req);
     if (m_new <= 0) return fail(kInvalidArgument, "max_new must be positive [request=%lld]", (long long)req);
     if (find(req) >= 0) return fail(kInvalidArgument, "duplicate request id [request=%lld]", (long long)req);
-    if (cfg.blocks(p_len) > cfg.capacity_blocks) return fail(kCapacity, "prompt does not fit in the kv pool [request=%lld]", (long long)req);
-    if (committed() + cfg.blocks(p_len + m_new) > cfg.threshold())
-      return fail(kCapacity, "concurrent sequences exceed the kv watermark [request=%lld]", (long long)req);
+    for (int g = 0; g < G(); ++g)
+      if (cfg.blocks(g, p_len) > cfg.groups[g].capacity) return fail(kCapacity, "prompt does not fit in the kv pool [request=%lld]", (long long)req);
+    for (int g = 0; g < G(); ++g)
+      if (committed(g) + cfg.blocks(g, p_len + m_new) > cfg.threshold(g))
+        return fail(kCapacity, "concurrent sequences exceed the kv watermark [request=%lld]", (long long)req);
     int slot = -1;
     for (int i = 0; i < cfg.n_slots && slot < 0; ++i)
       if (state[i] == ST_FREE) slot = i;
@@ -219,13 +262,15 @@ struct Sched {
     return 0;
   }
   void release(int slot, bool to_cache) {
-    const int64_t held = cfg.blocks(done[slot] + generated[slot]);
-    if (to_cache) {
-      const int64_t whole = cfg.blocks(prompt_len[slot] + max_new[slot]);
-      blocks_used += whole - held;
-      cached_blocks += whole;
-    } else {
-      blocks_used -= held;
+    for (int g = 0; g < G(); ++g) {
+      const int64_t held = cfg.blocks(g, done[slot] + generated[slot]);
+      if (to_cache) {
+        const int64_t whole = cfg.blocks(g, prompt_len[slot] + max_new[slot]);
+        blocks_used[g] += whole - held;
+        cached_blocks[g] += whole;
+      } else {
+        blocks_used[g] -= held;
+      }
     }
     ids[slot] = prompt_len[slot] = done[slot] = generated[slot] = max_new[slot] = wait_ticks[slot] = preempt_count[slot] = 0;
     state[slot] = ST_FREE;
@@ -234,7 +279,7 @@ struct Sched {
     for (int i = cfg.n_slots - 1; i >= 0; --i) {
       if (i != protect && state[i] == ST_RUNNING && done[i] + generated[i] > 0) {
         act.preempted.push_back(ids[i]);
-        blocks_used -= cfg.blocks(done[i] + generated[i]);
+        for (int g = 0; g < G(); ++g) blocks_used[g] -= cfg.blocks(g, done[i] + generated[i]);
         done[i] = generated[i] = wait_ticks[i] = 0;
         ++preempt_count[i];
         ++preempt_total;
@@ -249,24 +294,24 @@ struct Sched {
     const int64_t chunk = std::min({cfg.max_chunk, prompt_len[slot] - done[slot], budget});
     if (chunk <= 0) return budget;
     const int64_t new_done = done[slot] + chunk;
-    const int64_t need = cfg.blocks(new_done) - cfg.blocks(done[slot]);
-    if (blocks_used + need > cfg.capacity_blocks) return budget;  // pages ran out: this request waits for a later tick
+    std::vector<int64_t> need;
+    if (!growth_fits(done[slot], new_done, need, true)) return budget;  // pages ran out: this request waits for a later tick
     act.prefill.insert(act.prefill.end(), {ids[slot], done[slot], new_done});
-    blocks_used += need;
+    for (int g = 0; g < G(); ++g) blocks_used[g] += need[g];
     done[slot] = new_done;
     progressed[slot] = 1;
     wait_ticks[slot] = 0;
     return budget - chunk;
   }
-  int step(const int64_t* arrivals, int n_arr, const int64_t* cancelled, int n_c, const int64_t* finished, int n_f, int64_t freed, Action& act) {
+  // freed: per group, cache blocks the engine gave back
+  int step(const int64_t* arrivals, int n_arr, const int64_t* cancelled, int n_c, const int64_t* finished, int n_f, const int64_t* freed, Action& act) {
     const int n = cfg.n_slots;
     ++tick_seq;
     std::vector<char> progressed(n, 0);
-    if (freed > 0) {  // 0
-      if (freed > cached_blocks) return fail(kInvalidArgument, "engine freed more blocks than the scheduler holds cached");
-      cached_blocks -= freed;
-      blocks_used -= freed;
-    }
+    for (int g = 0; g < G(); ++g)  // 0
+      if (freed[g] > cached_blocks[g]) return fail(kInvalidArgument, "engine freed more blocks than the scheduler holds cached");
+    for (int g = 0; g < G(); ++g)
+      if (freed[g] > 0) cached_blocks[g] -= freed[g], blocks_used[g] -= freed[g];
     for (int i = 0; i < n_c; ++i) {  // 1
       const int slot = find(cancelled[i]);
       if (slot >= 0) release(slot, false);
@@ -296,14 +341,13 @@ struct Sched {
     for (int i = 0; i < n; ++i)  // 5
       if (state[i] == ST_WAITING && done[i] >= prompt_len[i] && prompt_len[i] > 0) state[i] = ST_RUNNING, wait_ticks[i] = 0;
     int64_t budget = cfg.token_budget;
+    std::vector<int64_t> need;
     for (int i = 0; i < n && budget > 0; ++i) {  // 6
       if (state[i] != ST_RUNNING) continue;
       const int64_t seq = done[i] + generated[i];
-      const int64_t need = cfg.blocks(seq + 1) - cfg.blocks(seq);
-      if (need > 0)
-        while (blocks_used + need > cfg.capacity_blocks)
-          if (!preempt_one(act, i)) return fail(kCapacity, "kv pool too small for this batch");
-      blocks_used += need;
+      while (!growth_fits(seq, seq + 1, need, false))
+        if (!preempt_one(act, i)) return fail(kCapacity, "kv pool too small for this batch");
+      for (int g = 0; g < G(); ++g) blocks_used[g] += need[g];
       ++generated[i];
       act.decode.push_back(ids[i]);
       --budget;
@@ -316,7 +360,7 @@ struct Sched {
       if (state[i] == ST_WAITING && wait_ticks[i] >= cfg.max_wait_ticks) budget = try_prefill(i, budget, act, progressed);
     for (int i = 0; i < n; ++i)  // 8
       if (state[i] == ST_WAITING) budget = try_prefill(i, budget, act, progressed);
-    while (blocks_used > cfg.threshold())  // 9
+    while (over_watermark())  // 9
       if (!preempt_one(act, -1)) break;
     return 0;
   }
@@ -350,10 +394,13 @@ int alofa_pool_high_water(void* p) { return static_cast<Pool*>(p)->high_water; }
 int alofa_pool_n_blocks(void* p) { return static_cast<Pool*>(p)->n_blocks; }
 
 // ---- cache
-void* alofa_cache_new(int n_groups, const int64_t* windows, int n_blocks, int block_size, int max_requests) {
-  if (n_groups < 0 || n_blocks <= 0 || block_size <= 0 || max_requests <= 0) return nullptr;
+// n_blocks: the pages of every group's own pool
+void* alofa_cache_new(int n_groups, const int64_t* windows, const int64_t* n_blocks, int block_size, int max_requests) {
+  if (n_groups < 0 || block_size <= 0 || max_requests <= 0) return nullptr;
+  for (int g = 0; g < n_groups; ++g)
+    if (n_blocks[g] <= 0 || n_blocks[g] > INT32_MAX) return nullptr;
   Cache* c = new Cache{block_size, max_requests, {}, {}, {}};
-  for (int g = 0; g < n_groups; ++g) c->groups.push_back(Group{windows[g], Pool(n_blocks)});
+  for (int g = 0; g < n_groups; ++g) c->groups.push_back(Group{windows[g], Pool(static_cast<int>(n_blocks[g]))});
   c->reqs.resize(max_requests);
   for (int s = max_requests - 1; s >= 0; --s) c->free_slots.push_back(s);
   return c;
@@ -523,7 +570,16 @@ int alofa_cache_plan_step(void* cv, int n_entries, const int* slots, const int* 
       if (slots[j] == slots[i]) return fail(kInvalidArgument, "a request appears twice in one step [slot=%d]", slots[i]);
     if (r->length + n_tokens[i] > max_positions)
       return fail(kCapacity, "the request would pass the context bound [slot=%d length=%lld bound=%lld]", slots[i], (long long)(r->length + n_tokens[i]), (long long)max_positions);
-    for (int g = 0; g < G; ++g) need[g] += c->needed(*r, g, r->length + n_tokens[i]);
+    for (int g = 0; g < G; ++g) {
+      need[g] += c->needed(*r, g, r->length + n_tokens[i]);
+      const int64_t wide = std::max<int64_t>(blocks_for(r->length + n_tokens[i], c->block_size), r->tables[g].size());
+      if (wide > width) return fail(kCapacity, "table is wider than the buffer [width=%d need=%d]", width, (int)wide);
+      // pages held already for positions this step writes (reserved earlier, or the tail of the last one) must still be there
+      const int64_t last = std::min<int64_t>(blocks_for(r->length + n_tokens[i], c->block_size), r->tables[g].size());
+      for (int64_t b = r->length / c->block_size; b < last; ++b)
+        if (r->tables[g][b] < 0)
+          return fail(kCapacity, "no page is held for this position [slot=%d group=%d position=%lld]", slots[i], g, (long long)std::max<int64_t>(r->length, b * c->block_size));
+    }
     rows += n_tokens[i];
   }
   if (rows != total_rows) return fail(kInvalidArgument, "row count does not fit the buffers [rows=%lld buffers=%lld]", (long long)rows, (long long)total_rows);
@@ -535,8 +591,7 @@ int alofa_cache_plan_step(void* cv, int n_entries, const int* slots, const int* 
     c->reserve(slots[i], r.length + n_tokens[i]);
     pos0[i] = r.length;
     for (int g = 0; g < G; ++g) {
-      const auto& t = r.tables[g];
-      if (static_cast<int>(t.size()) > width) return fail(kCapacity, "table is wider than the buffer [width=%d need=%d]", width, (int)t.size());
+      const auto& t = r.tables[g];  // (no wider than the buffer: checked above, before anything was taken)
       int* dst = tables + (static_cast<int64_t>(g) * n_entries + i) * width;
       std::copy(t.begin(), t.end(), dst);
       std::fill(dst + t.size(), dst + width, -1);
@@ -546,8 +601,7 @@ int alofa_cache_plan_step(void* cv, int n_entries, const int* slots, const int* 
       positions[row] = static_cast<int>(p);
       req_of_token[row] = i;
       for (int g = 0; g < G; ++g) {
-        const int page = r.tables[g][p / c->block_size];
-        if (page < 0) return fail(kCapacity, "no page is held for this position [slot=%d group=%d position=%lld]", slots[i], g, (long long)p);
+        const int page = r.tables[g][p / c->block_size];  // (held: checked above, or taken just now)
         row_slots[static_cast<int64_t>(g) * total_rows + row] = static_cast<int64_t>(page) * c->block_size + p % c->block_size;
       }
     }
@@ -566,22 +620,25 @@ int alofa_cache_commit_step(void* cv, int n_entries, const int* slots, const int
 }
 
 // ---- scheduler
-// cfg8: token_budget, max_chunk, block_size, capacity_blocks, watermark_permille, max_wait_ticks, n_slots, held_tokens
-void* alofa_sched_new(const int64_t* cfg8) {
-  return new Sched(SchedConfig{cfg8[0], cfg8[1], cfg8[2], cfg8[3], cfg8[4], cfg8[5], static_cast<int>(cfg8[6]), cfg8[7]});
+// cfg: see config_from
+void* alofa_sched_new(const int64_t* cfg) {
+  if (cfg[8] < 0) return nullptr;
+  return new Sched(config_from(cfg));
 }
 void alofa_sched_free(void* s) { delete static_cast<Sched*>(s); }
-// a new configuration for the next ticks (the slot count cannot change)
-int alofa_sched_set_config(void* sv, const int64_t* cfg8) {
+// a new configuration for the next ticks (neither the slot count nor the number of groups can change)
+int alofa_sched_set_config(void* sv, const int64_t* cfg) {
   Sched* s = static_cast<Sched*>(sv);
-  if (cfg8[6] != s->cfg.n_slots) return fail(kInvalidArgument, "the slot count of a scheduler cannot change");
-  s->cfg = SchedConfig{cfg8[0], cfg8[1], cfg8[2], cfg8[3], cfg8[4], cfg8[5], static_cast<int>(cfg8[6]), cfg8[7]};
+  if (cfg[6] != s->cfg.n_slots) return fail(kInvalidArgument, "the slot count of a scheduler cannot change");
+  if (cfg[8] + 1 != s->G()) return fail(kInvalidArgument, "the number of groups of a scheduler cannot change");
+  s->cfg = config_from(cfg);
   return 0;
 }
+// freed: per group, the cache blocks the engine gave back.
 // out: prefill triples, then decode, preempted, finished ids, each at offset k * cap of `out` (4 * cap long);
 // counts[4]; scalars: tick_seq, preempt_total, state_digest
 int alofa_sched_step(void* sv, const int64_t* arrivals, int n_arr, const int64_t* cancelled, int n_c, const int64_t* finished, int n_f,
-                     int64_t freed, int64_t* out, int cap, int* counts, int64_t* scalars) {
+                     const int64_t* freed, int64_t* out, int cap, int* counts, int64_t* scalars) {
   Sched* s = static_cast<Sched*>(sv);
   Action act;
   if (int e = s->step(arrivals, n_arr, cancelled, n_c, finished, n_f, freed, act)) return e;
@@ -598,10 +655,13 @@ int alofa_sched_find(void* s, int64_t req) { return static_cast<Sched*>(s)->find
 int alofa_sched_would_admit(void* sv, int64_t p_len, int64_t m_new, const int64_t* pending, int n_pending) {
   Sched* s = static_cast<Sched*>(sv);
   const SchedConfig& c = s->cfg;
-  if (p_len <= 0 || m_new <= 0 || c.blocks(p_len) > c.capacity_blocks) return 0;
-  int64_t committed = s->committed();
-  for (int i = 0; i < n_pending; ++i) committed += c.blocks(pending[2 * i] + pending[2 * i + 1]);
-  if (committed + c.blocks(p_len + m_new) > c.threshold()) return 0;
+  if (p_len <= 0 || m_new <= 0) return 0;
+  for (int g = 0; g < s->G(); ++g) {
+    if (c.blocks(g, p_len) > c.groups[g].capacity) return 0;
+    int64_t committed = s->committed(g);
+    for (int i = 0; i < n_pending; ++i) committed += c.blocks(g, pending[2 * i] + pending[2 * i + 1]);
+    if (committed + c.blocks(g, p_len + m_new) > c.threshold(g)) return 0;
+  }
   return s->n_live() + n_pending < c.n_slots;
 }
 // which: 0 ids, 1 prompt_len, 2 done, 3 generated, 4 max_new, 5 state, 6 wait_ticks, 7 preempt_count
@@ -612,20 +672,23 @@ int alofa_sched_slots(void* sv, int which, int64_t* out) {
   std::copy(v[which]->begin(), v[which]->end(), out);
   return 0;
 }
-// which: 0 blocks_used, 1 cached_blocks, 2 preempt_total, 3 tick_seq, 4 blocks_held, 5 blocks_wanted, 6 digest, 7 n_live
-int64_t alofa_sched_scalar(void* sv, int which) {
+// which: 0 blocks_used, 1 cached_blocks, 2 preempt_total, 3 tick_seq, 4 blocks_held, 5 blocks_wanted, 6 digest, 7 n_live;
+// the counts of pages are those of group `g`
+int64_t alofa_sched_scalar_of(void* sv, int which, int g) {
   Sched* s = static_cast<Sched*>(sv);
+  if (g < 0 || g >= s->G()) return fail(kOutOfRange, "no such group [group=%d]", g);
   switch (which) {
-    case 0: return s->blocks_used;
-    case 1: return s->cached_blocks;
+    case 0: return s->blocks_used[g];
+    case 1: return s->cached_blocks[g];
     case 2: return s->preempt_total;
     case 3: return s->tick_seq;
-    case 4: return s->blocks_held();
-    case 5: return s->blocks_wanted();
+    case 4: return s->blocks_held(g);
+    case 5: return s->blocks_wanted(g);
     case 6: return s->digest();
     case 7: return s->n_live();
   }
   return fail(kOutOfRange, "no such scalar [which=%d]", which);
 }
+int64_t alofa_sched_scalar(void* sv, int which) { return alofa_sched_scalar_of(sv, which, 0); }
 
 }  // extern "C"

@@ -74,9 +74,15 @@ class EngineCore:
         self.share_prefixes = bool(share_prefixes)
         self.shared_tokens = 0
         self.cache = step_fn.cache
-        pool_blocks = min((g.pool.n_blocks for g in self.cache.groups), default=sched_cfg.capacity_blocks)
-        if sched_cfg.capacity_blocks > pool_blocks:
-            raise AlofaError("invalid_argument", "the scheduler counts more blocks than the pool has", f"scheduler={sched_cfg.capacity_blocks} pool={pool_blocks}")
+        # the scheduler counts the pages of every group of layers: one rule per group (a scheduler with a single
+        # rule over several groups counts for all of them with it, so every pool must hold what it counts)
+        rules, pools = sched_cfg.groups, [g.pool.n_blocks for g in self.cache.groups]
+        if len(rules) not in (1, len(pools)):
+            raise AlofaError("invalid_argument", "the scheduler's groups are not the cache's", f"scheduler={len(rules)} cache={len(pools)}")
+        for g, n in enumerate(pools):
+            capacity = rules[g if len(rules) > 1 else 0][0]
+            if capacity > n:
+                raise AlofaError("invalid_argument", "the scheduler counts more blocks than the pool has", f"group={g} scheduler={capacity} pool={n}")
         if sched_cfg.block_size != self.cache.block_size:
             raise AlofaError("invalid_argument", "scheduler and cache disagree on the block size", f"scheduler={sched_cfg.block_size} cache={self.cache.block_size}")
         self.sched = Scheduler(sched_cfg)
@@ -84,7 +90,7 @@ class EngineCore:
         self._arrivals: list = []
         self._cancels: list = []
         self._to_report: list = []
-        self._freed_blocks = 0
+        self._freed_blocks = [0] * len(rules)     # per group of the scheduler
         # blocks the scheduler charges a request with when it finishes (prompt + max_new), kept from
         # submission until the scheduler has let go of the id: a finished request may be released
         # before the tick that reports its completion
@@ -110,7 +116,8 @@ class EngineCore:
             raise AlofaError("out_of_range", "token id outside the vocabulary", f"request={req} vocab={vocab}")
         self.requests[req] = Request(req, [int(t) for t in prompt], int(max_new), params or SampleParams(temperature=0.0), int(seed),
                                      rng=SplitMix64(seed))
-        self._charge[req] = self.sched.cfg.blocks(len(prompt) + int(max_new))
+        cfg = self.sched.cfg
+        self._charge[req] = [cfg.blocks(len(prompt) + int(max_new), g) for g in range(len(cfg.groups))]
         self._arrivals.append(req)
 
     def can_admit(self, prompt_len: int, max_new: int) -> bool:
@@ -136,7 +143,7 @@ class EngineCore:
         del self.requests[req]
 
     def has_work(self) -> bool:
-        return (bool(self._arrivals) or bool(self._cancels) or bool(self._to_report) or self._freed_blocks > 0
+        return (bool(self._arrivals) or bool(self._cancels) or bool(self._to_report) or any(self._freed_blocks)
                 or bool(self._inflight) or any(r.state != DONE for r in self.requests.values()))
 
     def _scheduler_let_go(self, cancelled: list, finished: list) -> None:
@@ -151,7 +158,8 @@ class EngineCore:
                 self._drop(r)
                 r.state = DONE
         for f in finished:
-            self._freed_blocks += self._charge.pop(f, 0)
+            for g, n in enumerate(self._charge.pop(f, ())):
+                self._freed_blocks[g] += n
 
     # ---------------------------------------------------------------- tick
     def _drop(self, r: Request) -> None:
@@ -162,9 +170,9 @@ class EngineCore:
         """One scheduler tick; returns the entries of the step and who owes a token."""
         inp = SchedInput(
             arrivals=[(a, len(self.requests[a].prompt), self.requests[a].max_new) for a in self._arrivals],
-            cancelled=list(self._cancels), finished=list(self._to_report), freed_blocks=self._freed_blocks)
+            cancelled=list(self._cancels), finished=list(self._to_report), freed_blocks=list(self._freed_blocks))
         arrivals, self._arrivals = self._arrivals, []
-        self._cancels, self._to_report, self._freed_blocks = [], [], 0
+        self._cancels, self._to_report, self._freed_blocks = [], [], [0] * len(self._freed_blocks)
         try:
             act = self.sched.step(inp)
         except AlofaError:

@@ -49,20 +49,36 @@ class SchedConfig:
     # the reference, whose layers all keep every key): below zero for no bound, a window's length plus what a
     # step adds where every group gives back what its window has passed, 0 where no layer keeps pages.
     held_tokens: int = -1
+    # Further groups of layers with pools of their own, (capacity_blocks, held_tokens) each: every count and every
+    # decision is made per group, and the group that binds decides (not in the reference, which has one group).
+    more_groups: tuple = ()
+
+    @classmethod
+    def for_groups(cls, rules: list, **fields) -> "SchedConfig":
+        """A configuration from (capacity_blocks, held_tokens) per group (``CacheManager.group_rules``)."""
+        (capacity, held), more = rules[0], tuple((int(c), int(h)) for c, h in rules[1:])
+        return cls(capacity_blocks=int(capacity), held_tokens=int(held), more_groups=more, **fields)
+
+    @property
+    def groups(self) -> tuple:
+        return ((self.capacity_blocks, self.held_tokens), *self.more_groups)
 
     def __post_init__(self):
         if self.token_budget < 0 or self.max_chunk <= 0 or self.block_size <= 0 or self.capacity_blocks <= 0:
             raise AlofaError("invalid_argument", "scheduler sizes must be positive", repr(self))
         if not 0 < self.watermark_permille <= 1000 or self.max_wait_ticks < 0 or self.n_slots <= 0:
             raise AlofaError("invalid_argument", "watermark is 1..1000 permille, wait ticks and slots non-negative", repr(self))
+        if any(len(g) != 2 or g[0] <= 0 for g in self.more_groups):
+            raise AlofaError("invalid_argument", "a further group is (capacity_blocks > 0, held_tokens)", repr(self))
 
     @property
     def threshold_blocks(self) -> int:
         return self.capacity_blocks * self.watermark_permille // 1000
 
-    def blocks(self, tokens: int) -> int:
-        """Pages that a request of ``tokens`` tokens holds (in the group that holds the most)."""
-        return blocks_for(tokens if self.held_tokens < 0 else min(tokens, self.held_tokens), self.block_size)
+    def blocks(self, tokens: int, group: int = 0) -> int:
+        """Pages that a request of ``tokens`` tokens holds in ``group``."""
+        held = self.groups[group][1]
+        return blocks_for(tokens if held < 0 else min(tokens, held), self.block_size)
 
 
 @dataclass
@@ -70,7 +86,7 @@ class SchedInput:
     arrivals: list = field(default_factory=list)    # (id, prompt_len, max_new)
     cancelled: list = field(default_factory=list)
     finished: list = field(default_factory=list)    # completions the engine reports
-    freed_blocks: int = 0                           # cache blocks the engine gave back
+    freed_blocks: object = 0                        # cache blocks the engine gave back: of the first group, or a list per group
 
 
 @dataclass
@@ -111,7 +127,8 @@ class Scheduler:
     @staticmethod
     def _cfg_array(cfg: SchedConfig):
         return hostlib.long_array([cfg.token_budget, cfg.max_chunk, cfg.block_size, cfg.capacity_blocks,
-                                   cfg.watermark_permille, cfg.max_wait_ticks, cfg.n_slots, cfg.held_tokens])
+                                   cfg.watermark_permille, cfg.max_wait_ticks, cfg.n_slots, cfg.held_tokens,
+                                   len(cfg.more_groups), *(x for g in cfg.more_groups for x in g)])
 
     @property
     def cfg(self) -> SchedConfig:
@@ -119,7 +136,7 @@ class Scheduler:
 
     @cfg.setter
     def cfg(self, cfg: SchedConfig) -> None:
-        """A new configuration for the next ticks (the slot count cannot change)."""
+        """A new configuration for the next ticks (neither the slot count nor the number of groups can change)."""
         hostlib.check(self._lib.alofa_sched_set_config(self._h, self._cfg_array(cfg)))
         self._cfg = cfg
 
@@ -132,6 +149,11 @@ class Scheduler:
         if name in Scheduler._SCALARS:
             return int(self._lib.alofa_sched_scalar(self._h, Scheduler._SCALARS.index(name)))
         raise AttributeError(name)
+
+    def of_group(self, name: str, group: int) -> int:
+        """``blocks_used``, ``cached_blocks``, ``blocks_held`` or ``blocks_wanted`` of one group."""
+        which = {"blocks_used": 0, "cached_blocks": 1, "blocks_held": 4, "blocks_wanted": 5}[name]
+        return hostlib.check(int(self._lib.alofa_sched_scalar_of(self._h, which, group)))
 
     def find(self, req: int) -> int:
         return self._lib.alofa_sched_find(self._h, ctypes.c_int64(req))
@@ -167,9 +189,13 @@ class Scheduler:
         if len(inp.arrivals) + 8 > self._cap // 4:   # the out buffer must hold every list an action can carry
             self._cap = 4 * (len(inp.arrivals) + self._cfg.n_slots + 8)
             self._out = hostlib.long_array(4 * self._cap)
+        G = 1 + len(self._cfg.more_groups)
+        freed = list(inp.freed_blocks) if isinstance(inp.freed_blocks, (list, tuple)) else [int(inp.freed_blocks)] + [0] * (G - 1)
+        if len(freed) != G:
+            raise AlofaError("invalid_argument", "freed blocks are one count per group", f"groups={G} given={len(freed)}")
         hostlib.check(self._lib.alofa_sched_step(
             self._h, hostlib.long_array(flat), len(inp.arrivals), hostlib.long_array(list(inp.cancelled)), len(inp.cancelled),
-            hostlib.long_array(list(inp.finished)), len(inp.finished), ctypes.c_int64(inp.freed_blocks),
+            hostlib.long_array(list(inp.finished)), len(inp.finished), hostlib.long_array(freed),
             self._out, self._cap, self._counts, self._scalars))
         out, cap, n = self._out, self._cap, self._counts
         return Action(prefill=[(out[3 * i], out[3 * i + 1], out[3 * i + 2]) for i in range(n[0] // 3)],

@@ -31,7 +31,9 @@ def parse_config(line: str) -> SchedConfig:
 
 def input_line(inp: SchedInput) -> str:
     arrivals = ",".join(f"{a}:{p}:{m}" for a, p, m in inp.arrivals) if inp.arrivals else "-"
-    return f"IN=A={arrivals}|C={_ints(inp.cancelled)}|F={_ints(inp.finished)}|R={inp.freed_blocks}"
+    # (R: the blocks given back in the first group of layers, the one the reference's single count stands for)
+    freed = inp.freed_blocks[0] if isinstance(inp.freed_blocks, (list, tuple)) else inp.freed_blocks
+    return f"IN=A={arrivals}|C={_ints(inp.cancelled)}|F={_ints(inp.finished)}|R={freed}"
 
 
 def action_line(act: Action) -> str:

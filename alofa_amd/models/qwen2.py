@@ -50,6 +50,14 @@ class Qwen2Config(ModelConfig):
 
     @classmethod
     def from_dict(cls, raw: dict, where: str = "<dict>") -> "Qwen2Config":
+        # keys the reference does not read (qwen.mojo:939-954) but whose other values would change the
+        # model: refused by name rather than computed wrongly
+        if raw.get("rope_scaling") is not None:
+            raise AlofaError("unsupported", "scaled rotary positions are not built", f"key=rope_scaling value={raw['rope_scaling']!r} config={where}")
+        if raw.get("hidden_act", "silu") != "silu":
+            raise AlofaError("unsupported", "the feed-forward's activation is SiLU", f"key=hidden_act value={raw['hidden_act']!r} config={where}")
+        if raw.get("use_mrope", False) not in (False, None):
+            raise AlofaError("unsupported", "multi-axis rotary positions are not built", f"key=use_mrope value={raw['use_mrope']!r} config={where}")
         hidden = _need(raw, "hidden_size", int, where)
         heads = _need(raw, "num_attention_heads", int, where)
         if heads <= 0:

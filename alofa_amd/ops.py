@@ -442,7 +442,7 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     if max_context <= 2 * step:
         return 1
     blocks = tokens * kv_heads * -(-(heads // kv_heads) // 16)
-    by_chip = max(1, 256 // max(1, blocks))
+    by_chip = max(1, compute_units() // max(1, blocks))
     if max_context <= 4 * step:
         return 4 if by_chip >= 4 else 1
     if max_context <= 8 * step and by_chip < 4:
@@ -674,6 +674,7 @@ def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_he
 # ------------------------------------------------------------------ sampling
 
 _argmax_scratch: dict = {}
+_argmax_retired: list = []       # outgrown scratch buffers: a captured step may still address them
 
 
 def _store_operands(store, store_index, n: int):
@@ -700,7 +701,10 @@ def argmax(out: torch.Tensor, logits: torch.Tensor, store: Optional[torch.Tensor
         key = logits.device
         scratch = _argmax_scratch.get(key)
         if scratch is None or scratch.numel() < 2 * 64 * n:
-            scratch = _argmax_scratch[key] = torch.empty(2 * 64 * max(n, 64), dtype=torch.float32, device=logits.device)
+            if scratch is not None:
+                _argmax_retired.append(scratch)
+            # (room for twice the rows asked for: batches that grow one by one do not pile up retired buffers)
+            scratch = _argmax_scratch[key] = torch.empty(2 * 64 * max(2 * n, 64), dtype=torch.float32, device=logits.device)
     if store is None:
         _call("alofa_argmax", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(n), _I(logits.shape[1]), _ptr(scratch), _stream())
     else:
@@ -716,6 +720,7 @@ def can_gemm_argmax(M: int, w: torch.Tensor) -> bool:
 
 
 _gemm_argmax_scratch: dict = {}
+_argmax_retired: list = []       # outgrown scratch buffers: a captured step may still address them
 _gemm_argmax_retired: list = []
 
 

@@ -82,8 +82,10 @@ class GQAAttention(Mixer):
         self.window = p.get("window")
         if self.kv_heads <= 0 or self.heads % self.kv_heads:
             raise AlofaError("unsupported", "kv_heads must be positive and divide heads", f"heads={self.heads} kv_heads={self.kv_heads}")
-        if self.d % 16 or not 16 <= self.d <= ops.MAX_HEAD_DIM:
-            raise AlofaError("unsupported", f"the attention kernels take head sizes 16..{ops.MAX_HEAD_DIM} in steps of 16", f"head_dim={self.d}")
+        if self.d % 2 or not 2 <= self.d <= ops.MAX_HEAD_DIM:
+            raise AlofaError("unsupported", f"the attention kernels take even head sizes up to {ops.MAX_HEAD_DIM}", f"head_dim={self.d}")
+        # (the matrix-core kernels take head sizes in steps of 16; any other even size runs on the always-valid kernels, in both dtypes)
+        self.mfma_heads = self.d % 16 == 0
         if self.window is not None and self.window <= 0:
             raise AlofaError("invalid_argument", "an attention window must be positive", f"window={self.window}")
         pre = p["prefix"]
@@ -133,7 +135,7 @@ class GQAAttention(Mixer):
         pow2_pages = kv.k.shape[2] >= ops.MIN_FAST_PAGE and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
         fast_prefill = self.d in ops.PREFILL_HEAD_DIMS
         # one new token per request: the decode kernel rotates it and writes its cache slot itself
-        fused = (not exact and pow2_pages and kv.owner and ctx.max_q_len == 1 and plan.long_runs is None
+        fused = (not exact and pow2_pages and self.mfma_heads and kv.owner and ctx.max_q_len == 1 and plan.long_runs is None
                  and ops.can_fuse_rope_into_decode(self.d))
         if fused:
             pass
@@ -141,7 +143,7 @@ class GQAAttention(Mixer):
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d, kv.slots, kv.k, kv.v)
         else:
             ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
-        if exact or not pow2_pages or (plan.long_runs is not None and not fast_prefill):
+        if exact or not pow2_pages or not self.mfma_heads or (plan.long_runs is not None and not fast_prefill):
             # the exact path, and page or head sizes the bfloat16 kernels are not built for
             ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
         else:

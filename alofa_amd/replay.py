@@ -2,7 +2,7 @@
 logits; it samples nothing. It drives the engine's own model, step function,
 cache and kernels — the ones generation uses.
 
-    bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+    bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--blocks N] [--window-blocks N]
 
 Steps come on standard input, one JSON object a line:
 
@@ -10,7 +10,14 @@ Steps come on standard input, one JSON object a line:
 
 For a step in which something is wanted, ``DIR/<step>.f32`` receives the logits
 at the wanted places ([wanted, vocab] little-endian float32, in the order of the
-entries and of ``want``). After every step a line ``done <step>`` is printed.
+entries and of ``want``), and ``DIR/<step>.tsv`` one line ``request<TAB>position``
+per row of them (the position counts from the request's first token), so that
+outputs of different cuttings can be compared position by position without the
+input. After every step a line ``done <step>`` is printed.
+
+The cache pool is made for ``--max-tokens`` tokens, or, with ``--blocks``, of so
+many pages; ``--window-blocks`` gives the pools of layers that see only a window
+of keys a size of their own.
 
 A request's first entry may start on pages another live request has filled:
 
@@ -31,6 +38,7 @@ import argparse
 import json
 import sys
 from pathlib import Path
+from typing import Optional
 
 from .errors import AlofaError
 
@@ -38,7 +46,10 @@ from .errors import AlofaError
 class Replayer:
     """The replay loop as an object: one ``step`` per input line."""
 
-    def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device: str = "cuda:0"):
+    def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device: str = "cuda:0",
+                 blocks: Optional[int] = None, window_blocks: Optional[int] = None):
+        """``blocks``: pages of every pool (default: what ``max_tokens`` tokens take); ``window_blocks``: pages of
+        the pools of groups of layers that see a window only, when they are to differ."""
         from .csrc.build import load
         load()  # compile at the first call if nothing is built; fail loudly if it cannot
         from .cache.manager import CacheManager
@@ -46,14 +57,18 @@ class Replayer:
         from .model import load_model
 
         self.config, self.model = load_model(model_dir, dtype, device)
-        n_blocks = max(1, (int(max_tokens) + block_size - 1) // block_size)
-        self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), n_blocks, block_size,
+        n_blocks = int(blocks) if blocks is not None else max(1, (int(max_tokens) + block_size - 1) // block_size)
+        needs = self.model.cache_needs()
+        if window_blocks is not None:
+            n_blocks = {w: n_blocks if w is None else int(window_blocks) for w in CacheManager.windows_of(needs)}
+        self.cache = CacheManager(needs, self.model.state_needs(), n_blocks, block_size,
                                   max_requests=8, device=self.model.rt.device, dtype=self.model.rt.dtype)
         # the position table is as long as a request can get here, not the checkpoint's
         # max_position_embeddings, which the reference does not read (qwen.mojo:849)
         self.fn = StepFunction(self.model, self.cache, n_positions=max(int(max_tokens), 64))
         self.tokens: dict = {}       # request -> the tokens it has been given so far
         self.shared: dict = {}       # request -> tokens it took over from another request's pages
+        self.last_index: list = []   # (request, position) of every row of the last step's logits
 
     def step(self, rec: dict):
         """Run one step record; returns float32 logits [wanted, vocab] as a NumPy
@@ -75,6 +90,7 @@ class Replayer:
                 self.tokens[e["id"]] = []
             entries.append(StepEntry(e["id"], tokens, want))
         out = None
+        self.last_index = [(e.request, len(self.tokens[e.request]) + w) for e in entries for w in e.want]
         if entries:
             logits = self.fn.run(entries)
             for e in entries:
@@ -113,10 +129,12 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each request rounded up to a multiple of 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--blocks", type=int, default=None, help="pages of the cache pool, instead of what --max-tokens tokens take")
+    ap.add_argument("--window-blocks", type=int, default=None, help="pages of the pools of layers that see a window only (default: as the others)")
     args = ap.parse_args(argv)
     out = Path(args.out)
     out.mkdir(parents=True, exist_ok=True)
-    replayer = Replayer(args.model, args.dtype, args.max_tokens, args.block_size)
+    replayer = Replayer(args.model, args.dtype, args.max_tokens, args.block_size, blocks=args.blocks, window_blocks=args.window_blocks)
     for line in sys.stdin:
         line = line.strip()
         if not line:
@@ -125,6 +143,7 @@ def main(argv=None) -> int:
         logits = replayer.step(rec)
         if logits is not None:
             logits.tofile(out / f"{rec['step']}.f32")
+            (out / f"{rec['step']}.tsv").write_text("".join(f"{r}\t{p}\n" for r, p in replayer.last_index))
         print(f"done {rec['step']}", flush=True)
     return 0
 

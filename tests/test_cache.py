@@ -141,6 +141,66 @@ def test_random_orders_keep_the_invariants(seed):
     assert all(g.pool.n_free == g.pool.n_blocks for g in m.groups) and len(m.free_slots) == 4
 
 
+def test_every_group_has_a_pool_of_its_own_size():
+    """A group whose layers see a window only is given what its window needs, whatever the group that keeps
+    every key has: with the window's pool at its bound (requests x (window + step + two pages)) no step of
+    at most that many tokens is ever refused for it, under random orders of requests."""
+    bs, window, step, live_max = 8, 24, 16, 3
+    needs = [CacheNeed.keys_and_values(2, 16, w) for w in (None, window, window, None)]
+    assert CacheManager.windows_of(needs) == [None, window]
+    assert CacheManager.held_tokens_of(None, step, bs) == -1 and CacheManager.held_tokens_of(window, step, bs) == window + step + 2 * bs
+    at_bound = CacheManager.pages_for(window, live_max, 10_000, step, bs)
+    assert at_bound == live_max * blocks_for(window + step + 2 * bs, bs) == 21
+    assert CacheManager.pages_for(window, 2, 10, step, bs) == 4 and CacheManager.pages_for(None, 2, 100, step, bs) == 26    # short requests hold their length
+    m = CacheManager(needs, [None] * 4, {None: 200, window: at_bound}, bs, max_requests=4)
+    assert [g.pool.n_blocks for g in m.groups] == [200, at_bound] and m.group_rules(step) == [(200, -1), (at_bound, window + step + 2 * bs)]
+    assert err_name(CacheManager, needs, [None] * 4, {None: 200}, bs) == "invalid_argument"          # a group without a count
+    assert err_name(CacheManager, needs, [None] * 4, {None: 200, window: 0}, bs) == "invalid_argument"
+    rnd = random.Random(5)
+    live, names, peak = {}, iter(range(10_000)), 0
+    for _ in range(600):
+        op = rnd.random()
+        if op < 0.2 and len(live) < live_max:
+            r = next(names)
+            m.admit(r)
+            live[r] = 0
+        elif op < 0.9 and live:
+            r = rnd.choice(list(live))
+            if live[r] > 400:
+                continue
+            target = live[r] + rnd.randint(1, step)
+            m.reserve(r, target)                                  # never refused: the full group is large, the window's at its bound
+            peak = max(peak, m.groups[1].pool.used)
+            m.commit(r, target)
+            live[r] = target
+        elif live:
+            r = rnd.choice(list(live))
+            m.free(r)
+            del live[r]
+        m.check()
+    assert live_max * blocks_for(window, bs) < peak <= at_bound  # more than the bare windows were held at some time, never more than the bound
+
+
+def test_a_step_that_cannot_be_laid_out_changes_nothing():
+    """Every refusal of ``plan_step`` comes before the first page is taken: too few pages, a table wider than
+    the caller's buffer, a request beyond the context bound."""
+    import numpy as np
+    m = manager(n_blocks=6, windows=(None,))
+    m.admit("a"), m.admit("b")
+    slots, n_tokens = np.array([0, 1], dtype=np.int32), np.array([20, 9], dtype=np.int32)
+    before = m.groups[0].pool.n_free
+    assert err_name(m.plan_step, slots, n_tokens, 64, 2) == "capacity"                                   # the first entry needs three blocks of table
+    assert m.groups[0].pool.n_free == before and m.table("a", 0) == [] and m.table("b", 0) == []
+    assert err_name(m.plan_step, slots, np.array([20, 40], dtype=np.int32), 64) == "capacity"            # eight pages of six
+    assert err_name(m.plan_step, slots, n_tokens, 19) == "capacity"                                      # past the context bound
+    assert m.groups[0].pool.n_free == before and m.length("a") == 0
+    m.check()
+    pos0, positions, req_of_token, tables, row_slots = m.plan_step(slots, n_tokens, 64)
+    assert pos0.tolist() == [0, 0] and tables.shape == (1, 2, 3) and tables[0].tolist() == [[0, 1, 2], [3, 4, -1]]
+    m.commit_step(slots, n_tokens)
+    m.check()
+
+
 def test_state_slots_without_a_device_are_counted_only():
     m = manager(state=True)
     s = m.admit("a")

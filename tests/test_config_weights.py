@@ -59,6 +59,12 @@ def test_config_errors_are_named():
     assert err_name(config_from_dict, broken(architectures=None)) == "invalid_argument"
     assert err_name(config_from_dict, broken(hidden_size=12, num_attention_heads=4, head_dim=3)) == "unsupported"   # odd head
     assert err_name(config_from_dict, broken(use_sliding_window=True)) == "invalid_argument"   # window asked, none given
+    # keys whose other values would change the model are refused by name, not ignored
+    for key, value in (("rope_scaling", {"type": "yarn", "factor": 4.0}), ("hidden_act", "gelu"), ("use_mrope", True)):
+        with pytest.raises(AlofaError) as e:
+            config_from_dict(broken(**{key: value}))
+        assert e.value.name == "unsupported" and key in str(e.value)
+    config_from_dict(dict(TINY["A"], rope_scaling=None, hidden_act="silu", use_mrope=False))          # the values the engine computes
 
 
 def test_config_file_errors(tmp_path):

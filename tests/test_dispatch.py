@@ -39,7 +39,8 @@ def test_product_kernel_by_shape():
         ops._product_entry("fast", 4, 64, 64)
 
 
-def test_decode_splits_follow_the_context():
+def test_decode_splits_follow_the_context(monkeypatch):
+    monkeypatch.setattr(ops, "_compute_units", 256)                                # the rule counts the chip's compute units: an MI355X's here
     assert ops.decode_splits(8, 14, 2, 64, 512) == 1                              # the waves of one block cover two steps each
     assert ops.decode_splits(8, 14, 2, 64, 1024) == 4 and ops.decode_splits(32, 14, 2, 64, 1024) == 4 and ops.decode_splits(64, 14, 2, 64, 1024) == 1    # four parts up to four steps, with room for four
     assert ops.decode_splits(8, 14, 2, 64, 2048) == 8                             # a part per step of all the waves
@@ -48,6 +49,8 @@ def test_decode_splits_follow_the_context():
     assert ops.decode_splits(64, 14, 2, 64, 2048) == 1 and ops.decode_splits(64, 14, 2, 64, 4096) == 2 and ops.decode_splits(32, 14, 2, 64, 2048) == 4    # many blocks already: fewer parts
     assert ops.decode_splits(8, 28, 4, 128, 256) == 1 and ops.decode_splits(8, 28, 4, 128, 512) == 4 and ops.decode_splits(8, 28, 4, 128, 4096) == 8
     assert ops.decode_splits(32, 28, 4, 128, 512) == 1 and ops.decode_splits(32, 28, 4, 128, 1024) == 1 and ops.decode_splits(32, 28, 4, 128, 2048) == 2 and ops.decode_splits(64, 28, 4, 128, 4096) == 1
+    monkeypatch.setattr(ops, "_compute_units", 64)                                 # a smaller chip is full sooner
+    assert ops.decode_splits(8, 14, 2, 64, 1024) == 4 and ops.decode_splits(8, 14, 2, 64, 1 << 16) == 4 and ops.decode_splits(32, 14, 2, 64, 1 << 16) == 1
     assert ops.HAND_OVER_MAX_PARTS == 8
     assert ops.decode_waves(64) == 8 and ops.decode_waves(128) == 4 and ops.decode_waves(256) == 4
 

@@ -176,6 +176,56 @@ def test_long_context(tiny_dirs, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_context_of_8200_tokens(tiny_dirs, dtype):
+    """One request of 8,200 tokens, the contexts at which decoding is timed: the bulk in portions of 2,048
+    (prompt portions that start deep in the context), the last 40 tokens one by one (decode attention over
+    more than 500 pages, its keys shared out among parts that a second kernel merges); the logits of the
+    last 104 positions against the plain model (token by token against the whole prompt:
+    tests/unit/test_model_parity.mojo:181-217 of the reference)."""
+    from alofa_amd.replay import Replayer
+    n, tail, wanted = 8200, 40, 104
+    ids = random_ids(41, n, TINY["B"]["vocab_size"])
+    ref = plain_logits(tiny_dirs["B"], tuple(ids))[n - wanted:]
+    r = Replayer(tiny_dirs["B"], dtype, round64(n))
+    steps, pos = [], 0
+    while pos < n - tail:
+        m = min(2048, n - tail - pos)
+        steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": ids[pos:pos + m],
+                                                       "want": [w for w in range(m) if pos + w >= n - wanted]}], "end": []})
+        pos += m
+    for i in range(n - tail, n):
+        steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": [ids[i]], "want": [0]}], "end": ["a"] if i == n - 1 else []})
+    got = collect(r, steps)["a"]
+    assert got.shape[0] == wanted
+    assert_close(got, ref, dtype, "8,200 tokens")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("head_dim,heads,kv_heads", [(8, 4, 2), (24, 3, 1)])
+def test_heads_of_any_even_size(tmp_path, dtype, head_dim, heads, kv_heads):
+    """Head sizes that are no multiple of 16 (the reference's own paged fixture has heads of 8): the
+    always-valid kernels take any even size in both dtypes, through every cutting."""
+    from alofa_amd.replay import Replayer
+    from alofa_amd.weights import write_random_model
+    cfg = dict(TINY["A"], hidden_size=heads * head_dim, num_attention_heads=heads, num_key_value_heads=kv_heads,
+               intermediate_size=88, vocab_size=203, max_position_embeddings=256)
+    write_random_model(cfg, tmp_path, seed=head_dim)
+    ids = random_ids(51, 120, cfg["vocab_size"])
+    ref = plain_logits(tmp_path, tuple(ids))
+    r = Replayer(tmp_path, dtype, 256)
+    assert_close(collect(r, whole("w", ids))["w"], ref, dtype, f"d={head_dim} whole")
+    assert_close(collect(r, bulk_and_tail("t", ids))["t"], ref, dtype, f"d={head_dim} bulk+tail")
+    assert_close(collect(r, portions("p", ids))["p"], ref, dtype, f"d={head_dim} portions")
+    requests = {f"r{i}": random_ids(400 + i, n, cfg["vocab_size"]) for i, n in enumerate([120, 41, 90, 64, 35])}
+    steps, peak = mixed(requests, seed=3)
+    r = Replayer(tmp_path, dtype, peak)
+    got = collect(r, steps)
+    r.cache.check()
+    for k, v in requests.items():
+        assert_close(got[k], plain_logits(tmp_path, tuple(v)), dtype, f"d={head_dim} mixed {k}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_first_tokens_of_a_sequence(replayers, tiny_dirs, name, dtype):
     ids = ids_of(name, seed=9, n=5)
@@ -450,15 +500,22 @@ def test_trace_run_program(tiny_dirs, tmp_path):
     text = "".join(json.dumps(s) + "\n" for s in steps)
     env = dict(os.environ, HOME=str(tmp_path / "home"))
     p = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(tiny_dirs["B"]), "--dtype", "float32",
-                        "--out", str(tmp_path / "out"), "--max-tokens", "128"], input=text, capture_output=True, text=True, env=env, timeout=300)
+                        "--out", str(tmp_path / "out"), "--max-tokens", "128", "--blocks", "6"], input=text, capture_output=True, text=True, env=env, timeout=300)
     assert p.returncode == 0, p.stderr[-2000:]
     assert p.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
     ref = plain_logits(tiny_dirs["B"], tuple(ids))
     first = np.fromfile(tmp_path / "out" / "0.f32", dtype="<f4").reshape(-1, TINY["B"]["vocab_size"])
     assert_close(first, ref[:58], "float32", "program, first step")
-    assert not (tmp_path / "out" / "3.f32").exists()
+    # beside the floats, which (request, position) every row belongs to
+    assert (tmp_path / "out" / "0.tsv").read_text() == "".join(f"a\t{p}\n" for p in range(58))
+    assert not (tmp_path / "out" / "3.f32").exists() and not (tmp_path / "out" / "3.tsv").exists()
     last = np.fromfile(tmp_path / "out" / f"{steps[-1]['step']}.f32", dtype="<f4").reshape(1, -1)
     assert_close(last, ref[-1:], "float32", "program, last step")
+    assert (tmp_path / "out" / f"{steps[-1]['step']}.tsv").read_text() == "a\t89\n"
+    # --blocks sizes the pool instead of --max-tokens: five pages of 16 do not hold 90 tokens
+    few = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(tiny_dirs["B"]), "--dtype", "float32",
+                          "--out", str(tmp_path / "o3"), "--max-tokens", "128", "--blocks", "5"], input=text, capture_output=True, text=True, env=env, timeout=300)
+    assert few.returncode != 0 and "exhausted" in few.stderr
     # unknown dtype and a missing model are refused, not worked around
     bad = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(tmp_path / "none"), "--dtype", "float32",
                           "--out", str(tmp_path / "o2"), "--max-tokens", "64"], input="", capture_output=True, text=True, timeout=300)

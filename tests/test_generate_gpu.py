@@ -5,6 +5,7 @@ import subprocess
 
 import numpy as np
 import pytest
+import torch
 
 from conftest import ROOT, TINY
 from helpers import plain_model, random_ids
@@ -74,8 +75,8 @@ def test_tiny_b_mixed_batch_greedy_and_sampled(tiny_dirs, tmp_path):
 def test_pages_run_out_preemption_recomputes(tiny_dirs):
     """With so few pages that running requests are preempted, every request
     still gets exactly the tokens it gets alone."""
+    import dataclasses
     from alofa_amd import Engine
-    from alofa_amd.engine.scheduler import SchedConfig
     prompts = [random_ids(30 + i, n, 331) for i, n in enumerate((30, 45, 20, 38))]
     alone = [Engine(tiny_dirs["C"], dtype="float32", max_tokens=128).generate([p], max_new=40)[0] for p in prompts]
     eng = Engine(tiny_dirs["C"], dtype="float32", max_tokens=128, kv_blocks=20, watermark_permille=1000, max_chunk=32, token_budget=64)
@@ -85,12 +86,13 @@ def test_pages_run_out_preemption_recomputes(tiny_dirs):
     while not all(len(r.out) >= 3 for r in core.requests.values()):
         core.tick()
     # pages run short while all four decode: the watermark drops for one tick
-    core.sched.cfg = SchedConfig(64, 32, 16, 20, 400, 8, 32)
+    assert eng.sched_cfg.groups[0] == (20, -1) and len(eng.sched_cfg.groups) == 2
+    core.sched.cfg = dataclasses.replace(eng.sched_cfg, watermark_permille=400)
     core.tick()
     victims = list(core.last_action.preempted)
     assert victims and core.sched.preempt_total == len(victims)
     assert all(not eng.cache.has(v) and core.requests[v].out == [] and core.requests[v].fed == 0 for v in victims)
-    core.sched.cfg = SchedConfig(64, 32, 16, 20, 1000, 8, 32)
+    core.sched.cfg = eng.sched_cfg
     core.run(max_ticks=2000)
     outs = [eng.core.output(i + 1) for i in range(4)]
     assert outs == alone
@@ -100,7 +102,9 @@ def test_pages_run_out_preemption_recomputes(tiny_dirs):
 
 def held_nothing(eng):
     s = eng.core.sched
-    assert s.blocks_used == 0 and s.cached_blocks == 0 and s.n_live() == 0
+    assert s.n_live() == 0
+    for g in range(len(s.cfg.groups)):
+        assert s.of_group("blocks_used", g) == 0 and s.of_group("cached_blocks", g) == 0
     eng.cache.check()
     assert not eng.cache.requests and all(g.pool.n_free == g.pool.n_blocks for g in eng.cache.groups)
 
@@ -299,7 +303,8 @@ def test_a_model_of_windows_only_is_admitted_by_what_it_holds(tmp_path):
     prompts = [random_ids(300 + i, 170 + 10 * i, cfg["vocab_size"]) for i in range(4)]
     want = [plain_greedy(d, p, 24) for p in prompts]
     eng = Engine(d, dtype="float32", max_tokens=256, max_batch=4, kv_blocks=40, block_size=16, max_chunk=32, token_budget=64)
-    assert eng.sched_cfg.held_tokens == 40 + 32 + 2 * 16 and [g.window for g in eng.cache.groups] == [40]
+    # (of the 40 pages offered the pool takes what four such requests can hold under the watermark: 4 x 7 / 0.9 + 1)
+    assert eng.sched_cfg.groups == ((33, 40 + 32 + 2 * 16),) and [g.window for g in eng.cache.groups] == [40]
     core = eng.core
     for i, p in enumerate(prompts):
         core.submit(i + 1, p, 24)
@@ -314,6 +319,72 @@ def test_a_model_of_windows_only_is_admitted_by_what_it_holds(tmp_path):
         core.release(i + 1)
     core.run(10)
     held_nothing(eng)
+
+
+def test_windowed_layers_get_a_pool_of_their_own_size(tiny_dirs):
+    """Configuration C: one layer keeps every key, three see the last 40 only. The windowed group's pool holds what
+    its window needs of every request (window + a step's tokens + two pages), not what whole requests would take, so
+    the cache takes far less memory; the scheduler counts both groups; five requests of up to 250 tokens run through
+    it with the tokens each gives alone."""
+    from alofa_amd import Engine
+    from alofa_amd.cache.manager import blocks_for
+    name, bs, chunk, batch, context = "C", 16, 32, 4, 256
+    eng = Engine(tiny_dirs[name], dtype="float32", max_tokens=context, max_batch=batch, block_size=bs, max_chunk=chunk, token_budget=64)
+    full, windowed = eng.cache.groups
+    assert (full.window, windowed.window) == (None, 40) and len(full.entries) == 1 and len(windowed.entries) == 3
+    per_request = blocks_for(40 + chunk + 2 * bs, bs)
+    assert full.pool.n_blocks >= batch * context // bs and batch * per_request <= windowed.pool.n_blocks <= batch * per_request * 1000 // 900 + 2
+    assert eng.sched_cfg.groups == ((full.pool.n_blocks, -1), (windowed.pool.n_blocks, 40 + chunk + 2 * bs))
+    # every owner's tensors have its group's pages: the three windowed layers take their share less
+    pages = {owner: t["k"].shape[0] for owner, t in eng.cache.tensors.items()}
+    assert sorted(pages.values()) == [windowed.pool.n_blocks] * 3 + [full.pool.n_blocks]
+    one_size = Engine(tiny_dirs[name], dtype="float32", max_tokens=context, max_batch=batch, block_size=bs, max_chunk=chunk, token_budget=64,
+                      kv_blocks={None: full.pool.n_blocks, 40: full.pool.n_blocks})
+    saved = one_size.memory()["cache_pool"] - eng.memory()["cache_pool"]
+    assert saved == 3 * (full.pool.n_blocks - windowed.pool.n_blocks) * eng.cache.tensors[(1, 0)]["k"][0].numel() * 2 * 4 > 0.4 * one_size.memory()["cache_pool"]
+    del one_size
+    prompts = [random_ids(500 + i, n, TINY[name]["vocab_size"]) for i, n in enumerate((230, 190, 60, 215, 120))]
+    want = [plain_greedy(tiny_dirs[name], p, 20) for p in prompts]
+    core = eng.core
+    waiting = list(enumerate(prompts))
+    while waiting or core.has_work():
+        while waiting and core.can_admit(len(waiting[0][1]), 20):
+            i, p = waiting.pop(0)
+            core.submit(i + 1, p, 20)
+        core.tick()
+        assert core.last_action.preempted == []
+        for g, group in enumerate(eng.cache.groups):       # what the scheduler counts covers what the pool really holds
+            assert group.pool.used <= core.sched.of_group("blocks_used", g) <= group.pool.n_blocks
+    core.flush()
+    assert [core.output(i + 1) for i in range(5)] == want
+    assert windowed.pool.high_water > batch * blocks_for(40, bs) - batch          # the windowed pool was really used up to about its bound
+    for i in range(5):
+        core.release(i + 1)
+    core.run(10)
+    held_nothing(eng)
+
+
+def test_a_request_that_ends_exactly_at_the_context_bound(tiny_dirs):
+    """prompt + max_new == max_tokens, and max_tokens == max_position_embeddings: the last token is chosen from
+    the last position the tables hold; one more token is refused by name."""
+    from alofa_amd import Engine
+    from alofa_amd.errors import AlofaError
+    bound = TINY["A"]["max_position_embeddings"]                      # 128
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine(tiny_dirs["A"], dtype=dtype, max_tokens=bound, max_batch=2)
+        assert eng.step_fn.n_positions == bound
+        prompts = [random_ids(600, bound - 12, 256), random_ids(601, 5, 256)]
+        got = eng.generate(prompts[:1], max_new=12) + eng.generate(prompts[1:], max_new=bound - 5)
+        want = [plain_greedy(tiny_dirs["A"], prompts[0], 12), plain_greedy(tiny_dirs["A"], prompts[1], bound - 5)]
+        assert [len(g) for g in got] == [12, bound - 5]
+        assert got == want if dtype == "float32" else agreement(got, want) >= 0.8
+        with pytest.raises(AlofaError) as e:
+            eng.generate(prompts[:1], max_new=13)
+        assert e.value.name == "out_of_range"
+        held_nothing(eng)
+    with pytest.raises(AlofaError) as e:
+        Engine(tiny_dirs["A"], dtype="float32", max_tokens=bound + 1)
+    assert e.value.name == "out_of_range" and "max_position_embeddings" in str(e.value)
 
 
 def test_greedy_choice_inside_the_step_changes_no_token(tmp_path, monkeypatch):
@@ -350,6 +421,43 @@ def test_greedy_choice_inside_the_step_changes_no_token(tmp_path, monkeypatch):
     before = len(calls)
     mixed.core.run()
     assert mixed.core.output(1) == by_step[0] and len(mixed.core.output(2)) == 20 and len(calls) == before
+
+
+def test_batches_that_grow_past_64_rows_and_shrink_again_replay_their_graphs(tmp_path, monkeypatch):
+    """A vocabulary of 9,001 (searched by the two-stage argmax through a scratch buffer that is kept between
+    calls; too short for the product that takes the argmax with it) and batches that rise from 60 to 70 rows
+    one request at a time, then fall as requests end: every batch size captures a graph that addresses the
+    scratch buffer of its day, and the graphs of the smaller batches are replayed after the buffer was
+    outgrown. Token for token what steps run kernel by kernel give."""
+    from alofa_amd import Engine, ops
+    from alofa_amd.weights import write_random_model
+    cfg = dict(TINY["A"], vocab_size=9001)
+    d = tmp_path / "vocabulary_9001"
+    write_random_model(cfg, d, seed=93)
+    prompts = [random_ids(700 + i, 3 + i % 5, cfg["vocab_size"]) for i in range(70)]
+
+    def play():
+        eng = Engine(d, dtype="bfloat16", max_tokens=64, max_batch=72, token_budget=256)
+        core, sizes = eng.core, set()
+        for i in range(60):
+            core.submit(i + 1, prompts[i], 30 + i % 7)
+        n = 60
+        while core.has_work():
+            core.tick()
+            if core.last_action.decode and not core.last_action.prefill:
+                sizes.add(len(core.last_action.decode))
+            if n < 70 and core.ticks % 2 == 0:
+                core.submit(n + 1, prompts[n], 12 + n % 5)
+                n += 1
+        core.flush()
+        return [core.output(i + 1) for i in range(70)], sizes, eng.step_fn.graph_replays
+
+    assert not ops.can_gemm_argmax(70, torch.empty(9001, 64, dtype=torch.bfloat16))
+    captured, sizes, replays = play()
+    assert max(sizes) > 64 and min(sizes) < 60 and len(sizes) > 12 and replays > 20
+    monkeypatch.setenv("ALOFA_GRAPHS", "0")
+    eager, sizes_eager, none = play()
+    assert none == 0 and sizes_eager == sizes and eager == captured
 
 
 def test_cancel_and_request_verbs(tiny_dirs):

@@ -562,6 +562,161 @@ def test_decode_attention_with_many_splits(heads, kv_heads, d):
     assert err <= 1e-2 * np.abs(ref).max(), f"{err} vs {np.abs(ref).max()}"
 
 
+def long_case(rng, lens, q_lens, heads, kv_heads, d, bs, peak=1.2, holes=None, far=None):
+    """Requests over long contexts, built without a loop per position: request r sees the first ``lens[r]`` of one
+    shared run of random keys and values, laid out on pages of its own in shuffled order; its queries are the last
+    ``q_lens[r]`` positions. Every last query leans towards one key near the start of its context (3 + 5 r): with
+    ``peak`` 1.2 that key carries about a fifth of the weight among tens of thousands, so both a dropped far key
+    and a wrong sum over the many show at the result's own scale (``far[r]``: another place for it). ``holes[r]``: so many leading pages are missing
+    from the table (-1), as behind a window that has passed them. Pages in no table hold NaN."""
+    L = max(lens)
+    k = bf(rng.standard_normal((L, kv_heads * d)).astype(np.float32))
+    v = bf(rng.standard_normal((L, kv_heads * d)).astype(np.float32))
+    per = [(n + bs - 1) // bs for n in lens]
+    n_blocks = sum(per) + 3
+    order = rng.permutation(n_blocks)
+    kc = torch.full((n_blocks, kv_heads, bs, d), float("nan"), dtype=torch.bfloat16)
+    vc = torch.full((n_blocks, kv_heads, bs, d), float("nan"), dtype=torch.bfloat16)
+    k_t, v_t = torch.from_numpy(k).to(torch.bfloat16).view(L, kv_heads, d), torch.from_numpy(v).to(torch.bfloat16).view(L, kv_heads, d)
+    table = np.full((len(lens), max(per)), -1, np.int32)
+    qs, pos, req, used = [], [], [], 0
+    for r, n in enumerate(lens):
+        table[r, :per[r]] = order[used:used + per[r]]
+        used += per[r]
+        at = np.arange(n)
+        first = (holes[r] if holes else 0) * bs
+        pages, places = torch.from_numpy(table[r, at[first:] // bs].astype(np.int64)), torch.from_numpy(at[first:] % bs)
+        kc[pages, :, places] = k_t[first:n]
+        vc[pages, :, places] = v_t[first:n]
+        if holes:
+            table[r, :holes[r]] = -1
+        q = bf(rng.standard_normal((q_lens[r], heads * d)).astype(np.float32))
+        j = far[r] if far else 3 + 5 * r
+        for h in range(heads):
+            hk = h // (heads // kv_heads)
+            q[-1, h * d:(h + 1) * d] = bf(peak * k[j, hk * d:(hk + 1) * d])
+        qs.append(q)
+        pos.extend(range(n - q_lens[r], n))
+        req.extend([r] * q_lens[r])
+    return dict(k=k, v=v, q=qs, kc=kc.to(DEV), vc=vc.transpose(2, 3).contiguous().to(DEV), table=t(table, torch.int32),
+                pos=t(np.array(pos, np.int32), torch.int32), req=t(np.array(req, np.int32), torch.int32),
+                qcat=t(np.concatenate(qs), torch.bfloat16), lens=lens)
+
+
+def long_reference(c, r, heads, kv_heads, d, window=None, rows=None):
+    """The plain attention of request r's queries (the last ``rows`` of them) over its context."""
+    n = c["lens"][r]
+    q = c["q"][r] if rows is None else c["q"][r][-rows:]
+    return pm.attention(q, c["k"][:n], c["v"][:n], heads, kv_heads, d, window)
+
+
+def close_at_own_scale(got, ref, what):
+    """Attention over tens of thousands of random keys is small: compared at the result's own scale, within the
+    eight bits of a bfloat16 output and weights."""
+    got = got.detach().float().cpu().numpy() if isinstance(got, torch.Tensor) else got
+    err, scale = np.abs(got.astype(np.float64) - ref).max(), np.abs(ref).max()
+    assert np.isfinite(got).all() and err <= 1.5e-2 * scale, f"{what}: {err:.3e} > 1.5e-2 x {scale:.3e}"
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+@pytest.mark.parametrize("context", [8192, 16384, 32768])
+@pytest.mark.parametrize("heads,kv_heads,d", [(14, 2, 64), (28, 4, 128)])
+def test_decode_attention_at_the_contexts_that_are_timed(heads, kv_heads, d, context, batch):
+    """One token per request over 8,192 to 32,768 real keys (every part of the context holds data, and a far key
+    carries weight): the parts the launch rule picks at that context, merged by the second kernel or handed over to
+    the last block, eight parts handed over, and the form that rotates and writes the new token itself."""
+    rng = np.random.default_rng(61)
+    o = ops()
+    lens = [context - 37 * r for r in range(batch)]
+    c = long_case(rng, lens, [1] * batch, heads, kv_heads, d, 16)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    ref = np.concatenate([long_reference(c, r, heads, kv_heads, d) for r in range(batch)])
+    assert np.abs(ref).max() > 0.15                                     # the far key counts
+    picked = o.decode_splits(batch, heads, kv_heads, d, context)
+    assert picked >= 8
+    out = torch.zeros(batch, heads * d, device=DEV, dtype=torch.bfloat16)
+    scratch = torch.empty(max(1, o.decode_scratch_floats(batch, heads, kv_heads, d, context, None)), device=DEV)
+    o.paged_attention(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, None, scale, False,
+                      max_q_len=1, max_context=context, scratch=scratch)
+    close_at_own_scale(out, ref, f"{picked} parts, as the rule picks")
+    big = torch.empty(batch * heads * 64 * (d + 2), device=DEV)
+    can_hand_over = o.decode_hand_over(batch, heads, kv_heads, d, 8)
+    assert can_hand_over or batch > 1
+    for parts, hand_over in ((picked, False), (8, True), (8, False), (64 if batch == 1 else 32, False)):
+        if hand_over and not can_hand_over:
+            continue
+        out.zero_()
+        o.attention_decode(out, c["qcat"], c["kc"], c["vc"], c["table"], c["req"], c["pos"], heads, kv_heads, d, None, scale, context, big,
+                           n_splits=parts, hand_over=hand_over)
+        close_at_own_scale(out, ref, f"{parts} parts, hand-over {hand_over}")
+    # the new token arrives as the fused projection's row, not yet rotated; its slot holds NaN before
+    cos, sin = pm.rope_table(context, d, 1e6)
+    qkv = np.zeros((batch, (heads + 2 * kv_heads) * d), np.float32)
+    slots, table = [], c["table"].cpu().numpy()
+    kc, vc = c["kc"].clone(), c["vc"].clone()
+    refs = []
+    for r, n in enumerate(lens):
+        q_raw, k_raw = c["q"][r], bf(rng.standard_normal((1, kv_heads * d)).astype(np.float32))
+        at = np.array([n - 1])
+        q_rot, k_rot = bf(pm.rope_apply(q_raw, cos, sin, at, d)), bf(pm.rope_apply(k_raw, cos, sin, at, d))
+        k = c["k"][:n].copy()
+        k[n - 1] = k_rot[0]
+        qkv[r] = np.concatenate([q_raw[0], k_raw[0], c["v"][n - 1]])
+        slot = int(table[r, (n - 1) // 16]) * 16 + (n - 1) % 16
+        slots.append(slot)
+        kc[slot // 16, :, slot % 16] = float("nan")
+        vc[slot // 16, :, :, slot % 16] = float("nan")
+        refs.append(pm.attention(q_rot, k, c["v"][:n], heads, kv_heads, d))
+    rope = (t(cos[:, :d // 2]), t(sin[:, :d // 2]), t(np.array(slots, np.int64), torch.int64))
+    for parts, hand_over in ((picked, False), (8, True)):
+        if hand_over and not can_hand_over:
+            continue
+        kc2, vc2 = kc.clone(), vc.clone()
+        out.zero_()
+        o.attention_decode(out, t(qkv, torch.bfloat16), kc2, vc2, c["table"], None, c["pos"], heads, kv_heads, d, None, scale, context, big,
+                           rope=rope, n_splits=parts, hand_over=hand_over)
+        close_at_own_scale(out, np.concatenate(refs), f"rotating form, {parts} parts, hand-over {hand_over}")
+        for slot in slots:
+            assert torch.isfinite(kc2[slot // 16, :, slot % 16].float()).all() and torch.isfinite(vc2[slot // 16, :, :, slot % 16].float()).all()
+
+
+@pytest.mark.parametrize("heads,kv_heads,d,shares", [(14, 2, 64, (0, 7)), (40, 8, 128, (0,)), (16, 2, 64, (0, 8))])
+@pytest.mark.parametrize("window", [None, 3000])
+def test_prefill_attention_of_portions_deep_in_a_context(heads, kv_heads, d, shares, window):
+    """A portion of 64 and one of 200 rows that start at position 16,000 (the portions of a long prompt's later
+    steps): every form the kernel has for these heads (a block per head with 16 rows a wave, and with 32 rows and
+    tiles of 32 keys at head size 128; the heads of a group sharing their tiles, with 16 and 32 rows a wave), the
+    last rows against the plain attention. With a window, the pages that the window has passed are gone from the
+    table (-1), as the cache manager leaves them."""
+    rng = np.random.default_rng(67)
+    o = ops()
+    start, bs = 16000, 16
+    lens, q_lens = [start + 64, start + 200], [64, 200]
+    holes = [max(0, (n - q - window + 1)) // bs for n, q in zip(lens, q_lens)] if window else None
+    far = [n - window + 2 + 5 * r for r, n in enumerate(lens)] if window else None      # just inside the last row's window
+    c = long_case(rng, lens, q_lens, heads, kv_heads, d, bs, holes=holes, far=far)
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    checked = 24                                                       # rows of every request that the plain side computes
+    ref = [long_reference(c, r, heads, kv_heads, d, window, rows=checked) for r in range(2)]
+    assert min(np.abs(x[-1]).max() for x in ref) > 0.15                 # the far key counts in the last rows
+    tiles, row = [], 0
+    for r, (L, n) in enumerate(zip(lens, q_lens)):
+        tiles += [(r, row + q0, min(64, n - q0), L - n + q0) for q0 in range(0, n, 64)]
+        row += n
+    out = torch.zeros(sum(q_lens), heads * d, device=DEV, dtype=torch.bfloat16)
+    forms = [(share, rows) for share in shares for rows in ((16, 32) if (share and d in (32, 64, 96)) or (not share and d == 128) else (16,))]
+    assert len(forms) >= 2
+    for share, rows in forms:
+        for name, blocks in (("paired", o.pair_tiles(tiles, window)), ("single", o.pair_tiles(tiles, window, 1))):
+            out.zero_()
+            o.attention_prefill(out, c["qcat"], c["kc"], c["vc"], c["table"], t(np.array(blocks, np.int32), torch.int32), heads, kv_heads, d, window, scale,
+                                share=share, rows=rows)
+            got = out.float().cpu().numpy()
+            assert np.isfinite(got).all()
+            close_at_own_scale(got[64 - checked:64], ref[0], f"64 rows at {start}, {name}, {share} share, {rows} rows a wave")
+            close_at_own_scale(got[264 - checked:264], ref[1], f"200 rows at {start}, {name}, {share} share, {rows} rows a wave")
+
+
 @pytest.mark.parametrize("heads,kv_heads,d,bs", [(6, 2, 48, 8), (8, 8, 16, 16), (5, 1, 96, 16), (4, 2, 128, 32), (2, 1, 256, 16), (14, 2, 64, 16), (3, 1, 32, 64),
                                                  (22, 2, 32, 16), (6, 1, 256, 16), (28, 4, 128, 16), (7, 1, 16, 8), (16, 2, 64, 16), (6, 1, 96, 16)])
 @pytest.mark.parametrize("window", [None, 21, 300])

@@ -149,6 +149,56 @@ def test_pages_are_counted_by_what_a_request_holds():
     assert "scheduler is full" in str(e.value)
 
 
+def test_the_group_of_layers_that_binds_decides():
+    """Not in the reference, which has one group: with a pool per group of layers, every count is kept per
+    group and a request is admitted, a chunk runs and a decode proceeds only where no group's bound is
+    passed. One group alone gives the reference's numbers (the traces above)."""
+    fields = dict(token_budget=64, max_chunk=16, block_size=4, watermark_permille=1000)
+    # a group that keeps every key (40 pages) and one that holds at most 28 tokens of a request (7 pages each) with 14 pages
+    cfg = SchedConfig.for_groups([(40, -1), (14, 28)], **fields)
+    assert cfg.groups == ((40, -1), (14, 28)) and cfg.blocks(100) == 25 and cfg.blocks(100, 1) == 7 and cfg.blocks(10, 1) == 3
+    s = Scheduler(cfg)
+    # by the first group three requests of 48 tokens fit (36 of 40 pages); the second holds two (14 of 14 pages)
+    with pytest.raises(AlofaError) as e:
+        s.step(SchedInput(arrivals=[(1, 40, 8), (2, 40, 8), (3, 40, 8)]))
+    assert e.value.name == "capacity" and "watermark" in str(e.value) and s.n_live() == 0
+    a = s.step(SchedInput(arrivals=[(1, 40, 8), (2, 40, 8)]))
+    assert a.prefill == [(1, 0, 16), (2, 0, 16)] and not s.would_admit(4, 4)            # the window's group is full, the other is not
+    assert (s.of_group("blocks_used", 0), s.of_group("blocks_used", 1)) == (8, 8) and s.blocks_used == 8
+    finished, ticks = [], 0
+    while s.n_live() and ticks < 100:
+        a = s.step(SchedInput())
+        ticks += 1
+        finished += a.finished
+        for g in range(2):
+            assert s.of_group("blocks_used", g) == s.of_group("blocks_held", g) + s.of_group("cached_blocks", g) <= cfg.groups[g][0]
+        assert a.preempted == []
+    assert sorted(finished) == [1, 2] and (s.of_group("cached_blocks", 0), s.of_group("cached_blocks", 1)) == (24, 14)
+    with pytest.raises(AlofaError):
+        s.step(SchedInput(freed_blocks=[24, 15]))                                       # more than the second group holds cached
+    s.step(SchedInput(freed_blocks=[24, 14]))
+    assert (s.of_group("blocks_used", 0), s.of_group("blocks_used", 1)) == (0, 0)
+    with pytest.raises(AlofaError):
+        s.step(SchedInput(freed_blocks=[0]))                                            # one count per group
+    # the other way round: the group that keeps every key binds (as in the single-group case above, pages run out
+    # only while a finished request's are still counted as cached), and a decode that needs a page of it preempts
+    s = Scheduler(SchedConfig.for_groups([(6, -1), (100, 28)], token_budget=64, max_chunk=64, block_size=4, watermark_permille=1000))
+    s.step(SchedInput(arrivals=[(1, 4, 1)]))
+    assert s.step(SchedInput()).finished == [1] and (s.of_group("cached_blocks", 0), s.of_group("cached_blocks", 1)) == (2, 2)
+    s.step(SchedInput(arrivals=[(2, 6, 6), (3, 6, 6)]))
+    seen = None
+    for _ in range(6):
+        a = s.step(SchedInput())
+        assert s.of_group("blocks_used", 0) <= 6 and s.of_group("blocks_used", 1) <= 100
+        if a.preempted:
+            seen = a
+            break
+    assert seen is not None and seen.preempted == [3] and 2 in seen.decode and 3 not in seen.decode
+    assert s.of_group("blocks_used", 1) == s.of_group("blocks_held", 1) + s.of_group("cached_blocks", 1) == 3 + 2
+    with pytest.raises(AlofaError):
+        s.cfg = SchedConfig(token_budget=64, max_chunk=64, block_size=4, capacity_blocks=6)    # the number of groups cannot change
+
+
 def test_cancel_blocks_arrival_in_the_same_tick_and_refusals_are_named():
     s = Scheduler(SchedConfig())
     a = s.step(SchedInput(arrivals=[(7, 5, 2)], cancelled=[7]))
