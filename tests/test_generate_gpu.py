@@ -425,38 +425,42 @@ def test_greedy_choice_inside_the_step_changes_no_token(tmp_path, monkeypatch):
 
 def test_batches_that_grow_past_64_rows_and_shrink_again_replay_their_graphs(tmp_path, monkeypatch):
     """A vocabulary of 9,001 (searched by the two-stage argmax through a scratch buffer that is kept between
-    calls; too short for the product that takes the argmax with it) and batches that rise from 60 to 70 rows
-    one request at a time, then fall as requests end: every batch size captures a graph that addresses the
-    scratch buffer of its day, and the graphs of the smaller batches are replayed after the buffer was
-    outgrown. Token for token what steps run kernel by kernel give."""
+    calls; too short for the product that takes the argmax with it). Thirty long requests decode (their graph
+    addresses the scratch buffer of that day), forty short ones join four a tick until seventy rows decode
+    (the buffer is outgrown at 65 rows and replaced), then end: the thirty are alone again and their old graph
+    is replayed for twenty more steps. Token for token what steps run kernel by kernel give."""
     from alofa_amd import Engine, ops
     from alofa_amd.weights import write_random_model
     cfg = dict(TINY["A"], vocab_size=9001)
     d = tmp_path / "vocabulary_9001"
     write_random_model(cfg, d, seed=93)
-    prompts = [random_ids(700 + i, 3 + i % 5, cfg["vocab_size"]) for i in range(70)]
+    long_ones = [random_ids(700 + i, 70, cfg["vocab_size"]) for i in range(30)]
+    short_ones = [random_ids(800 + i, 3 + i % 5, cfg["vocab_size"]) for i in range(40)]
+    assert not ops.can_gemm_argmax(70, torch.empty(9001, 64, dtype=torch.bfloat16))
 
     def play():
-        eng = Engine(d, dtype="bfloat16", max_tokens=64, max_batch=72, token_budget=256)
-        core, sizes = eng.core, set()
-        for i in range(60):
-            core.submit(i + 1, prompts[i], 30 + i % 7)
-        n = 60
+        monkeypatch.setattr(ops, "_argmax_scratch", {})
+        monkeypatch.setattr(ops, "_argmax_retired", [])
+        eng = Engine(d, dtype="bfloat16", max_tokens=128, max_batch=72, token_budget=4096)
+        core, sizes, n = eng.core, [], 0
+        for i, p in enumerate(long_ones):
+            core.submit(i + 1, p, 57)
         while core.has_work():
             core.tick()
             if core.last_action.decode and not core.last_action.prefill:
-                sizes.add(len(core.last_action.decode))
-            if n < 70 and core.ticks % 2 == 0:
-                core.submit(n + 1, prompts[n], 12 + n % 5)
-                n += 1
+                sizes.append(len(core.last_action.decode))
+            if core.ticks >= 4 and n < 40:
+                for p in short_ones[n:n + 4]:
+                    core.submit(100 + n, p, 20)
+                    n += 1
         core.flush()
-        return [core.output(i + 1) for i in range(70)], sizes, eng.step_fn.graph_replays
+        outs = [core.output(i + 1) for i in range(30)] + [core.output(100 + i) for i in range(40)]
+        return outs, sizes, eng.step_fn.graph_replays, len(ops._argmax_retired)
 
-    assert not ops.can_gemm_argmax(70, torch.empty(9001, 64, dtype=torch.bfloat16))
-    captured, sizes, replays = play()
-    assert max(sizes) > 64 and min(sizes) < 60 and len(sizes) > 12 and replays > 20
+    captured, sizes, replays, outgrown = play()
+    assert max(sizes) == 70 and sizes[0] == 30 and sizes[-20:] == [30] * 20 and replays > 25 and outgrown >= 1, (sizes, replays, outgrown)
     monkeypatch.setenv("ALOFA_GRAPHS", "0")
-    eager, sizes_eager, none = play()
+    eager, sizes_eager, none, _ = play()
     assert none == 0 and sizes_eager == sizes and eager == captured
 
 
