@@ -43,7 +43,7 @@ def _lib_name() -> str:
     return f"libalofa_hip_{_hash()}.so"
 
 
-HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-fopenmp"]      # (threads share out independent outputs of the plain path only)
 _host = None
 
 

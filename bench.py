@@ -349,12 +349,15 @@ def continuous_batch(args):
             assert len(core.output(base + r)) == new
             core.release(base + r)
         return dt, ticks, decode_s, decode_steps
+    roofs = measure_roofs()
     say("warm-up run")
     run()
-    dt, ticks, decode_s, decode_steps = run()
+    runs = [run() for _ in range(3)]                      # three timed runs after the warm-up; the median one is reported
+    dt, ticks, decode_s, decode_steps = sorted(runs, key=lambda r: r[0])[1]
     dbytes = 2 if args.dtype == "bfloat16" else 4
     mean_ctx = [n + new // 2 for n in lens]
     step_ms = decode_s / max(1, decode_steps) * 1e3
+    achieved = decode_bytes(cfg, mean_ctx, dbytes) / (step_ms / 1e3) / 1e9 if decode_steps else None
     out = {"metric": "generated tok/s, continuous batch of 64 requests (prompts U[128,2048], 256 new tokens, chunked prefill 512), Qwen2.5-7B sizes",
            "value": round(n_req * new / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": ticks, "warmup": ticks, "ms_per_step": round(dt / ticks * 1e3, 4),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
@@ -362,10 +365,14 @@ def continuous_batch(args):
            "config": flat_config(name, cfg, layers, global_batch=n_req, seq_len=context, prompt_tokens=sum(lens), new_tokens=new, max_chunk=512, token_budget=2048),
            "total_tok_s": round((sum(lens) + n_req * new) / dt, 1), "seconds": round(dt, 3),
            "roofline": {"bound": "hbm", "what": "the ticks in which all 64 requests decode and nothing is prefilled", "steps": decode_steps, "ms_per_step": round(step_ms, 4),
-                        "achieved": round(decode_bytes(cfg, mean_ctx, dbytes) / (step_ms / 1e3) / 1e9, 1) if decode_steps else None, "peak": PEAK_HBM_GBS, "unit": "GB/s"},
-           "memory": {k: int(v) for k, v in eng.memory().items()}}
-    if out["roofline"]["achieved"]:
-        out["roofline"]["frac"] = round(out["roofline"]["achieved"] / PEAK_HBM_GBS, 4)
+                        "achieved": round(achieved, 1) if achieved else None, "peak": PEAK_HBM_GBS, "unit": "GB/s"},
+           "spread": {"seconds": {"median": round(dt, 3), "min": round(min(r[0] for r in runs), 3), "max": round(max(r[0] for r in runs), 3), "repeats": len(runs)},
+                      "generated_tok_s": sorted(round(n_req * new / r[0], 1) for r in runs),
+                      "decode_step": spread([r[2] / max(1, r[3]) for r in runs])},
+           "roofs": roofs, "memory": {k: int(v) for k, v in eng.memory().items()}}
+    if achieved:
+        out["roofline"]["frac"] = round(achieved / PEAK_HBM_GBS, 4)
+        out["roofline"]["frac_measured"] = round(achieved / roofs["hbm_copy_gbs"], 4)
     print(json.dumps(out))
     return 0
 
@@ -383,51 +390,65 @@ def long_prompts(args):
     model = device_model(cfg, args.dtype, 20260918)
     dbytes = 2 if args.dtype == "bfloat16" else 4
     n_req, plen, new, context = 8, 16384, 128, 32768
+    roofs = measure_roofs()
     rng = np.random.default_rng(8)
     per_req = (plen + new + BLOCK - 1) // BLOCK
     eng = Engine(None, dtype=args.dtype, max_tokens=context, max_batch=n_req, kv_blocks=per_req * n_req + 64, block_size=BLOCK,
                  token_budget=4096, max_chunk=2048, watermark_permille=1000, model=model, report=say)
     core = eng.core
-    for r in range(n_req):
-        core.submit(r + 1, [int(t) for t in rng.integers(0, cfg["vocab_size"], plen)], new)
-    sync()
-    t0 = time.perf_counter()
-    prefill_s, prefill_tokens, prefill_fl, ticks = 0.0, 0, 0.0, 0
-    while core.has_work():
-        t1 = time.perf_counter()
-        core.tick()
-        act = core.last_action
-        if act.prefill:                     # ticks that bring prompt portions (later ones carry a few decoded tokens beside them)
-            sync()
-            prefill_s += time.perf_counter() - t1
-            prefill_tokens += sum(e - s for _, s, e in act.prefill)
-            prefill_fl += sum(prefill_flops(cfg, e - s, wanted=int(e == plen), start=s) for _, s, e in act.prefill)
-        ticks += 1
-        if ticks % 16 == 0:
-            say(f"tick {ticks}: {prefill_tokens} prompt tokens so far")
-    sync()
-    dt = time.perf_counter() - t0
+
+    def run(base):
+        """All eight prompts through the engine loop; the ticks that bring prompt portions are timed by themselves."""
+        for r in range(n_req):
+            core.submit(base + r, [int(t) for t in rng.integers(0, cfg["vocab_size"], plen)], new)
+        sync()
+        t0 = time.perf_counter()
+        prefill_s, prefill_tokens, prefill_fl, ticks = 0.0, 0, 0.0, 0
+        while core.has_work():
+            t1 = time.perf_counter()
+            core.tick()
+            act = core.last_action
+            if act.prefill:                     # ticks that bring prompt portions (later ones carry a few decoded tokens beside them)
+                sync()
+                prefill_s += time.perf_counter() - t1
+                prefill_tokens += sum(e - s for _, s, e in act.prefill)
+                prefill_fl += sum(prefill_flops(cfg, e - s, wanted=int(e == plen), start=s) for _, s, e in act.prefill)
+            ticks += 1
+            if ticks % 16 == 0:
+                say(f"tick {ticks}: {prefill_tokens} prompt tokens so far")
+        sync()
+        dt = time.perf_counter() - t0
+        for r in range(n_req):
+            assert len(core.output(base + r)) == new
+            core.release(base + r)
+        return {"prefill_s": prefill_s, "tokens": prefill_tokens, "flops": prefill_fl, "ticks": ticks, "seconds": dt}
+    passes = [run(1000), run(2000)]                           # two passes (the first also warms up); the faster one is reported
+    best = min(passes, key=lambda p: p["prefill_s"])
     memory = eng.memory()
-    for r in range(n_req):
-        assert len(core.output(r + 1)) == new
-        core.release(r + 1)
     del eng, core
     out = {"metric": "prefill tok/s over 8 prompts of 16,384 tokens (chunks of 2,048); decode tok/s @ batch 32, context 4,096 under points; Qwen2.5-32B sizes",
-           "value": round(prefill_tokens / prefill_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": ticks, "warmup": 0, "ms_per_step": round(dt / ticks * 1e3, 3),
+           "value": round(best["tokens"] / best["prefill_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": best["ticks"], "warmup": passes[0]["ticks"],
+           "ms_per_step": round(best["seconds"] / best["ticks"] * 1e3, 3),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic (random weights N(0, 0.02) drawn on the device, uniform random token ids)",
            "config": flat_config(name, cfg, layers, global_batch=n_req, seq_len=context, prompt_len=plen, new_tokens=new, max_chunk=2048, token_budget=4096),
-           "prefill": {"value": round(prefill_tokens / prefill_s, 1), "tokens": prefill_tokens, "ms": round(prefill_s * 1e3, 1),
-                       "frac": round(prefill_fl / prefill_s / PEAK_FLOPS[args.dtype], 4)},
-           "seconds_whole_run": round(dt, 2), "generated_tok_s_whole_run": round(n_req * new / dt, 1), "memory": {k: int(v) for k, v in memory.items()}}
-    p = DecodePoint(model, cfg, args.dtype, 32, 4096 - 64, context=4096 + 64)
+           "prefill": {"value": round(best["tokens"] / best["prefill_s"], 1), "tokens": best["tokens"], "ms": round(best["prefill_s"] * 1e3, 1),
+                       "frac": round(best["flops"] / best["prefill_s"] / PEAK_FLOPS[args.dtype], 4)},
+           "spread": {"prefill_tok_s": [round(p["tokens"] / p["prefill_s"], 1) for p in passes]},
+           "seconds_whole_run": round(best["seconds"], 2), "generated_tok_s_whole_run": round(n_req * new / best["seconds"], 1), "memory": {k: int(v) for k, v in memory.items()}}
+    if args.dtype == "bfloat16":
+        out["prefill"]["frac_measured"] = round(best["flops"] / best["prefill_s"] / (roofs["gemm_bf16_tflops"] * 1e12), 4)
+    p = DecodePoint(model, cfg, args.dtype, 32, 4096 - 128, context=4096 + 64)
     p.run(8)
-    ms = p.run(24)
+    samples = [p.run(24) for _ in range(3)]
+    ms = statistics.median(samples)
     ctx_lens = p.context_lengths()
     achieved = decode_bytes(cfg, ctx_lens, dbytes) / ms / 1e9
     out["points"] = {"decode_b32_ctx4096": round(32 / ms, 1)}
+    out["spread"]["decode_b32_ctx4096"] = spread(samples)
     out["roofline"] = {"bound": "hbm", "what": "decode step at batch 32, context about 4,096", "ms_per_step": round(ms * 1e3, 4), "achieved": round(achieved, 1),
-                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)}
+                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4), "frac_measured": round(achieved / roofs["hbm_copy_gbs"], 4)}
+    out["roofs"] = roofs
     p.close()
     print(json.dumps(out))
     return 0

@@ -71,3 +71,20 @@ def test_every_cutting_at_real_widths(sized, dtype):
     r.cache.check()
     if dtype == "bfloat16":     # the last use of this size: let the plain side's weights go
         plain_model.cache_clear()
+
+
+def test_six_layers_of_the_half_billion_model_against_the_librarys_own_plain_path(tmp_path):
+    """The library's plain path (C++ on the host: float64 sums in formula order, contiguous keys and values; the NumPy
+    transcription in tests/plain pins it on the tiny models) as a second twin where NumPy would take minutes: six
+    layers of the 0.5B widths with the full vocabulary, 96 tokens, float32 at the reference's 1e-5 in two cuttings."""
+    from alofa_amd.plain import PlainModel
+    from alofa_amd.replay import Replayer
+    from alofa_amd.weights import write_random_model
+    cfg = dict(config_of("0.5b"), num_hidden_layers=6)
+    write_random_model(cfg, tmp_path, seed=2100)
+    ids = random_ids(6, 96, cfg["vocab_size"])
+    print("the library's plain path, six layers at 0.5B widths", flush=True)
+    ref = PlainModel(tmp_path, max_tokens=128).run(ids)
+    r = Replayer(tmp_path, "float32", 256)
+    assert_close(collect(r, whole("w", ids))["w"], ref, "float32", "six layers whole")
+    assert_close(collect(r, bulk_and_tail("t", ids))["t"], ref, "float32", "six layers bulk+tail")
