@@ -314,7 +314,7 @@ def continuous_batch(args):
     tokens a tick): the whole run through the engine loop, timed from the first tick to the last."""
     import numpy as np
     from alofa_amd import Engine
-    name = "7b"
+    name = args.config
     layers = args.layers or CONFIGS[name]["num_hidden_layers"]
     cfg = dict(CONFIGS[name], num_hidden_layers=layers)
     say(f"drawing {name} weights on the device ({layers} layers)")
@@ -331,7 +331,7 @@ def continuous_batch(args):
         base = (core.ticks + 1) * 1000
         for r, n in enumerate(lens):
             core.submit(base + r, [int(t) for t in rng.integers(0, cfg["vocab_size"], n)], new)
-        ticks, decode_s, decode_steps, decode_ctx = 0, 0.0, 0, []
+        ticks, decode_s, decode_steps, mixed = 0, 0.0, 0, [0, 0.0, 0]
         sync()
         t0 = time.perf_counter()
         while core.has_work():
@@ -342,9 +342,14 @@ def continuous_batch(args):
                 sync()
                 decode_s += time.perf_counter() - t1
                 decode_steps += 1
+            elif act.prefill and args.time_mixed:         # (only on request: the synchronisation takes the host's head start away)
+                sync()
+                mixed[0], mixed[1], mixed[2] = mixed[0] + 1, mixed[1] + time.perf_counter() - t1, mixed[2] + core.last_rows
             ticks += 1
         sync()
         dt = time.perf_counter() - t0
+        if args.time_mixed and mixed[0]:
+            say(f"{mixed[0]} ticks with prompt portions: {mixed[1] / mixed[0] * 1e3:.3f} ms and {mixed[2] / mixed[0]:.0f} rows a tick")
         for r in range(n_req):
             assert len(core.output(base + r)) == new
             core.release(base + r)
@@ -358,7 +363,7 @@ def continuous_batch(args):
     mean_ctx = [n + new // 2 for n in lens]
     step_ms = decode_s / max(1, decode_steps) * 1e3
     achieved = decode_bytes(cfg, mean_ctx, dbytes) / (step_ms / 1e3) / 1e9 if decode_steps else None
-    out = {"metric": "generated tok/s, continuous batch of 64 requests (prompts U[128,2048], 256 new tokens, chunked prefill 512), Qwen2.5-7B sizes",
+    out = {"metric": f"generated tok/s, continuous batch of 64 requests (prompts U[128,2048], 256 new tokens, chunked prefill 512), Qwen2.5-{name.upper()} sizes",
            "value": round(n_req * new / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": ticks, "warmup": ticks, "ms_per_step": round(dt / ticks * 1e3, 4),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
            "data": "synthetic (random weights N(0, 0.02) drawn on the device, uniform random token ids)",
@@ -488,6 +493,8 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points, the prefill, the repeats and the roofs")
     ap.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its line")
+    ap.add_argument("--serve", action="store_true", help="the continuous batch of 64 requests (prompts of 128..2,048 tokens, 256 new tokens, chunks of 512) at the sizes of --config")
+    ap.add_argument("--time-mixed", action="store_true", help="with --serve: also time the ticks that bring prompt portions by themselves (one more synchronisation a tick)")
     ap.add_argument("--sweep", choices=["batch", "context"], default=None, help="decode steps over batch sizes or over contexts, a line per point (the sizes of --config)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -498,7 +505,7 @@ def main():
     load()
     if args.sweep:
         return sweep(args)
-    if args.config == "7b":
+    if args.config == "7b" or args.serve:
         return continuous_batch(args)
     if args.config == "32b":
         return long_prompts(args)
