@@ -246,7 +246,10 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     }
     // Every wave waits until its partial sums have been performed in memory; only then may the
     // block be counted. A release fence of workgroup scope does not wait for stores to memory (the
-    // counter could overtake them), and one of device scope would write this die's whole L2 back.
+    // counter could overtake them), and one of device scope writes this die's whole L2 back (measured with such
+    // fences in every hand-over of this library: a decode step of 32 requests 2.81 instead of 1.24 ms). What makes the
+    // hand-over sound here is the memory, not a fence: the workspace is uncached, the partial sums are stored and
+    // read at device scope (past the L2s), and the counter is bumped only after every store has been acknowledged.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
