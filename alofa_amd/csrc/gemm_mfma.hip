@@ -619,17 +619,92 @@ __global__ void __launch_bounds__(256) split_sum_kernel(TO* __restrict__ out, in
   }
 }
 
+// An RMSNorm that follows a product which adds to the residual stream, where the product's last launch has whole
+// rows in hand (the launch that adds the shares of K): weight null for none.
+struct ThenNorm {
+  const float* weight;   // [N]
+  float eps;
+  bf16_t* out;           // [M, ld]: rmsnorm(residual's new rows) * weight
+  int64_t ld;
+};
+constexpr ThenNorm kNoNorm = {nullptr, 0.f, nullptr, 0};
+
+// The shares added to the residual stream as in split_sum_kernel, by a block per row that keeps the row in registers
+// (K4 groups of four columns a thread) and goes on to normalise it: the sums, the threads' places and the arithmetic
+// are those of split_sum_kernel followed by rmsnorm_kernel (elementwise.hip), value for value, without the second
+// launch and its trip through memory.
+template <int K4>
+__global__ void __launch_bounds__(256) split_sum_norm_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ parts, int shares,
+                                                             int M, int N, ThenNorm then) {
+  __shared__ float scratch[4];
+  const int m = blockIdx.x, groups = N / 4;
+  const int64_t part = static_cast<int64_t>(M) * N;
+  float4 xs[K4], ws[K4];
+#pragma unroll
+  for (int i = 0; i < K4; ++i) {
+    const int g = threadIdx.x + 256 * i;
+    xs[i] = ws[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (g < groups) {     // uniform but for the row's last threads
+      const float* src = parts + static_cast<int64_t>(m) * N + 4 * g;
+      float* dst = out + static_cast<int64_t>(m) * ldo + 4 * g;
+      const float4 old = *reinterpret_cast<const float4*>(dst);
+      ws[i] = reinterpret_cast<const float4*>(then.weight)[g];
+      float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int s0 = 0; s0 < shares; s0 += 8) {     // (eight parts' loads on their way together)
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(src + min(s0 + u, shares - 1) * part);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < shares) { sum.x += v[u].x; sum.y += v[u].y; sum.z += v[u].z; sum.w += v[u].w; }
+      }
+      xs[i] = make_float4(old.x + sum.x, old.y + sum.y, old.z + sum.z, old.w + sum.w);
+      *reinterpret_cast<float4*>(dst) = xs[i];
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < K4; ++i) {      // ascending columns within the thread
+    ss += xs[i].x * xs[i].x;
+    ss += xs[i].y * xs[i].y;
+    ss += xs[i].z * xs[i].z;
+    ss += xs[i].w * xs[i].w;
+  }
+  ss = block_sum<float, 256>(ss, scratch);
+  const float scale = 1.f / sqrtf(ss / static_cast<float>(N) + then.eps);
+#pragma unroll
+  for (int i = 0; i < K4; ++i) {
+    const int g = threadIdx.x + 256 * i;
+    if (g < groups)
+      *reinterpret_cast<uint2*>(then.out + static_cast<int64_t>(m) * then.ld + 4 * g) =
+          make_uint2(pack_bf16x2(xs[i].x * scale * ws[i].x, xs[i].y * scale * ws[i].y), pack_bf16x2(xs[i].z * scale * ws[i].z, xs[i].w * scale * ws[i].w));
+  }
+}
+
 // K shared out among the blocks of a launch (tiles of 64 rows x 64 WTN columns, a ring of S slabs), and a second
 // launch that adds the shares and runs the epilogue. The parts lie in the workspace as [shares, M, N] floats.
 template <int kEpilogue, typename TO, int WTN, int S, int WTM = 1>
 static int launch_dma_sliced(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
-                             int shares, hipStream_t stream) {
+                             int shares, hipStream_t stream, const ThenNorm& then, int* then_done) {
   const int tiles_n = (N + 64 * WTN - 1) / (64 * WTN), tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
   const Workspace& g_ws = workspace();
   ALOFA_REQUIRE(g_ws.tiles != nullptr && N % 4 == 0 && static_cast<int64_t>(shares) * M * N <= g_ws.tile_floats,
                 "gemm_mfma: %d shares of %d x %d sums do not fit the workspace (or N is no multiple of four)", shares, M, N);
   gemm_dma_kernel<kMfStore, float, WTM, WTN, S, 2><<<tiles_n * tiles_m * shares, 256, 0, stream>>>(
       g_ws.tiles, N, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), nullptr, ldw, nullptr, M, N, K, tiles_m, tiles_n, 1, shares);
+  if constexpr (kEpilogue == kMfResidual && sizeof(TO) == 4) {
+    // the norm behind the product rides on the launch that adds the shares (rows up to 8,192 wide stay in registers)
+    if (then.weight != nullptr && N <= 8192 && ldo % 4 == 0 && then.ld % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(then.weight) % 16 == 0 && reinterpret_cast<uintptr_t>(then.out) % 8 == 0) {
+      float* o = static_cast<float*>(out);
+      if (N <= 1024) split_sum_norm_kernel<1><<<M, 256, 0, stream>>>(o, ldo, g_ws.tiles, shares, M, N, then);
+      else if (N <= 2048) split_sum_norm_kernel<2><<<M, 256, 0, stream>>>(o, ldo, g_ws.tiles, shares, M, N, then);
+      else if (N <= 4096) split_sum_norm_kernel<4><<<M, 256, 0, stream>>>(o, ldo, g_ws.tiles, shares, M, N, then);
+      else split_sum_norm_kernel<8><<<M, 256, 0, stream>>>(o, ldo, g_ws.tiles, shares, M, N, then);
+      *then_done = 1;
+      return 0;
+    }
+  }
   const int64_t threads = static_cast<int64_t>(M) * (N / 4);
   split_sum_kernel<kEpilogue, TO><<<static_cast<int>((threads + 255) / 256), 256, 0, stream>>>(static_cast<TO*>(out), ldo, g_ws.tiles, shares, bias, M, N);
   return 0;
@@ -670,7 +745,7 @@ static int k_shares(int64_t tiles, int64_t tile_floats, int K) {
 
 template <int kEpilogue, typename TO>
 static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
-                       const float* bias, int M, int N, int K, hipStream_t stream) {
+                       const float* bias, int M, int N, int K, hipStream_t stream, const ThenNorm& then, int* then_done) {
   if constexpr (kEpilogue == kMfSwiglu) {
     // A block computes gate and up of the same 64 columns. With K a multiple of 64 and tiles that do not fill the
     // chip twice over, the slabs go straight from memory into a ring in LDS (0.5B sizes, us against the kernel
@@ -795,13 +870,13 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
       if (kEpilogue != kMfSwiglu && ring && long_k && (M <= 64 || (M <= 256 && !tall && K >= 3072)) && wide_tiles <= 36 && N % 4 == 0 && slices > 1 &&
           static_cast<int64_t>(slices) * M * N <= workspace().tile_floats) {
         if constexpr (kEpilogue != kMfSwiglu) {
-          if (launch_dma_sliced<kEpilogue, TO, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, slices, stream)) return 1;
+          if (launch_dma_sliced<kEpilogue, TO, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, slices, stream, then, then_done)) return 1;
         }
       } else
       if (tall && kEpilogue != kMfSwiglu && ring && N % 4 == 0 &&
           static_cast<int64_t>(tall_shares) * M * N <= workspace().tile_floats) {
         if constexpr (kEpilogue != kMfSwiglu) {
-          if (launch_dma_sliced<kEpilogue, TO, 2, 3, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, tall_shares, stream)) return 1;
+          if (launch_dma_sliced<kEpilogue, TO, 2, 3, 2>(out, ldo, A, lda, W, ldw, bias, M, N, K, tall_shares, stream, then, then_done)) return 1;
         }
       } else
       if (ring && long_k && tiles_128x64 >= 144 && tiles_128x64 <= 256) {
@@ -839,8 +914,12 @@ using namespace alofa;
 
 // bfloat16 A [M, K] and W [N, K] (W2 for the swiglu epilogue); K a multiple of 8, rows 16-byte
 // aligned. Epilogues: 0 store (+ bias) as o_dtype, 1 add to the float residual, 2 swiglu.
+// then_w (may be null; residual epilogue only): an RMSNorm (then_w [N], then_eps) of the residual's new rows is
+// wanted in then_out (bfloat16 [M, then_ld]) afterwards. Where the product's last launch has whole rows in hand it
+// writes them and sets *then_done to 1; otherwise *then_done stays 0 and the norm is the caller's to run.
 extern "C" int alofa_gemm_mfma(void* out, int o_dtype, int64_t ldo, const void* A, int64_t lda, const void* W,
                                const void* W2, int64_t ldw, const float* bias, int M, int N, int K, int epilogue,
+                               const float* then_w, float then_eps, void* then_out, int64_t then_ld, int* then_done,
                                hipStream_t stream) {
   ALOFA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_mfma: M=%d N=%d K=%d must be positive", M, N, K);
   ALOFA_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_mfma: K=%d, lda=%lld, ldw=%lld must be multiples of 8", K,
@@ -848,15 +927,21 @@ extern "C" int alofa_gemm_mfma(void* out, int o_dtype, int64_t ldo, const void* 
   ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 &&
                     reinterpret_cast<uintptr_t>(W2) % 16 == 0, "gemm_mfma: operands must be 16-byte aligned");
   ALOFA_REQUIRE(lda >= K && ldw >= K && ldo >= N, "gemm_mfma: a leading dimension is shorter than its row");
+  ALOFA_REQUIRE(then_w == nullptr || (epilogue == kMfResidual && then_out != nullptr && then_ld >= N && then_eps > 0.f && then_done != nullptr),
+                "gemm_mfma: a norm behind the product goes with the residual epilogue, an output of the product's shape and a positive eps");
+  const ThenNorm then{then_w, then_eps, static_cast<bf16_t*>(then_out), then_ld};
+  int none = 0;
+  int* done = then_done ? then_done : &none;
+  *done = 0;
   if (epilogue == kMfStore && o_dtype == kBF16)
-    return launch_mfma<kMfStore, bf16_t>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream);
+    return launch_mfma<kMfStore, bf16_t>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream, kNoNorm, done);
   if (epilogue == kMfStore && o_dtype == kF32)
-    return launch_mfma<kMfStore, float>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream);
+    return launch_mfma<kMfStore, float>(out, ldo, A, lda, W, nullptr, ldw, bias, M, N, K, stream, kNoNorm, done);
   if (epilogue == kMfResidual && o_dtype == kF32)
-    return launch_mfma<kMfResidual, float>(out, ldo, A, lda, W, nullptr, ldw, nullptr, M, N, K, stream);
+    return launch_mfma<kMfResidual, float>(out, ldo, A, lda, W, nullptr, ldw, nullptr, M, N, K, stream, then, done);
   if (epilogue == kMfSwiglu && o_dtype == kBF16) {
     ALOFA_REQUIRE(W2 != nullptr, "gemm_mfma: the swiglu epilogue needs the up matrix");
-    return launch_mfma<kMfSwiglu, bf16_t>(out, ldo, A, lda, W, W2, ldw, nullptr, M, N, K, stream);
+    return launch_mfma<kMfSwiglu, bf16_t>(out, ldo, A, lda, W, W2, ldw, nullptr, M, N, K, stream, kNoNorm, done);
   }
   ALOFA_REQUIRE(false, "gemm_mfma: unsupported epilogue %d with out dtype %d", epilogue, o_dtype);
 }

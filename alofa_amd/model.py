@@ -103,8 +103,18 @@ class Model:
         """Run the tokens of the step through every entry; returns the float32
         residual stream [T, hidden]."""
         hidden = self.embedding.forward(ctx, ids)
+        rows, normed = hidden.shape[0], None
         for i, e in enumerate(self.order):
-            self.blocks[e.layer].forward(ctx, i, hidden)
+            block = self.blocks[e.layer]
+            if not block.takes_normed:
+                block.forward(ctx, i, hidden)
+                normed = None
+                continue
+            # the norm the next block starts with may be left by this block's last product (a launch less)
+            nxt = self.blocks[self.order[i + 1].layer] if i + 1 < len(self.order) else None
+            norm = nxt.wants_normed(rows) if nxt is not None and nxt.takes_normed else None
+            then = (norm, ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)) if norm is not None and norm.as_rmsnorm() is not None else None
+            normed = then[1] if block.forward(ctx, i, hidden, normed, then) else None
         return hidden
 
     def logits(self, ctx, hidden: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:

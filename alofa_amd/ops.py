@@ -279,15 +279,29 @@ def _norm_operands(a: torch.Tensor, norm: tuple, K: int):
 
 
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         add_to_out: bool = False, exact: bool = False, kernel: Optional[str] = None, norm: Optional[tuple] = None) -> None:
+         add_to_out: bool = False, exact: bool = False, kernel: Optional[str] = None, norm: Optional[tuple] = None,
+         then_norm: Optional[tuple] = None) -> None:
     """out = a @ w.T (+ bias), or out += a @ w.T when ``add_to_out`` (out is then
     the float32 residual stream). w is [out_features, in_features]. ``kernel``
     names the bfloat16 kernel ("rows", "stream" or "tiled") instead of ``few_rows_kernel``.
     ``norm`` = (weight, eps): ``a`` holds float32 rows that take an RMSNorm on their way
-    into the product (only where ``can_fuse_norm`` says so)."""
+    into the product (only where ``can_fuse_norm`` says so).
+    ``then_norm`` = (weight, eps, rows) with ``add_to_out``: afterwards ``rows`` (out's shape, the
+    activation dtype) holds the RMSNorm of out's new rows. Where the product's last launch has whole
+    rows in hand (the tiled kernel with K shared out and a launch that adds the shares) the norm rides
+    on it; everywhere else it is the norm kernel, run here: the values are the same either way."""
     _gpu("out", out, None, 2), _gpu("a", a, None, 2), _gpu("w", w, None, 2)
     M, K = a.shape
     N = w.shape[0]
+    then_w = then_rows = None
+    then_eps = 0.0
+    if then_norm is not None:
+        then_w, then_eps, then_rows = then_norm
+        if not add_to_out or norm is not None:
+            raise AlofaError("invalid_argument", "a norm behind a product goes with a product that adds to the residual stream")
+        _gpu("norm weight", then_w, torch.float32, 1), _contig("norm weight", then_w), _gpu("normed rows", then_rows, None, 2), _contig("normed rows", then_rows)
+        if then_w.shape[0] != N or tuple(then_rows.shape) != (M, N) or not then_eps > 0:
+            raise AlofaError("shape_mismatch", "the norm behind the product does not fit its output", f"weight={tuple(then_w.shape)} rows={tuple(then_rows.shape)} out={tuple(out.shape)}")
     if norm is not None:
         if add_to_out or exact or not can_fuse_norm(M, w, out.dtype, kernel=kernel) or tuple(out.shape) != (M, N) or w.shape[1] != K:
             raise AlofaError("unsupported", "no kernel takes a norm with this product", f"a={tuple(a.shape)} w={tuple(w.shape)} out={out.dtype}")
@@ -312,14 +326,23 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
     if not exact and _mfma_operands(a, w):
         _ensure_workspace(a.device)
         entry = _product_entry(kernel, M, N, K)
-        no_norm = (_ptr(None), _F(0.0)) if entry != "alofa_gemm_mfma" else ()
+        done = _I(0)
+        if entry == "alofa_gemm_mfma":
+            ride = then_rows is not None and then_rows.dtype is torch.bfloat16 and FUSE_NORMS
+            more = (_ptr(then_w if ride else None), _F(then_eps), _ptr(then_rows if ride else None), _L(N), ctypes.byref(done))
+        else:
+            more = (_ptr(None), _F(0.0))
         _call(entry, _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)),
               _ptr(a), _L(_rows("a", a)), _ptr(w), _ptr(None), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
-              _I(ADD_TO_RESIDUAL if add_to_out else STORE), *no_norm, _stream())
+              _I(ADD_TO_RESIDUAL if add_to_out else STORE), *more, _stream())
+        if then_rows is not None and not done.value:
+            rmsnorm(then_rows, out, then_w, then_eps, False)
         return
     _call("alofa_gemm_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
           _ptr(w), _I(dtype_code(w)), _L(_rows("w", w)), _ptr(bias), _I(M), _I(N), _I(K),
           _I(ADD_TO_RESIDUAL if add_to_out else STORE), _I(int(exact)), _stream())
+    if then_rows is not None:
+        rmsnorm(then_rows, out, then_w, then_eps, exact)
 
 
 def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, exact: bool = False,
@@ -341,9 +364,9 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate: torch.Tensor, w_up: 
     if not exact and out.dtype is torch.bfloat16 and _mfma_operands(a, w_gate) and _mfma_operands(a, w_up):
         _ensure_workspace(a.device)
         entry = _product_entry(kernel, M, 2 * N, K, True)
-        no_norm = (_ptr(None), _F(0.0)) if entry != "alofa_gemm_mfma" else ()
+        more = (_ptr(None), _F(0.0)) if entry != "alofa_gemm_mfma" else (_ptr(None), _F(0.0), _ptr(None), _L(0), _ptr(None))
         _call(entry, _ptr(out), _I(BF16), _L(_rows("out", out)), _ptr(a), _L(_rows("a", a)), _ptr(w_gate), _ptr(w_up),
-              _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), *no_norm, _stream())
+              _L(_rows("w_gate", w_gate)), _ptr(None), _I(M), _I(N), _I(K), _I(SWIGLU), *more, _stream())
         return
     _call("alofa_gemm_swiglu_simple", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(a), _I(dtype_code(a)), _L(_rows("a", a)),
           _ptr(w_gate), _ptr(w_up), _I(dtype_code(w_gate)), _L(_rows("w_gate", w_gate)), _I(M), _I(N), _I(K), _I(int(exact)), _stream())

@@ -113,7 +113,11 @@ class GQAAttention(Mixer):
         return (not self.rt.exact and norm.as_rmsnorm() is not None
                 and ops.can_fuse_norm(rows, self.w_qkv, self.rt.dtype))
 
-    def forward(self, ctx, entry, x, residual, norm=None):
+    @property
+    def gives_normed(self):
+        return self.b_o is None
+
+    def forward(self, ctx, entry, x, residual, norm=None, then=None):
         T = residual.shape[0]
         exact = self.rt.exact
         qkv = ctx.scratch("qkv", (T, self.qkv_width), self.rt.dtype)
@@ -161,8 +165,19 @@ class GQAAttention(Mixer):
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
             ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)
             residual.add_(proj)
-        else:
-            ops.gemm(residual, attn, self.w_o, add_to_out=True, exact=exact)
+        else:      # (then: the norm behind this part, left in the rows given with it)
+            ops.gemm(residual, attn, self.w_o, add_to_out=True, exact=exact, then_norm=_then(then))
+
+
+def _then(then):
+    """(norm, rows) as ``ops.gemm(then_norm=)`` wants it, for norms that are plain RMSNorms; any other norm runs here
+    by itself afterwards, which ``ops.gemm`` cannot do for it: such parts are not asked (``gives_normed`` holds only
+    for RMSNorm in the blocks of this package)."""
+    if then is None:
+        return None
+    norm, rows = then
+    weight, eps = norm.as_rmsnorm()
+    return weight, eps, rows
 
 
 register_part("mixer", "gqa_attention", GQAAttention)

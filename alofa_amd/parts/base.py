@@ -149,6 +149,12 @@ class Mixer(Part):
         says yes is called as ``forward(ctx, where, None, residual, norm=norm)``."""
         return False
 
+    # A part whose last product adds to the residual stream may see to the norm that follows it: the product's
+    # last launch often has whole rows in hand and normalises them on its way out, which saves the norm's own
+    # launch. A part that can sets ``gives_normed``; it is then called with ``then=(norm, rows)`` and leaves
+    # ``norm`` of the residual's new rows in ``rows`` (the activation dtype), however it gets there.
+    gives_normed = False
+
     def forward(self, ctx, where, x: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
 
@@ -160,6 +166,8 @@ class FeedForward(Part):
     def fuses_norm(self, norm, rows: int) -> bool:
         """As for a mixer: yes means ``forward(ctx, None, residual, norm=norm)``."""
         return False
+
+    gives_normed = False      # as for a mixer: ``forward(..., then=(norm, rows))``
 
     def forward(self, ctx, x: torch.Tensor, residual: torch.Tensor) -> None:
         raise NotImplementedError
@@ -200,6 +208,15 @@ class Block(Part):
     def prepare(self, n_positions: int) -> None:
         for m in self.mixers():
             m.prepare(n_positions)
+
+    # The norm a block starts with may be left by whatever ran before it (see ``Mixer.gives_normed``). A block that
+    # takes part sets ``takes_normed``: ``wants_normed(rows)`` names the norm it would like done for a step of so
+    # many rows (or None), ``forward`` takes the rows so normed as ``normed`` and, with ``then=(norm, rows)``,
+    # leaves the next block's. Blocks that know nothing of this take (ctx, entry, hidden) alone.
+    takes_normed = False
+
+    def wants_normed(self, rows: int):
+        return None
 
     def forward(self, ctx, entry: int, hidden: torch.Tensor) -> None:
         raise NotImplementedError

@@ -35,20 +35,38 @@ class PreNormBlock(Block):
     def mixers(self):
         return [self.mixer]
 
-    def forward(self, ctx, entry, hidden):
+    takes_normed = True
+
+    def wants_normed(self, rows):
+        return None if self.mixer.fuses_norm(self.norms[0], rows) else self.norms[0]
+
+    def forward(self, ctx, entry, hidden, normed=None, then=None):
+        """``normed``: the first norm's rows, where the block before has left them; ``then`` = (norm, rows): the norm
+        the next block starts with, to be left in ``rows``. Returns whether that was done."""
         rows = hidden.shape[0]
-        normed = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
-        # a part may take the norm into its first kernel (a launch less where launches are what a step costs)
-        if self.mixer.fuses_norm(self.norms[0], rows):
-            self.mixer.forward(ctx, entry, None, hidden, norm=self.norms[0])
+        buf = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
+        mixer, ff, (n0, n1) = self.mixer, self.feed_forward, self.norms
+        # a norm rides on the first kernel of the part behind it where that can (a launch less where launches are what
+        # a step costs); else the part before it sees to it, whose last launch may have whole rows in hand; else it
+        # is a kernel of its own
+        ff_rides = ff.fuses_norm(n1, rows)
+        more = {"then": (n1, buf)} if not ff_rides and mixer.gives_normed and n1.as_rmsnorm() is not None else {}
+        if normed is not None:
+            mixer.forward(ctx, entry, normed, hidden, **more)
+        elif mixer.fuses_norm(n0, rows):
+            mixer.forward(ctx, entry, None, hidden, norm=n0, **more)
         else:
-            self.norms[0].forward(normed, hidden)
-            self.mixer.forward(ctx, entry, normed, hidden)
-        if self.feed_forward.fuses_norm(self.norms[1], rows):
-            self.feed_forward.forward(ctx, None, hidden, norm=self.norms[1])
+            n0.forward(buf, hidden)
+            mixer.forward(ctx, entry, buf, hidden, **more)
+        given = then is not None and ff.gives_normed
+        more_ff = {"then": then} if given else {}
+        if ff_rides:
+            ff.forward(ctx, None, hidden, norm=n1, **more_ff)
         else:
-            self.norms[1].forward(normed, hidden)
-            self.feed_forward.forward(ctx, normed, hidden)
+            if not more:
+                n1.forward(buf, hidden)
+            ff.forward(ctx, buf, hidden, **more_ff)
+        return given
 
 
 register_part("block", "prenorm", PreNormBlock)

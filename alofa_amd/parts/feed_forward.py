@@ -35,13 +35,19 @@ class SwiGLU(FeedForward):
         return (not self.rt.exact and norm.as_rmsnorm() is not None
                 and ops.can_fuse_norm(rows, self.w_gate, self.rt.dtype, swiglu=True))
 
-    def forward(self, ctx, x, residual, norm=None):
+    gives_normed = True
+
+    def forward(self, ctx, x, residual, norm=None, then=None):
         act = ctx.scratch("ff_act", (residual.shape[0], self.intermediate), self.rt.dtype)
         if norm is not None:      # the norm before the feed-forward rides on the gate/up product
             ops.gemm_swiglu(act, residual, self.w_gate, self.w_up, norm=norm.as_rmsnorm())
         else:
             ops.gemm_swiglu(act, x, self.w_gate, self.w_up, exact=self.rt.exact)
-        ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact)
+        then_norm = None
+        if then is not None:      # the norm behind this part, left in the rows given with it
+            weight, eps = then[0].as_rmsnorm()
+            then_norm = (weight, eps, then[1])
+        ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact, then_norm=then_norm)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

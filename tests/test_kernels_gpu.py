@@ -162,6 +162,38 @@ def test_product_that_takes_the_norm_with_it(M, N, K):
     close(act, pm.swiglu(pm.linear(normed, w), pm.linear(normed, w2)), BF16, "norm + gate/up + swiglu")
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 896, 4864), (200, 896, 4864), (1030, 896, 4864), (2048, 896, 4864), (64, 3584, 3584), (40, 3584, 18944), (17, 1536, 8960),
+                                   (300, 3584, 18944), (64, 896, 896), (2048, 896, 896), (8, 896, 4864), (130, 1000, 3200), (256, 5120, 5120)])
+def test_norm_behind_a_product_that_adds_to_the_residual_stream(M, N, K):
+    """``gemm(..., add_to_out=True, then_norm=)``: the residual stream's new rows and their RMSNorm. Where the product
+    shares K out among blocks and a second launch adds the shares (long K, few tiles), that launch has whole rows in
+    hand and normalises them on its way; everywhere else the norm kernel runs behind the product. Either way the
+    values are those of the product followed by the norm kernel, bit for bit."""
+    o = ops()
+    rng = np.random.default_rng(73)
+    scale = rng.uniform(0.05, 30.0, (M, 1))
+    resid = (rng.standard_normal((M, N)) * scale).astype(np.float32)
+    a = bf((rng.standard_normal((M, K)) * scale).astype(np.float32))
+    w = bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1)
+    nw, eps = (1.0 + 0.3 * rng.standard_normal(N)).astype(np.float32), 1e-5
+    at, wt, nwt = t(a, torch.bfloat16), t(w, torch.bfloat16), t(nw)
+    plain, sep = t(resid), torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    o.gemm(plain, at, wt, add_to_out=True)
+    o.rmsnorm(sep, plain, nwt, eps, False)
+    out, rows = t(resid), torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+    o.gemm(out, at, wt, add_to_out=True, then_norm=(nwt, eps, rows))
+    assert torch.equal(out, plain) and torch.equal(rows, sep)
+    x = resid.astype(np.float64) + a.astype(np.float64) @ w.astype(np.float64).T
+    close(rows, pm.rmsnorm(x.astype(np.float32), nw, eps), BF16, "the norm of the new rows")
+    # float32 rows for the exact path: the norm kernel behind the exact product
+    exact_out, exact_rows = t(resid), torch.empty(M, N, device=DEV)
+    if M <= 300:
+        o.gemm(exact_out, t(a), t(w), add_to_out=True, exact=True, then_norm=(nwt, eps, exact_rows))
+        close(exact_rows, pm.rmsnorm(x.astype(np.float32), nw, eps), 2e-6, "exact")
+    with pytest.raises(AlofaError):
+        o.gemm(torch.empty(M, N, device=DEV, dtype=torch.bfloat16), at, wt, then_norm=(nwt, eps, rows))       # not the residual stream
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 1152, 896), (8, 896, 4864), (3, 97, 80), (7, 1000, 1544), (5, 130, 6144), (2, 64, 8), (4, 4864, 896), (6, 35, 520)])
 def test_product_for_very_few_rows(M, N, K):
     """The vector-unit product for at most eight rows, every form of it (store with bias, float32 store,
