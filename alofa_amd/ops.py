@@ -210,6 +210,17 @@ def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: b
     return "tiled" if elements >= 8 << 20 else "stream"
 
 
+RIDE_ON_SHARES = os.environ.get("ALOFA_RIDE_ON_SHARES", "1") != "0"
+
+
+def norm_rides_on_shares(M: int, N: int, K: int) -> bool:
+    """Whether a product of 17 to 64 rows that adds to the residual stream and has a norm behind it should go to the
+    tiled kernel although the streaming kernel alone would be as fast or a little faster: with K long and the columns
+    few the tiled kernel shares K out and adds the shares in a second launch, which has whole rows in hand and takes
+    the norm with it, and the norm's own launch (some 4.5 us) is saved."""
+    return RIDE_ON_SHARES and 16 < M <= SKINNY_MAX_ROWS and K % 64 == 0 and K >= 3072 and N % 4 == 0 and N <= 4608 and few_rows_kernel(M, N, K) == "stream"
+
+
 def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int, swiglu: bool = False, normed: bool = False) -> str:
     kernel = kernel or few_rows_kernel(M, w_rows, K, swiglu, normed)
     if kernel == "stream" and M <= SKINNY_MAX_ROWS:
@@ -325,6 +336,8 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, bias: Optional[tor
         raise AlofaError("unsupported", "a product that adds to the residual stream takes no bias; add the bias in a buffer of its own")
     if not exact and _mfma_operands(a, w):
         _ensure_workspace(a.device)
+        if kernel is None and then_rows is not None and then_rows.dtype is torch.bfloat16 and FUSE_NORMS and norm_rides_on_shares(M, N, K):
+            kernel = "tiled"
         entry = _product_entry(kernel, M, N, K)
         done = _I(0)
         if entry == "alofa_gemm_mfma":

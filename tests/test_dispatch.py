@@ -39,6 +39,15 @@ def test_product_kernel_by_shape():
         ops._product_entry("fast", 4, 64, 64)
 
 
+def test_a_norm_behind_a_product_moves_it_to_the_kernel_that_adds_shares():
+    # 17 to 64 rows, a long K, few columns: the tiled kernel's second launch takes the norm with it (the 0.5B down projection)
+    assert ops.norm_rides_on_shares(17, 896, 4864) and ops.norm_rides_on_shares(64, 896, 4864)
+    assert not ops.norm_rides_on_shares(16, 896, 4864) and not ops.norm_rides_on_shares(65, 896, 4864)      # the norm rides elsewhere / all is tiled anyway
+    assert not ops.norm_rides_on_shares(32, 896, 896)              # a short K is not shared out
+    assert not ops.norm_rides_on_shares(32, 3584, 18944)           # tiled already (and shared out): nothing to move
+    assert not ops.norm_rides_on_shares(32, 8192, 4096)            # too many columns for the launch that adds shares
+
+
 def test_decode_splits_follow_the_context(monkeypatch):
     monkeypatch.setattr(ops, "_compute_units", 256)                                # the rule counts the chip's compute units: an MI355X's here
     assert ops.decode_splits(8, 14, 2, 64, 512) == 1                              # the waves of one block cover two steps each
