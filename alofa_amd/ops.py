@@ -88,10 +88,15 @@ class stream_scope:
         return False
 
 
+_entries: dict = {}      # the library's entry points by name (looked up once: a step makes some two hundred calls)
+
+
 def _call(fn_name: str, *args) -> None:
-    lib = load()
-    if getattr(lib, fn_name)(*args) != 0:
-        raise AlofaError("invalid_argument", "kernel refused its arguments", lib.alofa_last_error().decode())
+    fn = _entries.get(fn_name)
+    if fn is None:
+        fn = _entries[fn_name] = getattr(load(), fn_name)
+    if fn(*args) != 0:
+        raise AlofaError("invalid_argument", "kernel refused its arguments", load().alofa_last_error().decode())
 
 
 def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
@@ -158,6 +163,20 @@ USE_ROWS_KERNEL = os.environ.get("ALOFA_ROWS_KERNEL", "1") != "0"
 
 
 def few_rows_kernel(M: int, w_rows: int, K: int, swiglu: bool = False, normed: bool = False) -> str:
+    """``few_rows_rule``, remembered per shape (every layer of every step asks)."""
+    key = (M, w_rows, K, swiglu, normed, USE_ROWS_KERNEL)
+    chosen = _few_rows_known.get(key)
+    if chosen is None:
+        if len(_few_rows_known) > 1 << 16:
+            _few_rows_known.clear()
+        chosen = _few_rows_known[key] = few_rows_rule(M, w_rows, K, swiglu, normed)
+    return chosen
+
+
+_few_rows_known: dict = {}
+
+
+def few_rows_rule(M: int, w_rows: int, K: int, swiglu: bool = False, normed: bool = False) -> str:
     """Which bfloat16 product takes ``M`` rows against ``w_rows`` rows of weights
     (gate and up together for the fused feed-forward entry): ``"rows"``, the
     vector-unit kernel for at most eight rows, whose blocks own four or eight
@@ -405,8 +424,23 @@ def check_cache(name: str, cache: torch.Tensor, kv_heads: int, d: int, transpose
     return bs
 
 
+_checked_caches: dict = {}      # id(key cache) -> (key cache, value cache, kv_heads, d, block size): what has been checked already
+
+
 def check_caches(k_cache: torch.Tensor, v_cache: torch.Tensor, kv_heads: int, d: int) -> int:
-    """Key cache and (transposed) value cache of one layer; returns block_size."""
+    """Key cache and (transposed) value cache of one layer; returns block_size. (A layer's caches are the same
+    two tensors step after step, and three kernels a layer ask: what has been checked is remembered by object.)"""
+    known = _checked_caches.get(id(k_cache))
+    if known is not None and known[0] is k_cache and known[1] is v_cache and known[2] == kv_heads and known[3] == d:
+        return known[4]
+    bs = _check_caches(k_cache, v_cache, kv_heads, d)
+    if len(_checked_caches) > 4096:
+        _checked_caches.clear()
+    _checked_caches[id(k_cache)] = (k_cache, v_cache, kv_heads, d, bs)
+    return bs
+
+
+def _check_caches(k_cache: torch.Tensor, v_cache: torch.Tensor, kv_heads: int, d: int) -> int:
     bs = check_cache("k_cache", k_cache, kv_heads, d)
     if check_cache("v_cache", v_cache, kv_heads, d, transposed=True) != bs or k_cache.shape[0] != v_cache.shape[0] or k_cache.dtype is not v_cache.dtype:
         raise AlofaError("shape_mismatch", "key and value caches must agree in blocks, block size and dtype",
@@ -473,6 +507,20 @@ def decode_splits(tokens: int, heads: int, kv_heads: int, d: int, max_context: i
     keys 9.2 with four against 11.9.)"""
     if FORCED_DECODE_PARTS:
         return FORCED_DECODE_PARTS
+    key = (tokens, heads, kv_heads, d, max_context, compute_units())
+    known = _decode_splits_known.get(key)
+    if known is None:
+        if len(_decode_splits_known) > 1 << 16:
+            _decode_splits_known.clear()
+        known = _decode_splits_known[key] = _decode_splits_rule(tokens, heads, kv_heads, d, max_context)
+    return known
+
+
+_decode_splits_known: dict = {}
+_hand_over_known: dict = {}
+
+
+def _decode_splits_rule(tokens: int, heads: int, kv_heads: int, d: int, max_context: int) -> int:
     waves = decode_waves(d)
     step = 32 * waves
     if max_context <= 2 * step:
@@ -498,8 +546,14 @@ def decode_hand_over(tokens: int, heads: int, kv_heads: int, d: int, n_splits: i
     second kernel."""
     if n_splits <= 1 or n_splits > HAND_OVER_MAX_PARTS:
         return False
-    _ensure_workspace(None)
-    return bool(load().alofa_attention_decode_can_hand_over(_I(tokens), _I(heads), _I(kv_heads), _I(d), _I(n_splits)))
+    key = (tokens, heads, kv_heads, d, n_splits)
+    known = _hand_over_known.get(key)
+    if known is None:      # (what fits the workspace does not change once it is there)
+        _ensure_workspace(None)
+        if len(_hand_over_known) > 1 << 16:
+            _hand_over_known.clear()
+        known = _hand_over_known[key] = bool(load().alofa_attention_decode_can_hand_over(_I(tokens), _I(heads), _I(kv_heads), _I(d), _I(n_splits)))
+    return known
 
 
 def decode_scratch_floats(tokens: int, heads: int, kv_heads: int, d: int, max_context: int, window: Optional[int]) -> int:

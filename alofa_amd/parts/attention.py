@@ -101,7 +101,9 @@ class GQAAttention(Mixer):
         # float32 1 / sqrt(float32 d), as the reference forms it (scalar.mojo:421)
         self.scale = float(np.float32(1.0) / np.sqrt(np.float32(self.d)))
         self.qkv_width = (self.heads + 2 * self.kv_heads) * self.d
-        self.capturable = self.position.table(1) is not None   # an encoding applied by other code is not captured
+        # an encoding applied by other code (``apply``) is captured only if it says that it may be: native kernels or
+        # library calls on the current stream that allocate nothing and record no memset
+        self.capturable = self.position.table(1) is not None or bool(getattr(self.position, "capturable", False))
 
     def cache_need(self):
         return CacheNeed.keys_and_values(self.kv_heads, self.d, self.window)

@@ -236,6 +236,7 @@ class Norm(Part):
 
 class PositionEncoding(Part):
     family = "position"
+    capturable = False      # for encodings that give no table: True if ``apply`` may run inside a captured decode step
 
     def table(self, n_positions: int):
         """(cos, sin) float32 [n_positions, d/2] on the device for encodings that
