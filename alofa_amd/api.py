@@ -30,11 +30,15 @@ class Engine:
     def __init__(self, model_dir, dtype: str = "bfloat16", max_tokens: int = 256, max_batch: int = 8,
                  kv_blocks: Optional[int] = None, block_size: int = 16, token_budget: int = 2048, max_chunk: Optional[int] = None,
                  watermark_permille: int = 900, max_wait_ticks: int = 8, seed: int = 1234, device: str = "cuda:0",
-                 trace_path=None, share_prefixes: bool = False, model=None, report=None, run_ahead: bool = True):
+                 trace_path=None, share_prefixes: bool = False, model=None, report=None, run_ahead: bool = True,
+                 memory_fraction: Optional[float] = None):
         """``model``: a (config, Model) pair already on the device, instead of a folder to load.
         ``report``: a callable that receives one line about device memory at start (default:
         standard error when ALOFA_REPORT_MEMORY is set). ``run_ahead``: a tick reads the tokens of the
         tick before only after its own step is launched (``EngineCore``); off, every tick is synchronous.
+        ``memory_fraction`` (with no ``kv_blocks``): the pool of the layers that keep every key takes this share
+        of the device memory that is free once the weights are loaded (less what the windowed layers' pools take),
+        instead of what ``max_batch`` requests of ``max_tokens`` need.
         ``max_chunk``: the most prompt tokens of one request in a tick; by default the whole ``token_budget``,
         so that a lone long prompt takes one step (requests are served in order of arrival either way, and the
         budget alone bounds a tick's length)."""
@@ -50,6 +54,8 @@ class Engine:
                 return (pages * 1000 + watermark_permille - 1) // watermark_permille + 1
             own = {w: under_watermark(CacheManager.pages_for(w, max_batch, max_tokens, max_chunk, block_size))
                    for w in CacheManager.windows_of(needs)}
+            if kv_blocks is None and memory_fraction is not None:
+                kv_blocks = self._pages_that_fit(needs, own, memory_fraction, block_size)
             kv_blocks = {w: n if kv_blocks is None else (int(kv_blocks) if w is None else min(int(kv_blocks), n)) for w, n in own.items()}
         self.cache = CacheManager(needs, self.model.state_needs(), kv_blocks, block_size,
                                   max_requests=max(32, max_batch), device=self.model.rt.device, dtype=self.model.rt.dtype)
@@ -69,6 +75,20 @@ class Engine:
             report(f"[alofa_amd] device memory: weights {m['weights'] / 2**20:.1f} MiB + cache pool {m['cache_pool'] / 2**20:.1f} MiB "
                    f"({' + '.join(str(g.pool.n_blocks) for g in self.cache.groups) or 0} pages of {block_size} tokens in {len(self.cache.groups)} group(s)) + scratch {m['scratch'] / 2**20:.1f} MiB "
                    f"(grows to the largest step, then stays) = {m['total'] / 2**20:.1f} MiB")
+
+    def _pages_that_fit(self, needs, own: dict, fraction: float, block_size: int) -> int:
+        """Pages for the pool of the layers that keep every key: what ``fraction`` of the free device memory holds
+        beside the windowed layers' pools (sized by their windows: ``own``)."""
+        import torch
+        if not 0.0 < fraction <= 1.0:
+            raise AlofaError("invalid_argument", "memory_fraction lies in (0, 1]", f"memory_fraction={fraction}")
+        per_page = CacheManager.page_bytes(needs, block_size, self.model.rt.dtype)
+        free = torch.cuda.mem_get_info(self.model.rt.device)[0]
+        left = int(free * fraction) - sum(own[w] * b for w, b in per_page.items() if w is not None)
+        pages = left // per_page[None] if None in per_page else 1
+        if pages <= 0:
+            raise AlofaError("capacity", "the cache pool does not fit the device memory that is free", f"free={free} fraction={fraction}")
+        return int(min(pages, (1 << 31) - 1))
 
     def memory(self) -> dict:
         """Bytes of device memory by use: the rule is weights + cache pool + scratch, nothing else

@@ -85,6 +85,21 @@ class CacheManager:
         held = CacheManager.held_tokens_of(window, step_tokens, block_size)
         return max(1, requests * blocks_for(tokens if held < 0 else min(tokens, held), block_size))
 
+    @staticmethod
+    def page_bytes(cache_needs, block_size: int, dtype=torch.bfloat16) -> dict:
+        """Bytes that one page of every group takes on the device, summed over the group's mixers and their tensors:
+        {window: bytes}."""
+        out: dict = {}
+        for need in _keyed(cache_needs).values():
+            n = 0
+            for t in need.tensors:
+                count = 1
+                for d in t.page_shape(block_size):
+                    count *= d
+                n += count * torch.empty((), dtype=t.dtype or dtype).element_size()
+            out[need.window] = out.get(need.window, 0) + n
+        return out
+
     def __init__(self, cache_needs, state_needs, n_blocks, block_size: int = 16,
                  max_requests: int = 64, device=None, dtype=torch.bfloat16):
         if block_size <= 0 or max_requests <= 0:

@@ -13,9 +13,12 @@ and the engine's own:
 
   ALOFA_DTYPE              bfloat16 | float32                   (bfloat16)
   ALOFA_PROMPT_IDS         prompts as token ids, "5,17,3;9,2"   (or the first argument)
+  ALOFA_PROMPT_FILE        a file of such prompts, one a line   (when neither of the two is given)
   ALOFA_MAX_NEW            tokens to generate per prompt        (16)
   ALOFA_TEMPERATURE ALOFA_TOP_K ALOFA_TOP_P ALOFA_MIN_P ALOFA_REPETITION_PENALTY
   ALOFA_FREQUENCY_PENALTY ALOFA_PRESENCE_PENALTY   sampling; temperature 0 = greedy (0)
+  ALOFA_KV_FRACTION        permille of the free device memory for the cache pool, when
+                           ALOFA_KV_BLOCKS is not set                  (0: by ALOFA_BATCH x ALOFA_MAX_TOKENS)
   ALOFA_BLOCK_SIZE ALOFA_KV_BLOCKS ALOFA_TOKEN_BUDGET ALOFA_MAX_CHUNK
   ALOFA_WATERMARK_PERMILLE ALOFA_MAX_WAIT_TICKS   cache and scheduler
   ALOFA_TRACE              file that receives the scheduler trace
@@ -95,7 +98,14 @@ def main(argv=None) -> int:
     if dtype not in ("bfloat16", "float32"):
         raise AlofaError("invalid_argument", "ALOFA_DTYPE is bfloat16 or float32", f"ALOFA_DTYPE={dtype}")
     max_new = env_int("ALOFA_MAX_NEW", 16, 1, 32768)
-    prompts = parse_prompts(argv[0] if argv else env_str("ALOFA_PROMPT_IDS", ""))
+    text = argv[0] if argv else env_str("ALOFA_PROMPT_IDS", "")
+    prompt_file = env_str("ALOFA_PROMPT_FILE", "")
+    if not text and prompt_file:
+        try:
+            text = Path(prompt_file).read_text()
+        except OSError as e:
+            raise AlofaError("io", "cannot read ALOFA_PROMPT_FILE", f"path={prompt_file} reason={e}") from None
+    prompts = parse_prompts(text)
     for p in prompts:
         if len(p) > max_prompt:
             raise AlofaError("out_of_range", "prompt is longer than ALOFA_MAX_PROMPT_TOKENS", f"tokens={len(p)} limit={max_prompt}")
@@ -107,6 +117,7 @@ def main(argv=None) -> int:
         write_random_model(json.loads(Path(random_config).read_text()), weights, seed)
     block = env_int("ALOFA_BLOCK_SIZE", 16, 1, 1024)
     kv_blocks = env_int("ALOFA_KV_BLOCKS", 0, 0, 1 << 30)
+    kv_permille = env_int("ALOFA_KV_FRACTION", 0, 0, 1000)
 
     budget = env_int("ALOFA_TOKEN_BUDGET", 2048, 1, 1 << 20)
     from .api import Engine
@@ -117,6 +128,7 @@ def main(argv=None) -> int:
                     max_wait_ticks=env_int("ALOFA_MAX_WAIT_TICKS", 8, 0, 1 << 20), seed=seed,
                     trace_path=env_str("ALOFA_TRACE", "") or None,
                     share_prefixes=bool(env_int("ALOFA_SHARE_PREFIX", 0, 0, 1)),
+                    memory_fraction=kv_permille / 1000.0 if kv_permille and not kv_blocks else None,
                     report=lambda line: print(line, file=sys.stderr, flush=True))
     outs = engine.generate(prompts, max_new=max_new,
                            temperature=env_float("ALOFA_TEMPERATURE", 0.0, 0.0, 1e6),

@@ -125,6 +125,35 @@ def test_random_model_round_trip(tmp_path):
     assert "lm_head.weight" not in wa and all(t.dtype is torch.float32 for t in wa.values())   # 32-bit stays 32-bit
 
 
+def test_checkpoint_in_several_files(tmp_path):
+    """model.safetensors.index.json names the file of every tensor (larger checkpoints come so): the same tensors, the
+    same one error for what is missing, and named errors for an index that is wrong."""
+    import json
+    cfg = config_from_dict(TINY["B"])
+    exp = expected_tensors(cfg.spec())
+    t = random_tensors(exp, 5)
+    names = list(t)
+    shards = {"model-00001-of-00003.safetensors": names[:7], "model-00002-of-00003.safetensors": names[7:20], "model-00003-of-00003.safetensors": names[20:]}
+    for file_name, part in shards.items():
+        write_safetensors(tmp_path / file_name, {n: t[n] for n in part})
+    index = {"metadata": {"total_size": 0}, "weight_map": {n: f for f, part in shards.items() for n in part}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    w = load_weights(tmp_path, exp)
+    assert set(w) == set(t) and all(torch.equal(w[n], t[n]) for n in t)
+    # a tensor the index leaves out is missing like any other
+    short = dict(index, weight_map={n: f for n, f in index["weight_map"].items() if n != "model.norm.weight"})
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(short))
+    with pytest.raises(AlofaError) as e:
+        load_weights(tmp_path, exp)
+    assert "missing: model.norm.weight" in str(e.value)
+    for bad, name in (({"weight_map": {"x": "../elsewhere.safetensors"}}, "invalid_argument"), ({"weight_map": {"x": "none.safetensors"}}, "io"),
+                      ({"weight_map": {"model.norm.weight": "model-00001-of-00003.safetensors"}}, "invalid_argument"), ({"weights": {}}, "parse")):
+        (tmp_path / "model.safetensors.index.json").write_text(json.dumps(bad))
+        assert err_name(load_weights, tmp_path, exp) == name
+    (tmp_path / "model.safetensors.index.json").unlink()
+    assert err_name(load_weights, tmp_path, exp) == "io"                 # neither one file nor an index
+
+
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     cfg = config_from_dict(TINY["A"])
     exp = expected_tensors(cfg.spec())

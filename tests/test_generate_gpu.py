@@ -497,6 +497,17 @@ def test_generate_command(tiny_dirs, tmp_path):
     for key, val in (("ALOFA_MAX_TOKENS", "lots"), ("ALOFA_MAX_TOKENS", "0"), ("ALOFA_DTYPE", "fp8"), ("ALOFA_MAX_PROMPT_TOKENS", "3")):
         bad = subprocess.run([str(ROOT / "bin" / "generate")], env=dict(env, **{key: val}), capture_output=True, text=True, timeout=300)
         assert bad.returncode != 0 and key in bad.stderr, (key, bad.stderr[-500:])
+    # prompts from a file, and a cache pool sized by a share of the free device memory
+    (tmp_path / "prompts.txt").write_text("\n".join(",".join(map(str, p)) for p in prompts) + "\n")
+    env3 = {k: v for k, v in env.items() if k != "ALOFA_PROMPT_IDS"}
+    p = subprocess.run([str(ROOT / "bin" / "generate")], env=dict(env3, ALOFA_PROMPT_FILE=str(tmp_path / "prompts.txt"), ALOFA_KV_FRACTION="1"),
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [[int(t) for t in line.split(",")] for line in p.stdout.strip().splitlines()] == want
+    pages = int(p.stderr.split("cache pool")[1].split("(")[1].split(" pages")[0])
+    assert pages > 1000, p.stderr[-500:]                  # a thousandth of the free memory is far more than 8 x 64 tokens take
+    bad = subprocess.run([str(ROOT / "bin" / "generate")], env=dict(env3, ALOFA_PROMPT_FILE=str(tmp_path / "none.txt")), capture_output=True, text=True, timeout=300)
+    assert bad.returncode != 0 and "ALOFA_PROMPT_FILE" in bad.stderr
     # random weights from a configuration and a seed
     cfgp = tmp_path / "cfg.json"
     import json
@@ -504,6 +515,27 @@ def test_generate_command(tiny_dirs, tmp_path):
     env2 = dict(os.environ, ALOFA_WEIGHTS=str(tmp_path / "made"), ALOFA_RANDOM_CONFIG=str(cfgp), ALOFA_SEED="5", ALOFA_MAX_NEW="3", ALOFA_MAX_TOKENS="64")
     p = subprocess.run([str(ROOT / "bin" / "generate"), "5,6,7"], env=env2, capture_output=True, text=True, timeout=300)
     assert p.returncode == 0 and (tmp_path / "made" / "model.safetensors").exists() and len(p.stdout.strip().split(",")) == 3
+
+
+def test_pool_sized_by_a_share_of_the_free_memory(tiny_dirs):
+    """``memory_fraction``: the layers that keep every key get what that share of the free device memory holds beside
+    the windowed layers' pools, which stay at what their windows need."""
+    import torch
+    from alofa_amd import Engine
+    from alofa_amd.cache.manager import CacheManager
+    from alofa_amd.errors import AlofaError
+    free = torch.cuda.mem_get_info()[0]
+    eng = Engine(tiny_dirs["C"], dtype="bfloat16", max_tokens=256, max_batch=4, memory_fraction=0.002)
+    full, windowed = eng.cache.groups
+    per_page = CacheManager.page_bytes(eng.model.cache_needs(), 16, torch.bfloat16)
+    assert per_page == {None: 2 * 5 * 16 * 48 * 2, 40: 3 * 2 * 5 * 16 * 48 * 2}
+    by_window = Engine(tiny_dirs["C"], dtype="bfloat16", max_tokens=256, max_batch=4)
+    assert windowed.pool.n_blocks == by_window.cache.groups[1].pool.n_blocks
+    want = (0.002 * free - windowed.pool.n_blocks * per_page[40]) / per_page[None]
+    assert 0.9 * want <= full.pool.n_blocks <= 1.02 * want and full.pool.n_blocks > by_window.cache.groups[0].pool.n_blocks
+    assert eng.generate([random_ids(1, 30, 331)], max_new=5) == by_window.generate([random_ids(1, 30, 331)], max_new=5)
+    with pytest.raises(AlofaError):
+        Engine(tiny_dirs["C"], dtype="bfloat16", max_tokens=256, memory_fraction=1.5)
 
 
 def test_a_lone_prompt_is_one_step_by_default(tiny_dirs):
