@@ -632,34 +632,51 @@ constexpr ThenNorm kNoNorm = {nullptr, 0.f, nullptr, 0};
 // The shares added to the residual stream as in split_sum_kernel, by a block per row that keeps the row in registers
 // (K4 groups of four columns a thread) and goes on to normalise it: the sums, the threads' places and the arithmetic
 // are those of split_sum_kernel followed by rmsnorm_kernel (elementwise.hip), value for value, without the second
-// launch and its trip through memory.
+// launch and its trip through memory. Everything a thread reads for up to four of its groups is asked for at once
+// (every thread issues every load, from the row's last group where its own lies past the end, and from the last
+// share where there are fewer than eight): the shares come from memory, and a thread that took its groups one
+// after the other would wait a memory latency for each (7B sizes, 64 rows of 3,584: the loop cost more than the
+// norm's own launch saves).
 template <int K4>
 __global__ void __launch_bounds__(256) split_sum_norm_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ parts, int shares,
                                                              int M, int N, ThenNorm then) {
   __shared__ float scratch[4];
+  constexpr int kTogether = K4 < 4 ? K4 : 4;
   const int m = blockIdx.x, groups = N / 4;
   const int64_t part = static_cast<int64_t>(M) * N;
   float4 xs[K4], ws[K4];
 #pragma unroll
-  for (int i = 0; i < K4; ++i) {
-    const int g = threadIdx.x + 256 * i;
-    xs[i] = ws[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (g < groups) {     // uniform but for the row's last threads
-      const float* src = parts + static_cast<int64_t>(m) * N + 4 * g;
-      float* dst = out + static_cast<int64_t>(m) * ldo + 4 * g;
-      const float4 old = *reinterpret_cast<const float4*>(dst);
-      ws[i] = reinterpret_cast<const float4*>(then.weight)[g];
-      float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-      for (int s0 = 0; s0 < shares; s0 += 8) {     // (eight parts' loads on their way together)
-        float4 v[8];
+  for (int i0 = 0; i0 < K4; i0 += kTogether) {
+    float4 old[kTogether], v[kTogether][8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(src + min(s0 + u, shares - 1) * part);
+    for (int j = 0; j < kTogether; ++j) {
+      const int g = threadIdx.x + 256 * (i0 + j), gc = g < groups ? g : groups - 1;
+      const float* src = parts + static_cast<int64_t>(m) * N + 4 * gc;
+      old[j] = *reinterpret_cast<const float4*>(out + static_cast<int64_t>(m) * ldo + 4 * gc);
+      ws[i0 + j] = reinterpret_cast<const float4*>(then.weight)[gc];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[j][u] = *reinterpret_cast<const float4*>(src + min(u, shares - 1) * part);
+    }
+#pragma unroll
+    for (int j = 0; j < kTogether; ++j) {
+      const int g = threadIdx.x + 256 * (i0 + j), gc = g < groups ? g : groups - 1;
+      float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (u < shares) { sum.x += v[j][u].x; sum.y += v[j][u].y; sum.z += v[j][u].z; sum.w += v[j][u].w; }
+      for (int s0 = 8; s0 < shares; s0 += 8) {     // (more than eight shares: the next eight, together again)
+        const float* src = parts + static_cast<int64_t>(m) * N + 4 * gc;
+        float4 more[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) more[u] = *reinterpret_cast<const float4*>(src + min(s0 + u, shares - 1) * part);
 #pragma unroll
         for (int u = 0; u < 8; ++u)
-          if (s0 + u < shares) { sum.x += v[u].x; sum.y += v[u].y; sum.z += v[u].z; sum.w += v[u].w; }
+          if (s0 + u < shares) { sum.x += more[u].x; sum.y += more[u].y; sum.z += more[u].z; sum.w += more[u].w; }
       }
-      xs[i] = make_float4(old.x + sum.x, old.y + sum.y, old.z + sum.z, old.w + sum.w);
-      *reinterpret_cast<float4*>(dst) = xs[i];
+      const bool mine = g < groups;
+      xs[i0 + j] = mine ? make_float4(old[j].x + sum.x, old[j].y + sum.y, old[j].z + sum.z, old[j].w + sum.w) : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (!mine) ws[i0 + j] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (mine) *reinterpret_cast<float4*>(out + static_cast<int64_t>(m) * ldo + 4 * g) = xs[i0 + j];
     }
   }
   float ss = 0.f;
