@@ -26,7 +26,6 @@ import torch
 
 from ..config.base import PartSpec
 from ..errors import AlofaError
-from ..weights.loader import TensorRule
 
 FAMILIES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head")
 _REGISTRY = {f: {} for f in FAMILIES}

@@ -9,8 +9,6 @@ from __future__ import annotations
 from dataclasses import dataclass
 from pathlib import Path
 
-import torch
-
 from ..errors import AlofaError
 from .safetensors_io import SafeTensorFile
 

@@ -4,13 +4,12 @@ logits at every position."""
 import json
 import os
 import subprocess
-import sys
 
 import numpy as np
 import pytest
 
 from conftest import ROOT, TINY
-from helpers import (assert_close, bound, bulk_and_tail, collect, mixed, plain_logits, portions, random_ids, round64, whole)
+from helpers import (assert_close, bulk_and_tail, collect, mixed, plain_logits, portions, random_ids, round64, whole)
 
 pytestmark = pytest.mark.gpu
 

@@ -3,7 +3,6 @@ step function, choice and settle together, against the plain implementation."""
 import os
 import subprocess
 
-import numpy as np
 import pytest
 import torch
 
