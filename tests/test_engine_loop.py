@@ -34,13 +34,13 @@ class AccountingStep:
         self.rows += int(n_tokens.sum())
 
 
-def engine(windows, pools, bs, max_chunk, budget, n_positions, watermark=900, requests=8):
+def engine(windows, pools, bs, max_chunk, budget, n_positions, watermark=900, requests=8, share=False):
     needs = [CacheNeed.keys_and_values(2, 16, w) for w in windows]
     cache = CacheManager(needs, [None] * len(needs), pools, bs, max_requests=requests)
     step = AccountingStep(cache, n_positions)
     cfg = SchedConfig.for_groups(cache.group_rules(max_chunk), token_budget=budget, max_chunk=max_chunk, block_size=bs,
                                  watermark_permille=watermark, max_wait_ticks=4, n_slots=requests)
-    return EngineCore(step, cfg, run_ahead=False), step, cache
+    return EngineCore(step, cfg, run_ahead=False, share_prefixes=share), step, cache
 
 
 def tick(core, step):
@@ -66,7 +66,11 @@ CASES = {
 @pytest.mark.parametrize("case", list(CASES))
 def test_random_traffic_never_asks_the_pools_for_more_than_they_hold(case, seed):
     windows, pools, bs, max_chunk, budget, n_positions = CASES[case]
-    core, step, cache = engine(windows, pools, bs, max_chunk, budget, n_positions)
+    # (every other seed: requests start on the pages of running requests whose prompts begin alike; the prompts
+    # below begin with one of three openings, so that there is something to share)
+    share = seed % 2 == 1
+    core, step, cache = engine(windows, pools, bs, max_chunk, budget, n_positions, share=share)
+    openings = [[7 + o] * 64 for o in range(3)]
     cfg = core.sched.cfg
     rnd = random.Random(1000 * seed + len(case))
     # what one request may ask for: the scheduler refuses by name what could never fit under the watermark
@@ -78,6 +82,9 @@ def test_random_traffic_never_asks_the_pools_for_more_than_they_hold(case, seed)
             total = rnd.randint(2, max(2, most // rnd.choice([1, 2, 3])))
             max_new = rnd.randint(1, max(1, min(40, total - 1)))
             prompt = [rnd.randrange(1000) for _ in range(total - max_new)]
+            if share:
+                opening = rnd.choice(openings)[:rnd.randint(0, len(prompt))]
+                prompt[:len(opening)] = opening
             if core.can_admit(len(prompt), max_new):     # (as the entry point does: what the watermark cannot hold yet waits outside)
                 core.submit(next_id, prompt, max_new)
                 asked[next_id] = max_new
@@ -124,6 +131,7 @@ def test_random_traffic_never_asks_the_pools_for_more_than_they_hold(case, seed)
     assert all(core.sched.of_group("blocks_used", g) == 0 for g in range(len(cache.groups)))
     assert core.sched.n_live() == 0
     assert len(asked) > 20 and step.rows > 1000
+    assert (core.shared_tokens > 0) == (share and all(w is None for w in windows))      # (a model with a group that sees a window shares nothing)
     # the pools were small enough to matter: some group was filled past half, and arrivals were turned away for a while
     assert max(p / g.pool.n_blocks for p, g in zip(peak, cache.groups)) > 0.5 and turned_away > 0 and preempted > 0
 
