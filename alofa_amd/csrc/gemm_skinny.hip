@@ -65,10 +65,14 @@ __device__ __forceinline__ void load_raw(RawNormed& dst, const void* row, int k,
     dst.hi = *reinterpret_cast<const float4*>(p + 4);
   }
 }
-// x * w rounded to bfloat16; the squares of x join the row's sum
+// the sum of four squares, in one fixed order of multiply-adds (both forms of the norm below add the same numbers alike)
+__device__ __forceinline__ float squares4(float4 x) {
+  return __builtin_fmaf(x.w, x.w, __builtin_fmaf(x.z, x.z, __builtin_fmaf(x.y, x.y, x.x * x.x)));
+}
+// x * w rounded to bfloat16; the squares of x join the row's sum, four and four
 __device__ __forceinline__ bf16x8 to_frag(const RawNormed& x, const RawNormed& w, float& ss) {
-  ss += x.lo.x * x.lo.x + x.lo.y * x.lo.y + x.lo.z * x.lo.z + x.lo.w * x.lo.w;
-  ss += x.hi.x * x.hi.x + x.hi.y * x.hi.y + x.hi.z * x.hi.z + x.hi.w * x.hi.w;
+  ss += squares4(x.lo);
+  ss += squares4(x.hi);
   const uint4 v = make_uint4(pack_bf16x2(x.lo.x * w.lo.x, x.lo.y * w.lo.y), pack_bf16x2(x.lo.z * w.lo.z, x.lo.w * w.lo.w),
                              pack_bf16x2(x.hi.x * w.hi.x, x.hi.y * w.hi.y), pack_bf16x2(x.hi.z * w.hi.z, x.hi.w * w.hi.w));
   return __builtin_bit_cast(bf16x8, v);
@@ -78,13 +82,19 @@ __device__ __forceinline__ bf16x8 to_frag(const RawNormed& x, const RawNormed& w
 // gate matrix, tile 1 the up matrix, same columns); TO: float or bf16_t.
 // kUnroll: steps of 32 along K whose loads are in flight together (twice that with the prefetch).
 // kNorm: A is float [M, K] and out = epilogue(rmsnorm(A, norm_w, eps) W^T) (no split of K over blocks then).
-template <int MT, int NT, int kWaves, int kEpilogue, typename TO, int kUnroll, bool kNorm>
+// kNorm == 2: the same for at most eight rows. A lane's eight values of a step are then fetched by two lanes, four each
+// (lane r < 8 of a row of 16 lanes the first four of row r, lane r + 8 the other four), multiplied by the norm's
+// weights and rounded there, and the halves meet by a lane move: with eight rows the plain form leaves half the lanes
+// of every fetch of A idle, and a fetch costs the memory pipeline the same whatever its lanes bring (gate and up
+// against eight rows of 896: 8.3 against 9.3 us).
+template <int MT, int NT, int kWaves, int kEpilogue, typename TO, int kUnroll, int kNorm>
 __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     TO* __restrict__ out, int64_t ldo, const void* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
     const bf16_t* __restrict__ W2, int64_t ldw, const float* __restrict__ bias, int M, int N, int K,
     f32x4* __restrict__ ws, int* __restrict__ counters, const float* __restrict__ norm_w, float eps) {
   __shared__ f32x4 red[kWaves][MT * NT][64];
   __shared__ float ssq[kNorm ? kWaves : 1][MT][16];
+  constexpr bool kHalf = kNorm == 2;
   __shared__ int last_block;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int r = lane % 16, g = lane / 16;
@@ -183,6 +193,10 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     // both sets' weights and rows, then the norm's weights, which all waves share through LDS.
     static_assert(!kNorm || MT == 1, "the norm rides on products of at most 16 rows");
     extern __shared__ __attribute__((aligned(16))) float norm_lds[];      // K floats
+    // (kHalf: this lane's row of A is r % 8, and of a step's eight values it fetches those from half_off on)
+    const int half_off = kHalf ? (r >> 3) * 4 : 0;
+    const bool half_ok = (r & 7) < M;
+    const float* half_row = static_cast<const float*>(A) + static_cast<int64_t>(half_ok ? (r & 7) : 0) * lda;
     RawNormed ra0[kUnroll], ra1[kUnroll];
     bf16x8 w0[kUnroll][NT], w1[kUnroll][NT];
     auto issue = [&](RawNormed (&ra)[kUnroll], bf16x8 (&w)[kUnroll][NT], int first) {
@@ -192,7 +206,12 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
         const bool k_ok = k < K && first + u * kWaves < n_steps;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) w[u][nt] = load_frag(w_row[nt] + k, k_ok && w_ok[nt]);
-        load_raw(ra[u], a_row[0], k, k_ok && a_ok[0]);
+        if constexpr (kHalf) {
+          ra[u].lo = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (k_ok && half_ok) ra[u].lo = *reinterpret_cast<const float4*>(half_row + k + half_off);
+        } else {
+          load_raw(ra[u], a_row[0], k, k_ok && a_ok[0]);
+        }
       }
     };
     auto multiply = [&](RawNormed (&ra)[kUnroll], bf16x8 (&w)[kUnroll][NT], int first) {
@@ -200,8 +219,21 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
       for (int u = 0; u < kUnroll; ++u) {
         int k = (first + u * kWaves) * 32 + g * 8;
         k = k < K ? k : 0;                   // (a step past the end holds zeros: any weights will do)
-        const RawNormed nw{*reinterpret_cast<const float4*>(norm_lds + k), *reinterpret_cast<const float4*>(norm_lds + k + 4)};
-        const bf16x8 a = to_frag(ra[u], nw, ss[0]);
+        bf16x8 a;
+        if constexpr (kHalf) {
+          const float4 x = ra[u].lo, nw = *reinterpret_cast<const float4*>(norm_lds + k + half_off);
+          // (the squares of a row's eight values join its sum four and four, in lane r as in the plain form)
+          const float sq = squares4(x), sq_other = lane_xor8(sq);
+          if (r < 8) { ss[0] += sq; ss[0] += sq_other; }
+          const uint32_t p0 = pack_bf16x2(x.x * nw.x, x.y * nw.y), p1 = pack_bf16x2(x.z * nw.z, x.w * nw.w);
+          // the other four values of lane r's eight come from lane r + 8 (row_ror:8: every lane reads the lane eight on in its row of 16)
+          const uint32_t q0 = __builtin_amdgcn_update_dpp(0u, p0, 0x128, 0xf, 0xf, false), q1 = __builtin_amdgcn_update_dpp(0u, p1, 0x128, 0xf, 0xf, false);
+          const uint4 v = r < 8 ? make_uint4(p0, p1, q0, q1) : make_uint4(0, 0, 0, 0);      // (rows 8 to 15 of the tile do not exist)
+          a = __builtin_bit_cast(bf16x8, v);
+        } else {
+          const RawNormed nw{*reinterpret_cast<const float4*>(norm_lds + k), *reinterpret_cast<const float4*>(norm_lds + k + 4)};
+          a = to_frag(ra[u], nw, ss[0]);
+        }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[0][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, w[u][nt], acc[0][nt], 0, 0, 0);
       }
@@ -229,7 +261,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     // the four lanes that hold slices of one row meet; the waves' shares of a row are added in wave order below
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      const float row_ss = rows_sum(ss[mt]);
+      const float row_ss = rows_sum(ss[mt]);      // (kHalf: lanes 8 to 15 of a row of lanes hold nothing, and stand for rows that do not exist)
       if (g == 0) ssq[wave][mt][r] = row_ss;
     }
   }
@@ -381,9 +413,14 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
     if (norm.weight != nullptr) {
       // (float rows take twice the registers: two sets of two steps keep two blocks on a compute unit)
       ALOFA_REQUIRE(K % 4 == 0 && K <= kMaxNormK, "gemm_skinny: the norm's weights must fit in LDS [K=%d, at most %d]", K, kMaxNormK);
-      gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, true><<<dim3(col_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
-          static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
-          reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps);
+      if (M <= 8)
+        gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, 2><<<dim3(col_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
+            static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
+            reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps);
+      else
+        gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, 1><<<dim3(col_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
+            static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
+            reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps);
       return check_launch("gemm_skinny (with norm)");
     }
   }
