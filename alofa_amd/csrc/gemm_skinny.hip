@@ -129,6 +129,21 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   // the sums are ready: this wave finishes tiles wave, wave + kWaves, ...
   constexpr int kOutTiles = (kEpilogue == kSkSwiglu) ? MT : MT * NT;
   constexpr int kMyTiles = (kOutTiles + kWaves - 1) / kWaves;
+  // With so few output tiles that they would leave most waves without work at the end (one or two), and K not
+  // shared out over blocks, every thread finishes one output instead (`flat` below): thread x the x-th float of
+  // the tiles as they lie in `red`. What it adds sets out now as well.
+  constexpr bool kFlatTail = kOutTiles * 4 <= kWaves;
+  const bool flat = kFlatTail && gridDim.y == 1;
+  const int f_tile = threadIdx.x >> 8, f_r = (threadIdx.x >> 2) & 15, f_g = (threadIdx.x >> 6) & 3, f_i = threadIdx.x & 3;
+  const int f_mt = (kEpilogue == kSkSwiglu) ? f_tile : f_tile / NT, f_nt = (kEpilogue == kSkSwiglu) ? 0 : f_tile % NT;
+  const int f_m = f_mt * 16 + f_g * 4 + f_i, f_n = (kEpilogue == kSkSwiglu) ? n0 + f_r : n0 + f_nt * 16 + f_r;
+  const bool f_ok = flat && f_tile < kOutTiles && f_m < M && f_n < N;
+  float f_add = 0.f;
+  if (f_ok) {
+    if (kEpilogue == kSkStore && bias) f_add = bias[f_n];
+    if (kEpilogue == kSkResidual) f_add = load_f32(out + static_cast<int64_t>(f_m) * ldo + f_n);
+  }
+
   float add[kMyTiles][4];
 #pragma unroll
   for (int it = 0; it < kMyTiles; ++it) {
@@ -139,7 +154,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     for (int i = 0; i < 4; ++i) {
       const int m = mt * 16 + g * 4 + i;
       add[it][i] = 0.f;
-      if (tile < kOutTiles && n < N && m < M) {
+      if (!flat && tile < kOutTiles && n < N && m < M) {
         if (kEpilogue == kSkStore && bias) add[it][i] = bias[n];
         if (kEpilogue == kSkResidual) add[it][i] = load_f32(out + static_cast<int64_t>(m) * ldo + n);
       }
@@ -266,6 +281,38 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     }
   }
   __syncthreads();
+
+  if (flat) {
+    // one output a thread: the waves' shares in wave order, the same sums and the same arithmetic as below
+    if (!f_ok) return;
+    const float* shares = reinterpret_cast<const float*>(&red[0][0][0]);       // [wave][MT * NT][64 lanes][4]
+    const int at = ((f_mt * NT + f_nt) * 64 + (f_g * 16 + f_r)) * 4 + f_i;
+    float sum = shares[at], up = 0.f;
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) sum += shares[w * (MT * NT * 256) + at];
+    if (kEpilogue == kSkSwiglu) {
+      up = shares[at + 256];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) up += shares[w * (MT * NT * 256) + at + 256];
+    }
+    if constexpr (kNorm) {
+      float total = ssq[0][f_mt][f_g * 4 + f_i];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) total += ssq[w][f_mt][f_g * 4 + f_i];
+      const float factor = __builtin_amdgcn_rsqf(total / static_cast<float>(K) + eps);
+      sum *= factor;
+      up *= factor;
+    }
+    TO* dst = out + static_cast<int64_t>(f_m) * ldo + f_n;
+    if (kEpilogue == kSkStore) {
+      store_f32(dst, sum + f_add);
+    } else if (kEpilogue == kSkResidual) {
+      store_f32(dst, f_add + sum);
+    } else {
+      store_f32(dst, sum / (1.f + __expf(-sum)) * up);
+    }
+    return;
+  }
 
   if (k_splits > 1) {
     // this block's tiles (its waves added in wave order) go to the workspace; the last block to arrive goes on
