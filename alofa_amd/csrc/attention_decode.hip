@@ -206,16 +206,20 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   auto compute = [&](int tile, Step& st) __attribute__((always_inline)) {
     // S^T of the two tiles (channels beyond d, in the last step of 32 of a head size that is no multiple of 32,
     // meet zeros of Q)
+    // Most steps of a long context touch neither end of the visible keys nor the new token: they skip the masks and
+    // the new token's insertion (branches of the whole wave with no loads inside; the results are the same bits).
+    const bool last_here = kRope && tile + 1 >= last;                                                   // the step holds the new token's tile
+    const bool inner = (tile << 4) >= lo && (((tile + 2) << 4) - 1) <= p && tile + 1 < tile_end;        // every key of the step is seen
     f32x4 s[2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
       // (kRope: the new token's key is not in the cache yet: its row of the last tile comes from the registers)
-      const bool new_row = kRope && tile + kt == last && c16 == (p & 15);
+      const bool new_row = last_here && tile + kt == last && c16 == (p & 15);
 #pragma unroll
       for (int ds = 0; ds < DS; ++ds) {
         uint4 kf = st.k[kt][ds];
-        if constexpr (kRope) {      // (word by word: a choice between two whole operands would be made through memory)
+        if (last_here) {      // (word by word: a choice between two whole operands would be made through memory)
           kf.x = new_row ? new_k[ds].x : kf.x;
           kf.y = new_row ? new_k[ds].y : kf.y;
           kf.z = new_row ? new_k[ds].z : kf.z;
@@ -227,12 +231,20 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     // scale, mask, running maximum; the four lanes of a head agree on the maximum
     float pw[8];
     float step_max = -FLT_MAX;
+    if (inner) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int key = ((tile + i / 4) << 4) + 4 * g + i % 4;
-      const bool seen = key >= lo && key <= p && tile + i / 4 < tile_end;
-      pw[i] = seen ? s[i / 4][i % 4] * scale2 : -FLT_MAX;
-      step_max = fmaxf(step_max, pw[i]);
+      for (int i = 0; i < 8; ++i) {
+        pw[i] = s[i / 4][i % 4] * scale2;
+        step_max = fmaxf(step_max, pw[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int key = ((tile + i / 4) << 4) + 4 * g + i % 4;
+        const bool seen = key >= lo && key <= p && tile + i / 4 < tile_end;
+        pw[i] = seen ? s[i / 4][i % 4] * scale2 : -FLT_MAX;
+        step_max = fmaxf(step_max, pw[i]);
+      }
     }
     step_max = rows_max(step_max);
     const float m_new = fmaxf(m, step_max);
@@ -241,7 +253,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      pw[i] = (pw[i] > -FLT_MAX) ? __builtin_amdgcn_exp2f(pw[i] - m_new) : 0.f;
+      pw[i] = (inner || pw[i] > -FLT_MAX) ? __builtin_amdgcn_exp2f(pw[i] - m_new) : 0.f;
       sum += pw[i];
     }
     l = l * corr + sum;   // this lane's share of the head's sum; the four lanes of a head meet at the end
@@ -249,20 +261,22 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     const bf16x8 pf = __builtin_bit_cast(bf16x8, w);
     // What lies beyond the visible keys is not data: it is cleared, so that a weight of zero times it is zero.
     // (Within lo..p a weight of zero meets a visible key's values.)
-    uint32_t keep_x[2], keep_y[2];
+    uint32_t keep_x[2] = {0xffffffffu, 0xffffffffu}, keep_y[2] = {0xffffffffu, 0xffffffffu};
+    if (!inner) {
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-      const int key4 = ((tile + kt) << 4) + 4 * g;
-      const int lo_e = lo - key4, hi_e = p - key4 + 1;       // elements lo_e .. hi_e - 1 are visible
-      keep_x[kt] = ((0 < lo_e || 0 >= hi_e) ? 0u : 0x0000ffffu) | ((1 < lo_e || 1 >= hi_e) ? 0u : 0xffff0000u);
-      keep_y[kt] = ((2 < lo_e || 2 >= hi_e) ? 0u : 0x0000ffffu) | ((3 < lo_e || 3 >= hi_e) ? 0u : 0xffff0000u);
+      for (int kt = 0; kt < 2; ++kt) {
+        const int key4 = ((tile + kt) << 4) + 4 * g;
+        const int lo_e = lo - key4, hi_e = p - key4 + 1;       // elements lo_e .. hi_e - 1 are visible
+        keep_x[kt] = ((0 < lo_e || 0 >= hi_e) ? 0u : 0x0000ffffu) | ((1 < lo_e || 1 >= hi_e) ? 0u : 0xffff0000u);
+        keep_y[kt] = ((2 < lo_e || 2 >= hi_e) ? 0u : 0x0000ffffu) | ((3 < lo_e || 3 >= hi_e) ? 0u : 0xffff0000u);
+      }
     }
     // O^T += V^T P^T
 #pragma unroll
     for (int nt = 0; nt < DT; ++nt) {
       o[nt] *= corr;
       uint32_t vw[4] = {st.v[0][nt].x & keep_x[0], st.v[0][nt].y & keep_y[0], st.v[1][nt].x & keep_x[1], st.v[1][nt].y & keep_y[1]};
-      if constexpr (kRope) {
+      if (last_here) {
         // the new token's value takes its place among this lane's four keys of the last tile
 #pragma unroll
         for (int w2 = 0; w2 < 4; ++w2) {
