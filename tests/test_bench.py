@@ -59,3 +59,14 @@ def test_the_continuous_batch_prints_its_line():
     assert d["roofline"]["steps"] > 100 and d["roofline"]["ms_per_step"] > 0            # the ticks in which all 64 decode, timed on the device
     assert abs(d["value"] - 64 * 256 / d["seconds"]) <= 0.01 * d["value"]
     assert "ticks with prompt portions" in err
+
+
+@pytest.mark.gpu
+def test_the_entry_points_smoke_run_agrees_with_the_plain_model(capsys):
+    """``__graft_entry__.smoke()``: a few tokens from a tiny random model in both dtypes, compared with the plain
+    implementation inside (it raises where they differ)."""
+    sys.path.insert(0, str(ROOT))
+    import __graft_entry__ as entry
+    entry.smoke()
+    said = capsys.readouterr().out
+    assert "smoke ok" in said and said.count("tokens agree") == 2
