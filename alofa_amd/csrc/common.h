@@ -148,6 +148,9 @@ struct Workspace {
 constexpr int kGemmCounters = 4096;   // counters the few-rows product may use
 const Workspace& workspace();
 
+// Compute units of the current device (asked once).
+int compute_units();
+
 // ---- error channel ---------------------------------------------------------
 
 void set_error(const char* fmt, ...);

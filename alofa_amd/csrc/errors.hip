@@ -28,6 +28,16 @@ int check_launch(const char* what) {
 static Workspace g_workspace = {nullptr, 0, nullptr, 0};
 const Workspace& workspace() { return g_workspace; }
 
+int compute_units() {
+  static int known = 0;
+  if (known == 0) {
+    int device = 0, n = 0;
+    if (hipGetDevice(&device) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && n > 0) known = n;
+    else return 256;      // (what an MI355X has; asked again next time)
+  }
+  return known;
+}
+
 }  // namespace alofa
 
 // Allocates the workspace (once; later calls do nothing). Kernels that would use it fall back to

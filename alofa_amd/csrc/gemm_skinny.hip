@@ -91,15 +91,15 @@ template <int MT, int NT, int kWaves, int kEpilogue, typename TO, int kUnroll, i
 __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     TO* __restrict__ out, int64_t ldo, const void* __restrict__ A, int64_t lda, const bf16_t* __restrict__ W,
     const bf16_t* __restrict__ W2, int64_t ldw, const float* __restrict__ bias, int M, int N, int K,
-    f32x4* __restrict__ ws, int* __restrict__ counters, const float* __restrict__ norm_w, float eps) {
+    f32x4* __restrict__ ws, int* __restrict__ counters, const float* __restrict__ norm_w, float eps, int cols) {
   __shared__ f32x4 red[kWaves][MT * NT][64];
   __shared__ float ssq[kNorm ? kWaves : 1][MT][16];
   constexpr bool kHalf = kNorm == 2;
   __shared__ int last_block;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int r = lane % 16, g = lane / 16;
-  constexpr int kColsPerBlock = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
-  const int n0 = blockIdx.x * kColsPerBlock;
+  // (cols: the columns a block owns, all that its tiles hold or fewer: see launch_skinny)
+  const int n0 = blockIdx.x * cols;
 
   const void* a_row[MT];
   bool a_ok[MT];
@@ -114,7 +114,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
-    w_ok[nt] = n < N;
+    w_ok[nt] = n < N && n - n0 < cols;
     const bf16_t* base = (kEpilogue == kSkSwiglu && nt == 1) ? W2 : W;
     w_row[nt] = base + static_cast<int64_t>(w_ok[nt] ? n : 0) * ldw;
   }
@@ -137,7 +137,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
   const int f_tile = threadIdx.x >> 8, f_r = (threadIdx.x >> 2) & 15, f_g = (threadIdx.x >> 6) & 3, f_i = threadIdx.x & 3;
   const int f_mt = (kEpilogue == kSkSwiglu) ? f_tile : f_tile / NT, f_nt = (kEpilogue == kSkSwiglu) ? 0 : f_tile % NT;
   const int f_m = f_mt * 16 + f_g * 4 + f_i, f_n = (kEpilogue == kSkSwiglu) ? n0 + f_r : n0 + f_nt * 16 + f_r;
-  const bool f_ok = flat && f_tile < kOutTiles && f_m < M && f_n < N;
+  const bool f_ok = flat && f_tile < kOutTiles && f_m < M && f_n < N && f_n - n0 < cols;
   float f_add = 0.f;
   if (f_ok) {
     if (kEpilogue == kSkStore && bias) f_add = bias[f_n];
@@ -154,7 +154,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
     for (int i = 0; i < 4; ++i) {
       const int m = mt * 16 + g * 4 + i;
       add[it][i] = 0.f;
-      if (!flat && tile < kOutTiles && n < N && m < M) {
+      if (!flat && tile < kOutTiles && n < N && n - n0 < cols && m < M) {
         if (kEpilogue == kSkStore && bias) add[it][i] = bias[n];
         if (kEpilogue == kSkResidual) add[it][i] = load_f32(out + static_cast<int64_t>(m) * ldo + n);
       }
@@ -379,7 +379,7 @@ __global__ void __launch_bounds__(kWaves * 64) gemm_skinny_kernel(
       }
     }
     const int n = (kEpilogue == kSkSwiglu) ? n0 + r : n0 + nt * 16 + r;
-    if (n >= N) continue;
+    if (n >= N || n - n0 >= cols) continue;
     if constexpr (kNorm) {
       // rows 4 g .. 4 g + 3 of the tile: their factors 1 / sqrt(mean of squares + eps)
 #pragma unroll
@@ -460,21 +460,37 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
     if (norm.weight != nullptr) {
       // (float rows take twice the registers: two sets of two steps keep two blocks on a compute unit)
       ALOFA_REQUIRE(K % 4 == 0 && K <= kMaxNormK, "gemm_skinny: the norm's weights must fit in LDS [K=%d, at most %d]", K, kMaxNormK);
+      // Where the blocks are more than the compute units, the one with the most decides: a compute unit takes in
+      // what its blocks read at some 30 GB/s, so the columns of a block are chosen for the least a compute unit's
+      // blocks read together (the weights of their columns and, each, all the rows): gate and up of 4,864 columns
+      // against eight rows of 896 in 487 blocks of ten columns (two a compute unit) 7.4 us, in 304 of sixteen 8.8,
+      // in 608 of eight 8.9.
+      int own = cols;
+      if (col_tiles > compute_units()) {
+        const int64_t row_bytes = static_cast<int64_t>(M) * K * 4, col_bytes = static_cast<int64_t>(kEpilogue == kSkSwiglu ? 2 : 1) * K * 2;
+        int64_t least = 0;
+        for (int c = cols; c >= cols / 2; --c) {
+          const int64_t blocks = (N + c - 1) / c, each = (blocks + compute_units() - 1) / compute_units();
+          const int64_t reads = each * (c * col_bytes + row_bytes);
+          if (least == 0 || reads < least) { least = reads; own = c; }
+        }
+      }
+      const int own_tiles = (N + own - 1) / own;
       if (M <= 8)
-        gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, 2><<<dim3(col_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
+        gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, 2><<<dim3(own_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
             static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
-            reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps);
+            reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps, own);
       else
-        gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, 1><<<dim3(col_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
+        gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, 2, 1><<<dim3(own_tiles, 1), kWaves * 64, K * sizeof(float), stream>>>(
             static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
-            reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps);
+            reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, norm.weight, norm.eps, own);
       return check_launch("gemm_skinny (with norm)");
     }
   }
   ALOFA_REQUIRE(norm.weight == nullptr, "gemm_skinny: the norm goes with at most 16 rows and the bfloat16 store and swiglu epilogues only");
   gemm_skinny_kernel<MT, NT, kWaves, kEpilogue, TO, unroll, false><<<dim3(col_tiles, k_splits), kWaves * 64, 0, stream>>>(
       static_cast<TO*>(out), ldo, A, lda, static_cast<const bf16_t*>(W),
-      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, nullptr, 0.f);
+      static_cast<const bf16_t*>(W2), ldw, bias, M, N, K, reinterpret_cast<f32x4*>(g_ws.tiles), g_ws.counters, nullptr, 0.f, cols);
   return check_launch("gemm_skinny");
 }
 

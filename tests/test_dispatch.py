@@ -20,7 +20,10 @@ def test_product_kernel_by_shape():
         assert ops.few_rows_kernel(rows, 1152, 896) == "rows" and ops.few_rows_kernel(rows, 896, 4864) == "rows"
         assert ops.few_rows_kernel(rows, 1152, 896, normed=True) == "rows"
     assert ops.few_rows_kernel(4, 2 * 27648, 5120, swiglu=True, normed=True) == "tiled" and ops.few_rows_kernel(2, 2 * 27648, 5120, swiglu=True) == "rows"
-    assert ops.few_rows_kernel(4, 2 * 4864, 896, swiglu=True, normed=True) == "rows" and ops.few_rows_kernel(5, 2 * 4864, 896, swiglu=True, normed=True) == "stream"
+    # gate and up of a small model with the norm: the streaming kernel from three rows on (its blocks are dealt out evenly), the vector units below
+    assert ops.few_rows_kernel(2, 2 * 4864, 896, swiglu=True, normed=True) == "rows" and ops.few_rows_kernel(3, 2 * 4864, 896, swiglu=True, normed=True) == "stream"
+    assert ops.few_rows_kernel(4, 2 * 4864, 896, swiglu=True, normed=True) == "stream" and ops.few_rows_kernel(5, 2 * 4864, 896, swiglu=True, normed=True) == "stream"
+    assert ops.few_rows_kernel(4, 2 * 4864, 896, swiglu=True) == "rows" and ops.few_rows_kernel(4, 2 * 18944, 3584, swiglu=True, normed=True) == "rows"
     assert ops.few_rows_kernel(4, 4608, 3584, normed=True) == "rows" and ops.few_rows_kernel(4, 7168, 5120, normed=True) == "stream"
     assert ops.few_rows_kernel(8, 4608, 3584, normed=True) == "stream" and ops.few_rows_kernel(8, 5120, 5120) == "rows"
     assert ops.few_rows_kernel(2, 3584, 18944) == "rows" and ops.few_rows_kernel(4, 3584, 18944) == "rows"    # long rows: its looping form
