@@ -460,20 +460,22 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
     if (norm.weight != nullptr) {
       // (float rows take twice the registers: two sets of two steps keep two blocks on a compute unit)
       ALOFA_REQUIRE(K % 4 == 0 && K <= kMaxNormK, "gemm_skinny: the norm's weights must fit in LDS [K=%d, at most %d]", K, kMaxNormK);
-      // Where the blocks are more than the compute units, the one with the most decides: a compute unit takes in
-      // what its blocks read at some 30 GB/s, so the columns of a block are chosen for the least a compute unit's
-      // blocks read together (the weights of their columns and, each, all the rows): gate and up of 4,864 columns
-      // against eight rows of 896 in 487 blocks of ten columns (two a compute unit) 7.4 us, in 304 of sixteen 8.8,
-      // in 608 of eight 8.9.
+      // A compute unit takes in what its blocks read (the weights of their columns and, each block, all the rows) at
+      // some 30 GB/s when all of them pull from memory, and the one with the most decides. So a block owns the number
+      // of columns, a quarter of its tiles' to all of them, for which the most a compute unit reads is least (fewer
+      // columns than all only for a tenth less): gate and up of 4,864 columns against eight rows of 896 in 487 blocks
+      // of ten columns, two a compute unit, 7.4 us where 304 blocks of sixteen take 8.8 and 608 of eight 8.9; QKV of
+      // 1,152 columns against sixteen rows in 231 blocks of five instead of 72 of sixteen (a decode step at batch 16
+      // 0.930 against 0.938 ms).
       int own = cols;
-      if (col_tiles > compute_units()) {
+      {
         const int64_t row_bytes = static_cast<int64_t>(M) * K * 4, col_bytes = static_cast<int64_t>(kEpilogue == kSkSwiglu ? 2 : 1) * K * 2;
-        int64_t least = 0;
-        for (int c = cols; c >= cols / 2; --c) {
+        auto reads = [&](int c) {
           const int64_t blocks = (N + c - 1) / c, each = (blocks + compute_units() - 1) / compute_units();
-          const int64_t reads = each * (c * col_bytes + row_bytes);
-          if (least == 0 || reads < least) { least = reads; own = c; }
-        }
+          return each * (c * col_bytes + row_bytes);
+        };
+        for (int c = cols - 1; c >= cols / 4; --c)
+          if (reads(c) * 10 < reads(own) * 9 || (reads(c) < reads(own) && own < cols)) own = c;
       }
       const int own_tiles = (N + own - 1) / own;
       if (M <= 8)
