@@ -418,18 +418,29 @@ struct NormArgs {
   float eps;
 };
 
-// Parts of K that the blocks of a column tile share out (1: no hand-over through the workspace).
+// Parts of K that the blocks of a column tile share out (1: no hand-over through the workspace). A block reads its
+// columns of W and every row of A over its share of K; a compute unit takes that in at a steady rate, the blocks come
+// in rounds of one a compute unit, and handing partial tiles over costs what some 40 KB of reading do, more with more
+// parts. So the parts are 1, 2, 4 or 8 (every wave keeps a step), the number for which rounds x bytes a block +
+// hand-over is least, and more parts only for 8 % less: QKV of 1,152 x 896 whole up to 32 rows (5.3-5.6 us where two
+// parts take 6.0-6.1) and in two parts from 48 on (64 rows 6.8 against 7.4); products of 1,536 to 2,048 columns in
+// two parts, never in four that outnumber the compute units (2,048 x 2,048 against 32 rows 7.7 against 11.0 us).
 template <int MT, int NT, int kWaves, int kEpilogue>
-static int skinny_splits(int N, int K) {
+static int skinny_splits(int M, int N, int K) {
   constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
   const int col_tiles = (N + cols - 1) / cols;
-  int k_splits = 1;
   const Workspace& g_ws = workspace();
-  if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr) {
-    const int steps = (K + 31) / 32;
-    const int min_steps = (MT == 1) ? 2 * kWaves : kWaves;
-    while (k_splits < 8 && col_tiles * k_splits * 2 <= 512 && steps / (k_splits * 2) >= min_steps) k_splits *= 2;
-    if (col_tiles > kGemmCounters || static_cast<int64_t>(col_tiles) * k_splits * MT * NT * 256 > g_ws.tile_floats) k_splits = 1;
+  if (kEpilogue == kSkSwiglu || g_ws.tiles == nullptr || col_tiles > kGemmCounters) return 1;
+  const int steps = (K + 31) / 32, units = compute_units();
+  const int64_t block_bytes = static_cast<int64_t>(M + cols) * K * 2;
+  auto cost = [&](int parts) {
+    const int64_t rounds = (static_cast<int64_t>(col_tiles) * parts + units - 1) / units;
+    return rounds * (block_bytes / parts) + (parts > 1 ? (24 + 8 * parts) * 1024 : 0);
+  };
+  int k_splits = 1;
+  for (int parts = 2; parts <= 8 && steps / parts >= kWaves; parts *= 2) {
+    if (static_cast<int64_t>(col_tiles) * parts * MT * NT * 256 > g_ws.tile_floats) break;
+    if (cost(parts) * 100 < cost(k_splits) * 92) k_splits = parts;
   }
   return k_splits;
 }
@@ -439,21 +450,13 @@ static int launch_skinny(void* out, int64_t ldo, const void* A, int64_t lda, con
                          const float* bias, int M, int N, int K, NormArgs norm, hipStream_t stream, int* splits_only) {
   constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
   const int col_tiles = (N + cols - 1) / cols;
-  // split K across blocks while the column tiles alone leave most of the chip idle
-  int k_splits = 1;
   const Workspace& g_ws = workspace();
   if (splits_only) {
-    *splits_only = skinny_splits<MT, NT, kWaves, kEpilogue>(N, K);
+    *splits_only = skinny_splits<MT, NT, kWaves, kEpilogue>(M, N, K);
     return 0;
   }
-  if (kEpilogue != kSkSwiglu && g_ws.tiles != nullptr && norm.weight == nullptr) {
-    const int steps = (K + 31) / 32;
-    // (a split costs a trip through memory: only while every wave keeps at least two steps of its own, four
-    // with one tile of rows, whose steps are light)
-    const int min_steps = (MT == 1) ? 2 * kWaves : kWaves;
-    while (k_splits < 8 && col_tiles * k_splits * 2 <= 512 && steps / (k_splits * 2) >= min_steps) k_splits *= 2;
-    if (col_tiles > kGemmCounters || static_cast<int64_t>(col_tiles) * k_splits * MT * NT * 256 > g_ws.tile_floats) k_splits = 1;
-  }
+  // (K is shared out over blocks only without a norm: the norm's sum of squares wants whole rows)
+  const int k_splits = norm.weight == nullptr ? skinny_splits<MT, NT, kWaves, kEpilogue>(M, N, K) : 1;
   // loads in flight: many for one row tile (latency is all there is), fewer as row tiles take the registers
   constexpr int unroll = (MT >= 4) ? 2 : 4;
   if constexpr (kEpilogue != kSkResidual && sizeof(TO) == 2 && MT == 1) {

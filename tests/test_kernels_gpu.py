@@ -289,8 +289,11 @@ def test_gemm_split_over_blocks_is_repeatable():
     of different shapes alternate, so that what the workspace held before is never the answer."""
     rng = np.random.default_rng(40)
     cases = []
-    for M, N, K, kernel in [(3, 1082, 672, "stream"), (40, 864, 672, "stream"), (5, 672, 4864, "stream"), (2, 144, 2048, "stream"),
+    from alofa_amd.csrc.build import load
+    for M, N, K, kernel in [(3, 1082, 4032, "stream"), (40, 864, 1344, "stream"), (5, 672, 4864, "stream"), (2, 144, 8192, "stream"),
                             (40, 864, 672, "tiled"), (150, 672, 4864, "tiled"), (20, 144, 2048, "tiled")]:
+        # (the product for few rows shares K out where a block would otherwise read much: these shapes are such)
+        assert kernel != "stream" or load().alofa_gemm_skinny_splits(0, M, N, K, 0) > 1, (M, N, K)
         a = t(bf(rng.standard_normal((M, K)).astype(np.float32)), torch.bfloat16)
         w = t(bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1), torch.bfloat16)
         out = torch.empty(M, N, device=DEV)
