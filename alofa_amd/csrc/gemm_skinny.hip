@@ -420,11 +420,14 @@ struct NormArgs {
 
 // Parts of K that the blocks of a column tile share out (1: no hand-over through the workspace). A block reads its
 // columns of W and every row of A over its share of K; a compute unit takes that in at a steady rate, the blocks come
-// in rounds of one a compute unit, and handing partial tiles over costs what some 40 KB of reading do, more with more
-// parts. So the parts are 1, 2, 4 or 8 (every wave keeps a step), the number for which rounds x bytes a block +
-// hand-over is least, and more parts only for 8 % less: QKV of 1,152 x 896 whole up to 32 rows (5.3-5.6 us where two
-// parts take 6.0-6.1) and in two parts from 48 on (64 rows 6.8 against 7.4); products of 1,536 to 2,048 columns in
-// two parts, never in four that outnumber the compute units (2,048 x 2,048 against 32 rows 7.7 against 11.0 us).
+// in rounds of one a compute unit (a round of four tiles of rows costs what 10 KB more would), and handing partial
+// tiles over costs what 44 KB of reading do with two parts, 76 with four, 140 with eight. The parts are 1, 2, 4 or 8
+// (every wave keeps a step): the number for which rounds x bytes a block + hand-over is least. The figures are fitted
+// to 45 measured shapes (projections of the 0.5B to 32B sizes against 6 to 64 rows, each in 1, 2, 4 and 8 parts): the
+// choice is the fastest or within 3 % of it for all but one matrix (2,048 x 11,008: two parts where four are 12 %
+// faster). QKV of 1,152 x 896 stays whole up to 32 rows (5.3-5.6 us where two parts take 6.0-6.1) and goes in two parts
+// from 48 on (64 rows 6.8 against 7.4); 2,048 x 2,048 against 32 rows goes in two parts (7.7 us; four, which outnumber
+// the compute units, 11.0); 2,560 x 2,048 against 64 rows stays whole (13.5; eight parts 18.0).
 template <int MT, int NT, int kWaves, int kEpilogue>
 static int skinny_splits(int M, int N, int K) {
   constexpr int cols = (kEpilogue == kSkSwiglu) ? 16 : 16 * NT;
@@ -435,12 +438,12 @@ static int skinny_splits(int M, int N, int K) {
   const int64_t block_bytes = static_cast<int64_t>(M + cols) * K * 2;
   auto cost = [&](int parts) {
     const int64_t rounds = (static_cast<int64_t>(col_tiles) * parts + units - 1) / units;
-    return rounds * (block_bytes / parts) + (parts > 1 ? (24 + 8 * parts) * 1024 : 0);
+    return rounds * (block_bytes / parts + (MT == 4 ? 10 : 0) * 1024) + (parts > 1 ? (12 + 16 * parts) * 1024 : 0);
   };
   int k_splits = 1;
   for (int parts = 2; parts <= 8 && steps / parts >= kWaves; parts *= 2) {
     if (static_cast<int64_t>(col_tiles) * parts * MT * NT * 256 > g_ws.tile_floats) break;
-    if (cost(parts) * 100 < cost(k_splits) * 92) k_splits = parts;
+    if (cost(parts) < cost(k_splits)) k_splits = parts;
   }
   return k_splits;
 }

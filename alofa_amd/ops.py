@@ -203,9 +203,12 @@ def few_rows_rule(M: int, w_rows: int, K: int, swiglu: bool = False, normed: boo
     its time grows with M; the tiled kernel's hardly does, but it needs more work
     per block to get going. Measured on one MI355X at the projection sizes of
     0.5B, 7B and 32B models, the tiled kernel wins from these weight sizes on
-    (w_rows * K, in elements): 64 M at 5..8 rows, 24 M at 9..16 rows, 8 M above
+    (w_rows * K, in elements): 64 M at 5..8 rows, 14 M at 9..16 rows (12 M where the rows
+    are longer than the vector-unit kernel takes in one go), 8 M at 17..32 rows
     (the gate and up matrices of the 0.5B sizes, 8.7 M: 12.0 against 13.5 us at 32
-    rows, 12.2 against 15.0 at 64; its down matrix, 4.4 M: 18.4 against 13.1);
+    rows, 12.2 against 15.0 at 64; its down matrix, 4.4 M: 18.4 against 13.1), 5 M above;
+    the sizes between those three models (1.5B, 3B, 14B) were measured later and moved
+    the thresholds where the comments below say so;
     and against a matrix as long as a vocabulary (256 column tiles of 128 or more)
     from the first row on."""
     if M > SKINNY_MAX_ROWS:
@@ -219,7 +222,9 @@ def few_rows_rule(M: int, w_rows: int, K: int, swiglu: bool = False, normed: boo
         small_gate_up = swiglu and normed and M >= 3 and elements <= 16 << 20
         if M <= 2 or (M <= 4 and not small_gate_up and ((swiglu and elements < 256 << 20) or (not swiglu and (not normed or elements < 24 << 20)))):
             return "rows"
-        if 4 < M <= 8 and not swiglu and elements <= ((4 << 20) if normed else (32 << 20)):
+        # (five to eight rows of more than ROWS_MAX_K values: its looping form loses, a 1,536 x 8,960 matrix 14.1-14.7 us
+        # against 11.5-12.1 for the streaming kernel, 2,048 x 11,008 19.1-19.4 against 15.9-16.5)
+        if 4 < M <= 8 and not swiglu and K <= ROWS_MAX_K and elements <= ((4 << 20) if normed else (32 << 20)):
             return "rows"
         if M > 8 and elements <= 8 << 20:
             return "rows"
@@ -228,8 +233,13 @@ def few_rows_rule(M: int, w_rows: int, K: int, swiglu: bool = False, normed: boo
     if M <= 8:
         return "tiled" if elements >= 64 << 20 else "stream"
     if M <= 16:
-        return "tiled" if elements >= 24 << 20 else "stream"
-    return "tiled" if elements >= 8 << 20 else "stream"
+        # (4,608 x 3,584: 16.0 against 16.9-17.4 us. Long rows against few columns, a down projection: the tiled kernel
+        # shares K out over more blocks, 2,048 x 11,008 15.9-16.1 us against 17.7-18.6, 1,536 x 8,960 13.4 against 13.4-14.4)
+        return "tiled" if elements >= 14 << 20 or (K > ROWS_MAX_K and elements >= 12 << 20) else "stream"
+    if M <= 32:
+        return "tiled" if elements >= 8 << 20 else "stream"
+    # (2,560 x 2,048 against 48 and 64 rows: 12.5 and 13.3 us against 14.0 and 15.9; 2,048 x 2,048 against 64: the same either way)
+    return "tiled" if elements >= 5 << 20 else "stream"
 
 
 RIDE_ON_SHARES = os.environ.get("ALOFA_RIDE_ON_SHARES", "1") != "0"
@@ -277,6 +287,19 @@ def _mfma_operands(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+def norm_goes_apart(M: int, N: int, K: int) -> bool:
+    """Whether a norm in front of a plain product of at most eight rows should run as a kernel of its own although
+    a product could take it along: the vector-unit kernel reads every row once per four columns, float32 rows
+    with the norm on it, so against a large matrix the rows' traffic (N / 4 x M x K x 4 bytes) outgrows what the
+    norm's own launch costs (some 3 us): from N x M x K of 63 M on the norm kernel and the product of bfloat16
+    rows win. Measured: 4,608 x 3,584 against 6 and 8 rows 13.6 and 14.1 us (norm kernel + product) where the
+    product with the norm takes 20.5 and 20.9 and the streaming kernel with the norm 15.2 and 15.6; 7,168 x 5,120
+    against 2, 3 and 4 rows 17.7, 18.8 and 19.2 against 19.6, 25.8 and 25.9 (streaming 23.0-24.1); smaller
+    products are faster with the norm on them (2,560 x 2,048 against 8 rows 7.3 against 8.0)."""
+    return (USE_ROWS_KERNEL and M <= ROWS_MAX_M and N * M * K > 63 << 20 and rows_kernel_takes(M, K)
+            and few_rows_kernel(M, N, K) == "rows")
+
+
 NORM_MAX_ROWS, NORM_MAX_COLUMNS = 16, 8192     # what the streaming kernel's norm form takes (one tile of rows; the norm's weights lie in LDS)
 FUSE_NORMS = os.environ.get("ALOFA_FUSE_NORMS", "1") != "0"   # 0: every norm runs as a kernel of its own
 
@@ -290,6 +313,8 @@ def can_fuse_norm(M: int, w: torch.Tensor, out_dtype, swiglu: bool = False, kern
     if not FUSE_NORMS:
         return False
     if w.dtype is not torch.bfloat16 or out_dtype is not torch.bfloat16 or K % 8 or w.stride(0) % 8 or w.data_ptr() % 16:
+        return False
+    if kernel is None and not swiglu and norm_goes_apart(M, N, K):
         return False
     chosen = kernel or few_rows_kernel(M, 2 * N if swiglu else N, K, swiglu, normed=True)
     if chosen == "rows":

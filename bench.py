@@ -49,7 +49,10 @@ def family(layers, hidden, heads, kv_heads, inter, vocab, tied, max_pos=32768):
 
 CONFIGS = {
     "0.5b": family(24, 896, 14, 2, 4864, 151936, True),
+    "1.5b": family(28, 1536, 12, 2, 8960, 151936, True),
+    "3b": family(36, 2048, 16, 2, 11008, 151936, True),
     "7b": family(28, 3584, 28, 4, 18944, 152064, False),
+    "14b": family(48, 5120, 40, 8, 13824, 152064, False),
     "32b": family(64, 5120, 40, 8, 27648, 152064, False, 40960),
 }
 QWEN25_05B = CONFIGS["0.5b"]
@@ -469,7 +472,7 @@ def sweep(args):
     cfg = dict(CONFIGS[name], num_hidden_layers=args.layers or CONFIGS[name]["num_hidden_layers"])
     model = device_model(cfg, args.dtype, 20260918)
     dbytes = 2 if args.dtype == "bfloat16" else 4
-    batches = (1, 2, 4, 8, 16, 17, 24, 32, 48, 64, 96, 128, 192, 256) if name == "0.5b" else (1, 2, 4, 8, 16, 32, 64)
+    batches = (1, 2, 4, 8, 16, 17, 24, 32, 48, 64, 96, 128, 192, 256) if name == "0.5b" else (1, 2, 4, 8, 16, 17, 32, 64) if name in ("1.5b", "3b") else (1, 2, 4, 8, 16, 32, 64)
     cases = ([(b, PROMPT) for b in batches] if args.sweep == "batch" else
              [(b, p) for p in (2048, 8192, 16384, 30000) for b in (1, 8, 32)])
     for batch, prompt in cases:
@@ -506,7 +509,7 @@ def main():
     load()
     if args.sweep:
         return sweep(args)
-    if args.config == "7b" or args.serve:
+    if args.config in ("1.5b", "3b", "7b", "14b") or args.serve:
         return continuous_batch(args)
     if args.config == "32b":
         return long_prompts(args)

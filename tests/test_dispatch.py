@@ -30,7 +30,13 @@ def test_product_kernel_by_shape():
     assert ops.few_rows_kernel(2, 2 * 4864, 8192, swiglu=True) == "stream" and ops.few_rows_kernel(2, 1024, 8192, normed=True) == "stream"    # (plain products only)
     assert ops.few_rows_kernel(2, 2 * 18944, 8192, swiglu=True) == "tiled"        # gate and up of 256 M weights or more: the tiled kernel's wide tiles
     assert ops.few_rows_kernel(8, 3584, 18944) == "tiled"
-    assert ops.few_rows_kernel(16, 4608, 3584) == "stream" and ops.few_rows_kernel(17, 4608, 3584) == "tiled"
+    assert ops.few_rows_kernel(16, 3584, 3584) == "stream" and ops.few_rows_kernel(16, 4608, 3584) == "tiled" and ops.few_rows_kernel(17, 3584, 3584) == "tiled"
+    # five to eight rows of more values than the vector-unit kernel takes in one go: not its looping form
+    assert ops.few_rows_kernel(8, 1536, 8960) == "stream" and ops.few_rows_kernel(4, 1536, 8960) == "rows" and ops.few_rows_kernel(8, 896, 4864) == "rows"
+    # nine to sixteen rows against a long, narrow matrix: the tiled kernel, which shares K out over more blocks
+    assert ops.few_rows_kernel(12, 2048, 11008) == "tiled" and ops.few_rows_kernel(12, 1536, 8960) == "tiled" and ops.few_rows_kernel(12, 2048, 2048) == "rows"
+    # beyond 32 rows the tiled kernel takes smaller matrices than below
+    assert ops.few_rows_kernel(32, 2560, 2048) == "stream" and ops.few_rows_kernel(48, 2560, 2048) == "tiled" and ops.few_rows_kernel(64, 2048, 2048) == "stream"
     assert ops._product_entry(None, 8, 896, 4864) == "alofa_gemm_rows" and ops._product_entry("stream", 8, 896, 4864) == "alofa_gemm_skinny"
     with pytest.raises(AlofaError):
         ops._product_entry("rows", 17, 64, 64)
@@ -40,6 +46,14 @@ def test_product_kernel_by_shape():
         ops._product_entry("stream", 65, 64, 64)
     with pytest.raises(AlofaError):
         ops._product_entry("fast", 4, 64, 64)
+
+
+def test_a_norm_in_front_of_a_large_product_of_few_rows_runs_apart():
+    # the vector-unit kernel reads float32 rows once per four columns: against a large matrix the norm's own kernel costs less
+    assert ops.norm_goes_apart(8, 4608, 3584) and ops.norm_goes_apart(6, 4608, 3584) and not ops.norm_goes_apart(2, 4608, 3584)
+    assert ops.norm_goes_apart(2, 7168, 5120) and ops.norm_goes_apart(4, 7168, 5120) and not ops.norm_goes_apart(1, 7168, 5120)
+    assert not ops.norm_goes_apart(8, 7168, 5120)                  # (the plain product of so many values is not the vector units' either)
+    assert not ops.norm_goes_apart(8, 1152, 896) and not ops.norm_goes_apart(8, 2560, 2048) and not ops.norm_goes_apart(12, 4608, 3584)
 
 
 def test_a_norm_behind_a_product_moves_it_to_the_kernel_that_adds_shares():
