@@ -24,7 +24,9 @@ tokens per second at the default batch of 8. Beside it:
 ``--config 7b`` and ``--config 32b`` run the larger configurations' workloads
 (a continuous batch of 64 requests with prompts of 128..2,048 tokens under
 chunked prefill; 8 prompts of 16,384 tokens and decoding at batch 32 with a
-context of 4,096) through the same engine and print their own line."""
+context of 4,096) through the same engine and print their own line;
+``--config 1.5b``, ``3b`` and ``14b`` run the continuous batch at those sizes.
+``--sweep batch`` and ``--sweep context`` take any of the configurations."""
 import argparse
 import json
 import statistics
@@ -467,7 +469,7 @@ def long_prompts(args):
 def sweep(args):
     """Decode steps over batch sizes (at a context of about 550) or over contexts (batch 1, 8, 32): one line per
     point with ms per step, tokens a second and the bytes the step has to read / time. At the 0.5B sizes, or with
-    --config 7b / 32b at those (batches up to 64; --layers for fewer layers than the configuration has)."""
+    --config 1.5b .. 32b at those (batches up to 64; --layers for fewer layers than the configuration has)."""
     name = args.config
     cfg = dict(CONFIGS[name], num_hidden_layers=args.layers or CONFIGS[name]["num_hidden_layers"])
     model = device_model(cfg, args.dtype, 20260918)
