@@ -557,6 +557,147 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
   tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out, ldo, bias, M, N, m0, n0, wm, wn, lane);
 }
 
+// The tiled product for many rows against a wide matrix: eight waves (WM x WN) on a tile of TM x TN outputs, slabs of 32
+// along K straight from memory into a ring of S in LDS. Against the four waves and slabs of 64 above: a wave's share of
+// a slab is small enough (a tile of 256 x 256 in 128 KB of ring) for two waves a SIMD, which fill one another's waits
+// at the barrier and for LDS, and a slab carries twice the products per byte fetched. The sums are the same numbers in
+// the same order as in the kernels above (one accumulator an output, ascending k). K a multiple of 32.
+// A slab is TM rows of A and TN rows of W, 64 bytes each; the four 16-byte chunks of a row are permuted by the row's
+// number (chunk c of row r lies at place c ^ ((r >> 2) & 3)), so that the sixteen rows whose fragments a quarter of a
+// wave reads together fall on distinct banks. kMfSwiglu: the slab's W rows are TN / 2 gate rows, then the up rows of the
+// same columns, and a wave holds gate and up of the same columns.
+__device__ __forceinline__ int swz32(int r) { return (r >> 2) & 3; }
+
+template <int kEpilogue, typename TO, int TM, int TN, int WM, int WN, int S>
+__global__ void __launch_bounds__(64 * WM * WN) gemm_wide_kernel(TO* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ A, int64_t lda,
+                                                                 const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2, int64_t ldw,
+                                                                 const float* __restrict__ bias, int M, int N, int K, int tiles_m, int tiles_n) {
+  constexpr int kSlabK = 32, kRows = TM + TN, kStageBytes = kRows * 64, kWaves = WM * WN;
+  constexpr int kLoads = kRows / 16 / kWaves;        // fetch instructions per wave and slab (each brings sixteen rows)
+  constexpr int TI = TM / 32 / WM, TJ = TN / 32 / WN;   // 32 x 32 tiles a wave
+  static_assert(kRows % (16 * kWaves) == 0 && TM % (32 * WM) == 0 && TN % (32 * WN) == 0, "the tile must divide among the waves");
+  static_assert(kEpilogue != kMfSwiglu || TJ % 2 == 0, "the swiglu epilogue needs gate and up tiles in every wave");
+  constexpr int kGateTiles = TJ / 2;
+  __shared__ __attribute__((aligned(1024))) char ring[S * kStageBytes];
+  const TilePlace place = place_tile(blockIdx.x, tiles_m, tiles_n, 1, true);
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int wm = wave / WN, wn = wave % WN;
+  constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
+  const int m0 = place.bm * TM, n0 = place.bn * kOutCols;
+
+  // what this lane fetches: instruction j of this wave brings slab rows 16 (kWaves j + wave) .. + 15, lane l place l % 4 of row l / 4
+  const bf16_t* src[kLoads];
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) {
+    const int r = 16 * (kWaves * j + wave) + lane / 4, c = (lane % 4) ^ swz32(r);
+    if (r < TM) {
+      src[j] = A + static_cast<int64_t>(min(m0 + r, M - 1)) * lda + c * 8;
+    } else {
+      const int row = r - TM;
+      int n = n0 + row;
+      const bf16_t* base = W;
+      if (kEpilogue == kMfSwiglu && row >= TN / 2) {
+        n = n0 + row - TN / 2;
+        base = W2;
+      }
+      src[j] = base + static_cast<int64_t>(min(n, N - 1)) * ldw + c * 8;
+    }
+  }
+  const unsigned ring_at = static_cast<unsigned>(reinterpret_cast<uintptr_t>(ring));
+  auto fetch = [&](int slab) {     // uniform over the block
+    const unsigned stage = ring_at + (slab % S) * kStageBytes + wave * 1024;
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+      const bf16_t* from = src[j] + static_cast<int64_t>(slab) * kSlabK;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :: "s"(__builtin_amdgcn_readfirstlane(stage + j * kWaves * 1024)), "v"(from), "r"(ring) : "memory", "m0");
+    }
+  };
+
+  f32x16 acc[TI][TJ];
+#pragma unroll
+  for (int i = 0; i < TI; ++i)
+#pragma unroll
+    for (int j = 0; j < TJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // fragments: lane l reads row l % 32 of its 32-row group, chunk 2 q + l / 32 in step q of the slab's two
+  const int sw = swz32(lane % 32), half = lane / 32;
+  const int a_row = (wm * 32 * TI + lane % 32) * 64;
+  const int w_row = (TM + lane % 32) * 64;
+  int place_of[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) place_of[q] = ((2 * q + half) ^ sw) * 16;
+  auto w_group = [&](int j) {      // byte offset of this wave's j-th 32-row group within the slab's W rows
+    if (kEpilogue == kMfSwiglu) return ((j < kGateTiles ? 0 : TN / 2) + (wn * kGateTiles + j % kGateTiles) * 32) * 64;
+    return (wn * TJ + j) * 32 * 64;
+  };
+  auto step = [&](int slab) {
+    const char* stage = ring + (slab % S) * kStageBytes;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      bf16x8 a[TI], w[TJ];
+#pragma unroll
+      for (int i = 0; i < TI; ++i) a[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(stage + a_row + i * 32 * 64 + place_of[q]));
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) w[j] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(stage + w_row + w_group(j) + place_of[q]));
+#pragma unroll
+      for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], w[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  // Slab k + S - 1 takes the place of slab k - 1, which every wave has read before the barrier of step k; a wave waits
+  // for its own fetches of slab k (the S - 2 slabs behind it stay on their way) before that barrier.
+  const int slabs = K / kSlabK;
+  constexpr int kLead = S - 1;
+#pragma unroll
+  for (int p = 0; p < kLead; ++p)
+    if (p < slabs) fetch(p);
+  int k = 0;
+  for (; k + kLead < slabs; ++k) {
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kLoads * (kLead - 1)) : "memory");
+    __syncthreads();
+    fetch(k + kLead);
+    step(k);
+  }
+  for (; k < slabs; ++k) {      // nothing more to set out: the last slabs as they come
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    step(k);
+  }
+  tile_epilogue<kEpilogue, TO, TI, TJ>(acc, out, ldo, bias, M, N, m0, n0, wm, wn, lane);
+}
+
+template <int kEpilogue, typename TO, int TM, int TN, int WM, int WN, int S>
+static int launch_wide(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
+                       hipStream_t stream, const void* W2 = nullptr) {
+  constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
+  const int tiles_n = (N + kOutCols - 1) / kOutCols, tiles_m = (M + TM - 1) / TM;
+  gemm_wide_kernel<kEpilogue, TO, TM, TN, WM, WN, S><<<tiles_n * tiles_m, 64 * WM * WN, 0, stream>>>(
+      static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
+      tiles_m, tiles_n);
+  return 0;
+}
+
+// Where the tiles of 256 x 256 with eight waves are the tiled product's choice: many rows against a long K, and so many
+// tiles that their rounds of one a compute unit are at least four fifths full. Measured against the forms below
+// (2,048 rows, us): gate/up + SwiGLU of the 7B sizes 524 against 586, of the 32B sizes 1,043 against 1,169 (4,096 rows:
+// 2,086 against 2,268; 256 rows, 216 tiles: 174 against 254); 7,168 x 5,120 150 against 183 (4,096 rows: 293 against
+// 350); 3,584 x 3,584 at 4,096 rows 116 against 142, 3,584 x 18,944 538 against 592. With rounds less full the forms
+// below stay ahead (7B gate/up at 512 rows, 296 tiles: 210 against 176; 5,120 x 27,648 at 4,096 rows, 320 tiles: 1,507
+// against 1,285), and so they do with a short K (0.5B gate/up at 2,048 rows 60.6 against 46.3).
+template <int kEpilogue>
+static bool wide_pays(int M, int N, int K) {
+  if (M <= 128 || K % 32 != 0 || K < 2048) return false;
+  constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? 128 : 256;
+  const int64_t tiles = static_cast<int64_t>((M + 255) / 256) * ((N + kOutCols - 1) / kOutCols), units = compute_units();
+  const int64_t rounds = (tiles + units - 1) / units;
+  return tiles * 5 >= rounds * units * 4;
+}
+
 template <int kEpilogue, typename TO, int WTM, int WTN, int PF, bool kSplitK>
 static int launch_tile(int tiles_n, int tiles_m, int shares, void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                        const float* bias, int M, int N, int K, hipStream_t stream) {
@@ -763,6 +904,12 @@ static int k_shares(int64_t tiles, int64_t tile_floats, int K) {
 template <int kEpilogue, typename TO>
 static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
                        const float* bias, int M, int N, int K, hipStream_t stream, const ThenNorm& then, int* then_done) {
+  if constexpr (kEpilogue != kMfArgmax) {
+    if (wide_pays<kEpilogue>(M, N, K)) {
+      if (launch_wide<kEpilogue, TO, 256, 256, 4, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+      return check_launch("gemm_wide");
+    }
+  }
   if constexpr (kEpilogue == kMfSwiglu) {
     // A block computes gate and up of the same 64 columns. With K a multiple of 64 and tiles that do not fill the
     // chip twice over, the slabs go straight from memory into a ring in LDS (0.5B sizes, us against the kernel
@@ -961,6 +1108,27 @@ extern "C" int alofa_gemm_mfma(void* out, int o_dtype, int64_t ldo, const void* 
     return launch_mfma<kMfSwiglu, bf16_t>(out, ldo, A, lda, W, W2, ldw, nullptr, M, N, K, stream, kNoNorm, done);
   }
   ALOFA_REQUIRE(false, "gemm_mfma: unsupported epilogue %d with out dtype %d", epilogue, o_dtype);
+}
+
+// The same product by the tiles of 256 x 256 with eight waves whatever the sizes (alofa_gemm_mfma takes them where they
+// pay): K a multiple of 32. The operands as for alofa_gemm_mfma; norm_w and eps stand where alofa_gemm_skinny has them
+// and must be null and zero (no norm rides on this kernel).
+extern "C" int alofa_gemm_wide(void* out, int o_dtype, int64_t ldo, const void* A, int64_t lda, const void* W, const void* W2, int64_t ldw,
+                               const float* bias, int M, int N, int K, int epilogue, const float* norm_w, float eps, hipStream_t stream) {
+  ALOFA_REQUIRE(M > 0 && N > 0 && K > 0 && K % 32 == 0, "gemm_wide: M=%d N=%d K=%d must be positive, K a multiple of 32", M, N, K);
+  ALOFA_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldo >= N, "gemm_wide: lda=%lld, ldw=%lld must be multiples of 8 and cover K, ldo=%lld cover N",
+                static_cast<long long>(lda), static_cast<long long>(ldw), static_cast<long long>(ldo));
+  ALOFA_REQUIRE(reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 && reinterpret_cast<uintptr_t>(W2) % 16 == 0,
+                "gemm_wide: operands must be 16-byte aligned");
+  ALOFA_REQUIRE(norm_w == nullptr && eps == 0.f, "gemm_wide: no norm rides on this kernel");
+  int failed = 1;
+  if (epilogue == kMfStore && o_dtype == kBF16) failed = launch_wide<kMfStore, bf16_t, 256, 256, 4, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream);
+  else if (epilogue == kMfStore && o_dtype == kF32) failed = launch_wide<kMfStore, float, 256, 256, 4, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream);
+  else if (epilogue == kMfResidual && o_dtype == kF32) failed = launch_wide<kMfResidual, float, 256, 256, 4, 2, 4>(out, ldo, A, lda, W, ldw, nullptr, M, N, K, stream);
+  else if (epilogue == kMfSwiglu && o_dtype == kBF16 && W2 != nullptr) failed = launch_wide<kMfSwiglu, bf16_t, 256, 256, 4, 2, 4>(out, ldo, A, lda, W, ldw, nullptr, M, N, K, stream, W2);
+  else ALOFA_REQUIRE(false, "gemm_wide: unsupported epilogue %d with out dtype %d", epilogue, o_dtype);
+  if (failed) return 1;
+  return check_launch("gemm_wide");
 }
 
 // out[m] = the column n with the highest sum_k A[m, k] * W[n, k] (the lowest n among equals), for M <= 64 rows

@@ -261,6 +261,8 @@ def _product_entry(kernel: Optional[str], M: int, w_rows: int, K: int, swiglu: b
         return "alofa_gemm_rows"
     if kernel == "tiled":
         return "alofa_gemm_mfma"
+    if kernel == "wide" and not normed and K % 32 == 0:      # (the tiled kernel's form for many rows, whatever the sizes: for tests and measurements)
+        return "alofa_gemm_wide"
     raise AlofaError("invalid_argument", "no such product kernel for these rows", f"kernel={kernel} M={M}")
 
 

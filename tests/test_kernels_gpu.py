@@ -340,6 +340,57 @@ def test_gemm_tiled_with_slabs_straight_into_lds(M, N, K):
     assert (one[0] - outf[M - 1]).abs().max().item() <= 2e-6 * outf[M - 1].abs().max().item()
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 400, 96), (256, 256, 32), (1, 5, 64), (513, 1030, 2080), (700, 130, 4096)])
+def test_gemm_tiled_with_eight_waves_and_slabs_of_32(M, N, K):
+    """The tiled product's form for many rows against a wide matrix (tiles of 256 x 256, eight waves, slabs of
+    32 along K straight into a ring of four in LDS), asked for by name at sizes with edges in both directions,
+    one slab and many, every epilogue it has, and rows that are a strided view; and the same bits as the tiled
+    product's other forms give (one accumulator an output, ascending k, in all of them)."""
+    rng = np.random.default_rng(48)
+    a, w, w2 = (bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1),
+                bf(rng.standard_normal((N, K)).astype(np.float32) * 0.1))
+    b = rng.standard_normal(N).astype(np.float32)
+    ta, tw, tw2 = t(a, torch.bfloat16), t(w, torch.bfloat16), t(w2, torch.bfloat16)
+    out = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm(out, ta, tw, t(b), kernel="wide")
+    close(out, pm.linear(a, w, b), BF16, "bf16 out")
+    outf = torch.empty(M, N, device=DEV)
+    ops().gemm(outf, ta, tw, kernel="wide")
+    close(outf, pm.linear(a, w), 1e-4, "f32 out")
+    tiled = torch.empty(M, N, device=DEV)
+    ops().gemm(tiled, ta, tw, kernel="tiled")
+    if K < 2048:      # (with a long K and few tiles the tiled product shares K out over blocks: other sums)
+        assert torch.equal(tiled, outf)
+    res = rng.standard_normal((M, N)).astype(np.float32)
+    acc = t(res)
+    ops().gemm(acc, ta, tw, add_to_out=True, kernel="wide")
+    close(acc, pm.add(res, pm.linear(a, w)), 1e-4, "residual")
+    outs = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm_swiglu(outs, ta, tw, tw2, kernel="wide")
+    close(outs, pm.swiglu(pm.linear(a, w), pm.linear(a, w2)), BF16, "swiglu")
+    view = torch.zeros(M, K + 72, device=DEV, dtype=torch.bfloat16)
+    view[:, 8:8 + K] = ta
+    ops().gemm(outf, view[:, 8:8 + K], tw, kernel="wide")
+    close(outf, pm.linear(a, w), 1e-4, "rows that are a view")
+    with pytest.raises(AlofaError):
+        ops().gemm(torch.empty(M, N, device=DEV), t(a[:, :K - 8].copy(), torch.bfloat16), t(w[:, :K - 8].copy(), torch.bfloat16), kernel="wide")      # K no multiple of 32
+
+
+def test_the_tiled_product_takes_its_wide_form_where_the_rounds_are_full():
+    """Many rows against a long K and tiles of 256 x 256 in nearly full rounds of the chip: the tiled product goes
+    to the form above by itself; its sums are those of the forms it replaces (2,048 x 7,168 x 2,048: 224 tiles)."""
+    rng = np.random.default_rng(49)
+    M, N, K = 2048, 7168, 2048
+    a = t(bf(rng.standard_normal((M, K)).astype(np.float32)), torch.bfloat16)
+    w = t(bf(rng.standard_normal((N, K)).astype(np.float32) * 0.05), torch.bfloat16)
+    by_rule, by_name = torch.empty(M, N, device=DEV, dtype=torch.bfloat16), torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    ops().gemm(by_rule, a, w, kernel="tiled")
+    ops().gemm(by_name, a, w, kernel="wide")
+    assert torch.equal(by_rule, by_name)
+    rows = slice(1000, 1040)
+    close(by_rule[rows], pm.linear(a[rows].float().cpu().numpy(), w.float().cpu().numpy()), BF16, "against the plain product")
+
+
 def test_gemm_takes_a_strided_view():
     rng = np.random.default_rng(4)
     big = rng.standard_normal((6, 300)).astype(np.float32)
