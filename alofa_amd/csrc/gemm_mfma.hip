@@ -26,6 +26,8 @@
 // W slab holds as many rows of each) and writes silu(gate) * up.
 #include "common.h"
 
+#include <cstdlib>
+
 namespace alofa {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -691,7 +693,8 @@ static int launch_wide(void* out, int64_t ldo, const void* A, int64_t lda, const
 // against 1,285), and so they do with a short K (0.5B gate/up at 2,048 rows 60.6 against 46.3).
 template <int kEpilogue>
 static bool wide_pays(int M, int N, int K) {
-  if (M <= 128 || K % 32 != 0 || K < 2048) return false;
+  static const bool switched_off = [] { const char* e = getenv("ALOFA_WIDE_TILES"); return e != nullptr && e[0] == '0'; }();     // (for measurements)
+  if (switched_off || M <= 128 || K % 32 != 0 || K < 2048) return false;
   constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? 128 : 256;
   const int64_t tiles = static_cast<int64_t>((M + 255) / 256) * ((N + kOutCols - 1) / kOutCols), units = compute_units();
   const int64_t rounds = (tiles + units - 1) / units;
