@@ -220,7 +220,12 @@ def few_rows_rule(M: int, w_rows: int, K: int, swiglu: bool = False, normed: boo
         # (gate and up with the norm at three and four rows against small matrices: the streaming kernel since its blocks
         # are dealt out evenly over the compute units, 0.5B sizes 7.0 and 7.1 against 7.3 us; at two rows 6.8 against 6.4)
         small_gate_up = swiglu and normed and M >= 3 and elements <= 16 << 20
-        if M <= 2 or (M <= 4 and not small_gate_up and ((swiglu and elements < 256 << 20) or (not swiglu and (not normed or elements < 24 << 20)))):
+        # (three and four rows against a large matrix of long rows whose blocks of four columns leave the last round
+        # of an MI355X's 256 compute units half empty: 3,584 x 18,944, 896 blocks, 35.4-36.3 us against the tiled
+        # kernel's 31.5; with 5,120 x 13,824, 1,280 blocks, five full rounds, it stays ahead: 34.9-35.8 against 37.4)
+        blocks = (w_rows + 3) // 4
+        ragged_rounds = K > ROWS_MAX_K and elements >= 64 << 20 and M >= 3 and blocks * 10 < -(-blocks // 256) * 256 * 9
+        if M <= 2 or (M <= 4 and not small_gate_up and not ragged_rounds and ((swiglu and elements < 256 << 20) or (not swiglu and (not normed or elements < 24 << 20)))):
             return "rows"
         # (five to eight rows of more than ROWS_MAX_K values: its looping form loses, a 1,536 x 8,960 matrix 14.1-14.7 us
         # against 11.5-12.1 for the streaming kernel, 2,048 x 11,008 19.1-19.4 against 15.9-16.5)
@@ -229,7 +234,9 @@ def few_rows_rule(M: int, w_rows: int, K: int, swiglu: bool = False, normed: boo
         if M > 8 and elements <= 8 << 20:
             return "rows"
     if M <= 4:
-        return "tiled" if swiglu and elements >= 256 << 20 else "stream"
+        if swiglu:
+            return "tiled" if elements >= 256 << 20 else "stream"
+        return "tiled" if K > ROWS_MAX_K and elements >= 64 << 20 else "stream"
     if M <= 8:
         return "tiled" if elements >= 64 << 20 else "stream"
     if M <= 16:

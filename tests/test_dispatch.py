@@ -26,7 +26,9 @@ def test_product_kernel_by_shape():
     assert ops.few_rows_kernel(4, 2 * 4864, 896, swiglu=True) == "rows" and ops.few_rows_kernel(4, 2 * 18944, 3584, swiglu=True, normed=True) == "rows"
     assert ops.few_rows_kernel(4, 4608, 3584, normed=True) == "rows" and ops.few_rows_kernel(4, 7168, 5120, normed=True) == "stream"
     assert ops.few_rows_kernel(8, 4608, 3584, normed=True) == "stream" and ops.few_rows_kernel(8, 5120, 5120) == "rows"
-    assert ops.few_rows_kernel(2, 3584, 18944) == "rows" and ops.few_rows_kernel(4, 3584, 18944) == "rows"    # long rows: its looping form
+    assert ops.few_rows_kernel(2, 3584, 18944) == "rows" and ops.few_rows_kernel(4, 5120, 13824) == "rows"    # long rows: its looping form
+    assert ops.few_rows_kernel(3, 3584, 18944) == "tiled" and ops.few_rows_kernel(4, 3584, 18944) == "tiled"  # (not where its blocks come in three and a half rounds)
+    assert ops.few_rows_kernel(4, 2048, 11008) == "rows" and ops.few_rows_kernel(4, 5120, 27648) == "rows"
     assert ops.few_rows_kernel(2, 2 * 4864, 8192, swiglu=True) == "stream" and ops.few_rows_kernel(2, 1024, 8192, normed=True) == "stream"    # (plain products only)
     assert ops.few_rows_kernel(2, 2 * 18944, 8192, swiglu=True) == "tiled"        # gate and up of 256 M weights or more: the tiled kernel's wide tiles
     assert ops.few_rows_kernel(8, 3584, 18944) == "tiled"
