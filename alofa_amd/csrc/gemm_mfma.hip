@@ -365,7 +365,7 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
                                                        const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2, int64_t ldw,
                                                        const float* __restrict__ bias, int M, int N, int K, int tiles_m,
                                                        int tiles_n, int by_die, int shares = 1, float* __restrict__ ws = nullptr,
-                                                       int* __restrict__ counters = nullptr) {
+                                                       int* __restrict__ counters = nullptr, int own = 0) {
   constexpr int TM = 64 * WTM, TN = 64 * WTN;
   constexpr int kGateTiles = WTN / 2;
   // (swiglu with WTN = 1: the waves of column 0 take 32 gate columns, those of column 1 the up columns of the same
@@ -380,7 +380,11 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int wm = wave / 2, wn = wave % 2;
   constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? TN / 2 : TN;
-  const int m0 = place.bm * TM, n0 = place.bn * kOutCols;
+  // (own: the output columns a block owns of those its tile holds, all of them if 0: see launch_dma. The columns
+  // beyond are fetched from the last owned one, which costs no memory traffic, and never stored.)
+  const int owned = own > 0 ? own : kOutCols;
+  const int m0 = place.bm * TM, n0 = place.bn * owned;
+  const int n_end = min(N, n0 + owned);
 
   // what this lane fetches: instruction j of this wave brings slab rows 8 (4 j + wave) .. + 7, lane l place l % 8 of row l / 8
   const bf16_t* src[kLoads];
@@ -397,7 +401,7 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
         n = n0 + row - TN / 2;
         base = W2;
       }
-      src[j] = base + static_cast<int64_t>(min(n, N - 1)) * ldw + c * 8;
+      src[j] = base + static_cast<int64_t>(min(n, n_end - 1)) * ldw + c * 8;
     }
   }
   // The fetches are written out as instructions: the compiler, which cannot tell the ring's slabs apart, would wait
@@ -499,7 +503,7 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
         for (int e = 0; e < 16; ++e) {
           const int m = m_first + 8 * (e / 4) + e % 4;
           const float g = acc[i][0][e], up = meet[((wm * WTM + i) * 16 + e) * 64 + lane];
-          if (m < M && n < N) store_f32(out + static_cast<int64_t>(m) * ldo + n, g / (1.f + __expf(-g)) * up);
+          if (m < M && n < n_end) store_f32(out + static_cast<int64_t>(m) * ldo + n, g / (1.f + __expf(-g)) * up);
         }
       }
     }
@@ -556,7 +560,7 @@ __global__ void __launch_bounds__(256) gemm_dma_kernel(TO* __restrict__ out, int
         }
       }
   }
-  tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out, ldo, bias, M, N, m0, n0, wm, wn, lane);
+  tile_epilogue<kEpilogue, TO, WTM, WTN>(acc, out, ldo, bias, M, n_end, m0, n0, wm, wn, lane);
 }
 
 // The tiled product for many rows against a wide matrix: eight waves (WM x WN) on a tile of TM x TN outputs, slabs of 32
@@ -873,15 +877,16 @@ static int launch_dma_sliced(void* out, int64_t ldo, const void* A, int64_t lda,
 
 template <int kEpilogue, typename TO, int WTM, int WTN, int S>
 static int launch_dma(void* out, int64_t ldo, const void* A, int64_t lda, const void* W, int64_t ldw, const float* bias, int M, int N, int K,
-                      hipStream_t stream, const void* W2 = nullptr) {
+                      hipStream_t stream, const void* W2 = nullptr, int own = 0) {
   constexpr int kOutCols = (kEpilogue == kMfSwiglu) ? 32 * WTN : 64 * WTN;     // (gate and up rows of the same columns share a slab)
-  const int tiles_n = (N + kOutCols - 1) / kOutCols, tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
+  const int owned = (own > 0 && own < kOutCols) ? own : kOutCols;
+  const int tiles_n = (N + owned - 1) / owned, tiles_m = (M + 64 * WTM - 1) / (64 * WTM);
   // (tiles dealt out die by die at every size: with weights that come from memory it is 3 to 9 % faster here than row
   // by row also where the operands would fit the L2s: 12.4 against 13.3 us for N = 1,152, K = 896 at 2,048 rows)
   const int by_die = 1;
   gemm_dma_kernel<kEpilogue, TO, WTM, WTN, S><<<tiles_n * tiles_m, 256, 0, stream>>>(
       static_cast<TO*>(out), ldo, static_cast<const bf16_t*>(A), lda, static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), ldw, bias, M, N, K,
-      tiles_m, tiles_n, by_die);
+      tiles_m, tiles_n, by_die, 1, nullptr, nullptr, owned == kOutCols ? 0 : owned);
   return 0;
 }
 
@@ -902,6 +907,21 @@ static int k_shares(int64_t tiles, int64_t tile_floats, int K) {
   while (shares < 16 && tiles * shares * 2 <= 512 && slabs / (shares * 2) >= 4 && tiles * shares * 2 * tile_floats <= g_ws.tile_floats)
     shares *= 2;
   return shares;
+}
+
+// The output columns a block owns where one tile of rows meets gate and up matrices whose whole tiles of 128 columns
+// are fewer than the compute units: the columns dealt out evenly over the compute units (at least 16), and the form
+// follows from that number (launch_mfma). A compute unit pulls its block's weight rows at a rate of its own, well below
+// its share of the memory's, so compute units without a block are lost: gate and up of 18,944 columns in 256 blocks
+// of 74 (of tiles that hold 128) 55-58 us at 8 to 64 rows where 148 blocks of 128 or 296 of 64 take 62-69; of 8,960
+// columns 15.2-16.1 against 17.3-20.0; of 13,824 57-61 against 60-66; of 11,008 24.0-25.2 against 25.4-26.3; no
+// difference at 27,648 (216 blocks of 128 already read at the memory's rate) and 4,864 (the launch itself). 0: whole
+// tiles.
+static int owned_columns(int N) {
+  const int units = compute_units();
+  if ((N + 127) / 128 >= units) return 0;
+  const int own = (N + units - 1) / units;
+  return own < 16 ? 16 : own;
 }
 
 template <int kEpilogue, typename TO>
@@ -930,23 +950,37 @@ static int launch_mfma(void* out, int64_t ldo, const void* A, int64_t lda, const
     const int64_t col_tiles = (N + 63) / 64;
     const int64_t tiles_64 = col_tiles * ((M + 63) / 64), tiles_128 = col_tiles * ((M + 127) / 128);
     const bool ring = K % TK == 0;
+    const int own = M <= 64 ? owned_columns(N) : 0;     // (one tile of rows: what a block owns if the blocks are dealt out evenly, 0 if whole tiles fill the chip)
+    if (ring && own > 0 && K >= 2048) {
+      if (own <= 64) {
+        if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, own)) return 1;
+      } else {
+        if (launch_dma<kEpilogue, TO, 1, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, own)) return 1;
+      }
+    } else if (ring && own > 0 && own <= 64) {
+      if (own <= 32) {
+        if (launch_dma<kEpilogue, TO, 1, 1, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, own)) return 1;
+      } else {
+        if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, own)) return 1;
+      }
+    } else
     if (ring && (M <= 64 || tiles_64 <= 256)) {
       if (K >= 2048 && ((N + 127) / 128 >= 192 || ((N + 127) / 128 >= 128 && M > 32))) {
         // a long and wide pair of matrices: 128 gate + 128 up columns per block, a ring of three, one block per
         // compute unit; the rows are read half as often (32B sizes: 105, 107, 109 us at 16, 32, 64 rows against
         // 114, 120, 125; with fewer such tiles than three quarters of the compute units only from 33 rows on: 7B
         // sizes, 148 tiles, 64.1 against 62.4 at 16 rows, 67.6 against 70.7 at 64)
-        if (launch_dma<kEpilogue, TO, 1, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+        if (launch_dma<kEpilogue, TO, 1, 4, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, 0)) return 1;
       } else if (K < 2048) {
         // (up to 64 rows and fewer tiles than half the compute units: tiles of 32 outputs, whose gate and up halves
         // are computed by different waves and meet in LDS; N = 4,864, K = 896 at 17 to 64 rows 8.5-9.4 us against
         // 9.9-11.2)
         if (M <= 64 && (N + 63) / 64 < 128) {
-          if (launch_dma<kEpilogue, TO, 1, 1, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+          if (launch_dma<kEpilogue, TO, 1, 1, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, 0)) return 1;
         } else
-        if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+        if (launch_dma<kEpilogue, TO, 1, 2, 4>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, 0)) return 1;
       } else {
-        if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;
+        if (launch_dma<kEpilogue, TO, 1, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2, 0)) return 1;
       }
     } else if (ring && tiles_128 <= 256) {
       if (launch_dma<kEpilogue, TO, 2, 2, 3>(out, ldo, A, lda, W, ldw, bias, M, N, K, stream, W2)) return 1;

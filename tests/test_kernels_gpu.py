@@ -391,6 +391,21 @@ def test_the_tiled_product_takes_its_wide_form_where_the_rounds_are_full():
     close(by_rule[rows], pm.linear(a[rows].float().cpu().numpy(), w.float().cpu().numpy()), BF16, "against the plain product")
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 1000, 128), (64, 4867, 896), (8, 18950, 2048), (33, 9000, 2112), (64, 14000, 2048), (5, 30, 64)])
+def test_gate_and_up_of_one_tile_of_rows_in_blocks_dealt_out_evenly(M, N, K):
+    """Up to 64 rows against gate and up matrices whose whole tiles are fewer than the compute units: the tiled
+    product's blocks own as many columns as deal them out evenly (74 of a tile's 128 for 18,944 columns), the
+    columns beyond are neither fetched nor stored. Odd column counts, every form the rule picks (tiles that hold
+    32, 64 and 128 columns, short and long K), against the plain product."""
+    rng = np.random.default_rng(50)
+    a, w, w2 = (bf(rng.standard_normal((M, K)).astype(np.float32)), bf(rng.standard_normal((N, K)).astype(np.float32) * 0.05),
+                bf(rng.standard_normal((N, K)).astype(np.float32) * 0.05))
+    out = torch.full((M, N + 5), 7.0, device=DEV, dtype=torch.bfloat16)      # (a wider buffer: nothing is written beside the outputs)
+    ops().gemm_swiglu(out[:, :N], t(a, torch.bfloat16), t(w, torch.bfloat16), t(w2, torch.bfloat16), kernel="tiled")
+    close(out[:, :N], pm.swiglu(pm.linear(a, w), pm.linear(a, w2)), BF16, "gate/up")
+    assert bool((out[:, N:] == 7.0).all())
+
+
 def test_gemm_takes_a_strided_view():
     rng = np.random.default_rng(4)
     big = rng.standard_normal((6, 300)).astype(np.float32)
@@ -981,7 +996,7 @@ def test_product_kernel_choice():
     rows or big weights are tiled; a kernel that cannot take the rows is an error, not a guess."""
     o = ops()
     assert o.few_rows_kernel(1, 151936, 896) == "tiled" and o.few_rows_kernel(1, 2 * 18944, 3584, swiglu=True) == "rows"
-    assert o.few_rows_kernel(4, 4608, 3584) == "rows" and o.few_rows_kernel(4, 3584, 18944) == "rows" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
+    assert o.few_rows_kernel(4, 4608, 3584) == "rows" and o.few_rows_kernel(2, 3584, 18944) == "rows" and o.few_rows_kernel(4, 5120, 13824) == "rows" and o.few_rows_kernel(8, 3584, 18944) == "tiled"
     assert o.few_rows_kernel(64, 2 * 4864, 896, swiglu=True) == "tiled" and o.few_rows_kernel(16, 2 * 4864, 896, swiglu=True) == "stream"
     assert o.few_rows_kernel(64, 896, 4864) == "stream" and o.few_rows_kernel(32, 3584, 3584) == "tiled"
     assert o.few_rows_kernel(65, 8, 8) == "tiled"
