@@ -1,12 +1,12 @@
 """Exactness at the layer widths of real models of the family, not only at the
-tiny ones: a few layers of the Qwen2.5 0.5B, 7B and 32B sizes (hidden width,
+tiny ones: a few layers of the Qwen2.5 0.5B, 1.5B, 3B, 7B and 32B sizes (hidden width,
 heads, head size, feed-forward width as in those models' config.json) with
 random weights, an 80-token request run whole, most of it at once with the
 last 32 tokens one by one, and in portions, in float32 (the reference's 1e-5
 criterion, tests/unit/test_layer0_parity.mojo:46 there) and in bfloat16,
 against the plain implementation.
 
-The 0.5B case keeps the full vocabulary of 151,936 rows; the two large ones
+The 0.5B case keeps the full vocabulary of 151,936 rows; the others
 cut it to a few thousand rows (a count that is no multiple of anything) and
 keep one layer, so that the plain NumPy side stays within seconds."""
 import numpy as np
@@ -20,12 +20,17 @@ WIDTHS = {
     # name: config.json of the real model's sizes; "real" lists the keys that are the model's own
     "0.5b": dict(num_hidden_layers=2, hidden_size=896, num_attention_heads=14, num_key_value_heads=2, intermediate_size=4864,
                  vocab_size=151936, tie_word_embeddings=True),
+    "1.5b": dict(num_hidden_layers=1, hidden_size=1536, num_attention_heads=12, num_key_value_heads=2, intermediate_size=8960,
+                 vocab_size=3001, tie_word_embeddings=True),
+    "3b": dict(num_hidden_layers=1, hidden_size=2048, num_attention_heads=16, num_key_value_heads=2, intermediate_size=11008,
+               vocab_size=2999, tie_word_embeddings=True),
     "7b": dict(num_hidden_layers=1, hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, intermediate_size=18944,
                vocab_size=3003, tie_word_embeddings=False),
     "32b": dict(num_hidden_layers=1, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=27648,
                 vocab_size=2051, tie_word_embeddings=False),
 }
 REAL_KEYS = {"0.5b": "hidden_size heads kv_heads head_dim intermediate_size vocab_size tying",
+             "1.5b": "hidden_size heads kv_heads head_dim intermediate_size tying", "3b": "hidden_size heads kv_heads head_dim intermediate_size tying",
              "7b": "hidden_size heads kv_heads head_dim intermediate_size tying", "32b": "hidden_size heads kv_heads head_dim intermediate_size tying"}
 
 
