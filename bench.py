@@ -475,6 +475,8 @@ def sweep(args):
     model = device_model(cfg, args.dtype, 20260918)
     dbytes = 2 if args.dtype == "bfloat16" else 4
     batches = (1, 2, 4, 8, 16, 17, 24, 32, 48, 64, 96, 128, 192, 256) if name == "0.5b" else (1, 2, 4, 8, 16, 17, 32, 64) if name in ("1.5b", "3b") else (1, 2, 4, 8, 16, 32, 64)
+    if args.batches:
+        batches = tuple(int(b) for b in args.batches.split(","))
     cases = ([(b, PROMPT) for b in batches] if args.sweep == "batch" else
              [(b, p) for p in (2048, 8192, 16384, 30000) for b in (1, 8, 32)])
     for batch, prompt in cases:
@@ -501,6 +503,7 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points, the prefill, the repeats and the roofs")
     ap.add_argument("--only-prefill", action="store_true", help="run the 2,048-token prefill alone (for profiling) and print its line")
     ap.add_argument("--serve", action="store_true", help="the continuous batch of 64 requests (prompts of 128..2,048 tokens, 256 new tokens, chunks of 512) at the sizes of --config")
+    ap.add_argument("--batches", default=None, help="with --sweep batch: these batch sizes only (comma-separated), e.g. to profile one point")
     ap.add_argument("--sweep", choices=["batch", "context"], default=None, help="decode steps over batch sizes or over contexts, a line per point (the sizes of --config)")
     args = ap.parse_args()
     if args.gpus != 1:
